@@ -1,0 +1,348 @@
+// extern "C" surface declared in include/chessrl_amd.h.
+#include <algorithm>
+#include <cstring>
+#include <thread>
+
+#include "model.hpp"
+
+using namespace crl;
+
+namespace {
+
+int hip_fail(const char* what, hipError_t e) {
+  set_error(std::string(what) + ": " + hipGetErrorString(e));
+  return CRL_ERR_HIP;
+}
+int arg_fail(const char* msg) {
+  set_error(msg);
+  return CRL_ERR_ARG;
+}
+
+// Run fn(i) for i in [0,n) on a few host threads; returns the first non-zero result.
+template <typename Fn>
+int parallel_for(int n, int threads, Fn fn) {
+  if (threads <= 0) threads = (int)std::min<unsigned>(16, std::max<unsigned>(1, std::thread::hardware_concurrency()));
+  threads = std::min(threads, std::max(1, n / 64));
+  if (threads <= 1) {
+    for (int i = 0; i < n; ++i) { int rc = fn(i); if (rc) return rc; }
+    return 0;
+  }
+  std::vector<int> rcs(threads, 0);
+  std::vector<std::string> errs(threads);
+  std::vector<std::thread> pool;
+  for (int t = 0; t < threads; ++t)
+    pool.emplace_back([&, t]() {
+      for (int i = t; i < n; i += threads) {
+        int rc = fn(i);
+        if (rc) { rcs[t] = rc; errs[t] = get_error(); return; }
+      }
+    });
+  for (auto& th : pool) th.join();
+  for (int t = 0; t < threads; ++t)
+    if (rcs[t]) { set_error(errs[t]); return rcs[t]; }
+  return 0;
+}
+
+int parse(const char* fen, Board& b) {
+  std::string err;
+  if (b.set_fen(fen, &err)) {
+    set_error("invalid FEN '" + std::string(fen ? fen : "(null)") + "': " + err);
+    return CRL_ERR_FEN;
+  }
+  return 0;
+}
+
+void put_str(char* dst, size_t cap, const std::string& s) {
+  std::memset(dst, 0, cap);
+  std::memcpy(dst, s.data(), std::min(cap - 1, s.size()));
+}
+
+}  // namespace
+
+extern "C" {
+
+const char* crl_last_error(void) { return get_error(); }
+const char* crl_version(void) { return "chessrl_amd 0.1 (gfx950)"; }
+
+const char* crl_policy_index(int i) {
+  const auto& v = policy_index();
+  return (i >= 0 && i < (int)v.size()) ? v[i].c_str() : nullptr;
+}
+const char* crl_policy_leela(int i) {
+  const auto& v = policy_leela();
+  return (i >= 0 && i < (int)v.size()) ? v[i].c_str() : nullptr;
+}
+int crl_move_to_index(const char* uci) {
+  if (!uci) return -1;
+  std::string s = uci;
+  if (s.size() == 5 && s[4] == 'n') s.pop_back();
+  const auto& v = policy_index();
+  for (int i = 0; i < (int)v.size(); ++i)
+    if (v[i] == s) return i;
+  return -1;
+}
+int crl_leela_to_rl_maps(int32_t* white_out, int32_t* black_out) {
+  if (white_out) std::memcpy(white_out, leela_to_rl_white(), sizeof(int32_t) * VOCAB_LEELA);
+  if (black_out) std::memcpy(black_out, leela_to_rl_black(), sizeof(int32_t) * VOCAB_LEELA);
+  return CRL_OK;
+}
+
+int crl_fen_to_planes(const char* fen, float* out) {
+  if (!out) return arg_fail("crl_fen_to_planes: null output");
+  Board b;
+  int rc = parse(fen, b);
+  if (rc) return rc;
+  b.planes(out);
+  return CRL_OK;
+}
+int crl_encode_fens(const char* const* fens, int n, float* out, int threads) {
+  if (n < 0 || (n && (!fens || !out))) return arg_fail("crl_encode_fens: bad arguments");
+  return parallel_for(n, threads, [&](int i) {
+    Board b;
+    int rc = parse(fens[i], b);
+    if (rc) return rc;
+    b.planes(out + (size_t)i * 64 * NUM_PLANES);
+    return 0;
+  });
+}
+int crl_encode_fens_compact(const char* const* fens, int n, uint8_t* ids, uint8_t* flags, int threads) {
+  if (n < 0 || (n && (!fens || !ids || !flags))) return arg_fail("crl_encode_fens_compact: bad arguments");
+  return parallel_for(n, threads, [&](int i) {
+    Board b;
+    int rc = parse(fens[i], b);
+    if (rc) return rc;
+    b.compact(ids + (size_t)i * 64, flags + (size_t)i * 4);
+    return 0;
+  });
+}
+int crl_legal_masks(const char* const* fens, int n, uint8_t* masks, int32_t* counts, int threads) {
+  if (n < 0 || (n && (!fens || !masks))) return arg_fail("crl_legal_masks: bad arguments");
+  return parallel_for(n, threads, [&](int i) {
+    Board b;
+    int rc = parse(fens[i], b);
+    if (rc) return rc;
+    int c = legal_mask_rl(b, masks + (size_t)i * VOCAB_RL);
+    if (counts) counts[i] = c;
+    return 0;
+  });
+}
+int crl_legal_masks_leela(const char* const* fens, int n, uint8_t* masks, int32_t* counts, int threads) {
+  if (n < 0 || (n && (!fens || !masks))) return arg_fail("crl_legal_masks_leela: bad arguments");
+  return parallel_for(n, threads, [&](int i) {
+    Board b;
+    int rc = parse(fens[i], b);
+    if (rc) return rc;
+    int c = legal_mask_leela(b, masks + (size_t)i * VOCAB_LEELA);
+    if (counts) counts[i] = c;
+    return 0;
+  });
+}
+int crl_legal_moves(const char* fen, char* out_uci6, int max_moves) {
+  Board b;
+  int rc = parse(fen, b);
+  if (rc) return rc;
+  std::vector<Move> mv;
+  b.legal(mv);
+  const int n = std::min<int>((int)mv.size(), max_moves);
+  for (int i = 0; i < n && out_uci6; ++i) put_str(out_uci6 + (size_t)i * 6, 6, move_uci(mv[i]));
+  return n;
+}
+int crl_child_fens(const char* fen, char* out_fens96, char* out_uci6, int max_moves) {
+  Board b;
+  int rc = parse(fen, b);
+  if (rc) return rc;
+  std::vector<Move> mv;
+  b.legal(mv);
+  const int n = std::min<int>((int)mv.size(), max_moves);
+  for (int i = 0; i < n; ++i) {
+    Board c = b;
+    c.make(mv[i]);
+    if (out_fens96) put_str(out_fens96 + (size_t)i * 96, 96, c.fen(true));
+    if (out_uci6) put_str(out_uci6 + (size_t)i * 6, 6, move_uci(mv[i]));
+  }
+  return n;
+}
+uint64_t crl_perft(const char* fen, int depth) {
+  Board b;
+  if (parse(fen, b)) return 0;
+  return b.perft(depth);
+}
+int crl_random_positions(uint64_t seed, int n, int max_plies, double late_fraction, int late_max_pieces,
+                         float* out_planes, uint8_t* out_masks_rl, uint8_t* out_masks_leela, char* out_fens96) {
+  if (n < 0 || max_plies < 0) return arg_fail("crl_random_positions: bad arguments");
+  // Every position has its own generator seeded from (seed, index), so the result does
+  // not depend on the thread count.
+  return parallel_for(n, 0, [&](int i) {
+    SplitMix64 mix(seed ^ (0xD1B54A32D192ED03ull * (uint64_t)(i + 1)));
+    SplitMix64 rng(mix.next());
+    const bool late = late_fraction > 0 && (double)(rng.next() >> 11) * (1.0 / 9007199254740992.0) < late_fraction;
+    Board b = random_playout(rng, max_plies, late ? late_max_pieces : 0);
+    if (out_planes) b.planes(out_planes + (size_t)i * 64 * NUM_PLANES);
+    if (out_masks_rl) legal_mask_rl(b, out_masks_rl + (size_t)i * VOCAB_RL);
+    if (out_masks_leela) legal_mask_leela(b, out_masks_leela + (size_t)i * VOCAB_LEELA);
+    if (out_fens96) put_str(out_fens96 + (size_t)i * 96, 96, b.fen(true));
+    return 0;
+  });
+}
+
+// ---------------------------------------------------------------------------- operators
+int crl_gemm(const void* A, int64_t lda, const void* W, int64_t ldw, void* C, int64_t ldc, int M, int N, int K, int in_dtype,
+             int out_dtype, const float* bias, int act, float descale, float alpha, const void* res, int64_t ldr, int res_dtype,
+             float out_scale, float* amax, int tile, void* stream) {
+  if (!A || !W || !C || M < 0 || N < 0 || K <= 0) return arg_fail("crl_gemm: bad arguments");
+  if (in_dtype != DT_BF16 && in_dtype != DT_F16 && in_dtype != DT_FP8) return arg_fail("crl_gemm: in_dtype must be bf16, f16 or fp8");
+  if (out_dtype < 0 || out_dtype > 3 || tile < 0 || tile > 3) return arg_fail("crl_gemm: bad out_dtype or tile");
+  GemmArgs g;
+  std::memset(&g, 0, sizeof(g));
+  g.A = A; g.lda = lda; g.W = W; g.ldw = ldw; g.C = C; g.ldc = ldc; g.M = M; g.N = N; g.K = K; g.nsplit = N;
+  g.bias = bias; g.act = act; g.descale = descale; g.alpha = alpha; g.res = res; g.ldr = ldr; g.res_dtype = res_dtype;
+  g.out_scale = out_scale; g.amax = amax;
+  hipError_t e = launch_gemm(g, in_dtype, out_dtype, tile, (hipStream_t)stream);
+  if (e == hipErrorInvalidValue) return arg_fail("crl_gemm: operands must be 16-byte aligned with K*elem_size a multiple of 16");
+  return e == hipSuccess ? CRL_OK : hip_fail("crl_gemm", e);
+}
+
+int crl_layernorm(const void* x, int64_t ldx, int in_dtype, const float* gamma, const float* beta, void* out, int out_dtype,
+                  uint8_t* out_fp8, float fp8_scale, int64_t ldo, int rows, int C, float eps, float* amax, void* stream) {
+  if (!x || !gamma || (!out && !out_fp8) || rows < 0) return arg_fail("crl_layernorm: bad arguments");
+  LayerNormArgs a;
+  std::memset(&a, 0, sizeof(a));
+  a.x = x; a.ldx = ldx; a.in_dtype = in_dtype; a.gamma = gamma; a.beta = beta; a.out = out; a.out_dtype = out_dtype;
+  a.out_fp8 = out_fp8; a.fp8_scale = fp8_scale; a.ldo = ldo; a.rows = rows; a.C = C; a.eps = eps; a.amax = amax;
+  hipError_t e = launch_layernorm(a, (hipStream_t)stream);
+  if (e == hipErrorInvalidValue) return arg_fail("crl_layernorm: C and strides must be multiples of 8 and C <= 8192");
+  return e == hipSuccess ? CRL_OK : hip_fail("crl_layernorm", e);
+}
+
+int crl_attention(const void* q, int64_t ldq, const void* k, int64_t ldk, const void* v, int64_t ldv, void* out, int64_t ldo,
+                  int out_dtype, float out_scale, int B, int H, int head_dim, int mode, float scale, const void* bias,
+                  const void* pos, const float* u_bias, const float* v_bias, float* amax, void* stream) {
+  if (!q || !k || !v || !out || B < 0 || H <= 0) return arg_fail("crl_attention: bad arguments");
+  AttnArgs a;
+  std::memset(&a, 0, sizeof(a));
+  a.q = q; a.k = k; a.v = v; a.ldq = ldq; a.ldk = ldk; a.ldv = ldv; a.out = out; a.ldo = ldo; a.out_dtype = out_dtype;
+  a.out_scale = out_scale; a.B = B; a.H = H; a.mode = mode; a.scale = scale; a.bias = bias; a.pos = pos;
+  a.u_bias = u_bias; a.v_bias = v_bias; a.amax = amax;
+  hipError_t e = launch_attention(a, head_dim, (hipStream_t)stream);
+  if (e == hipErrorInvalidValue) return arg_fail("crl_attention: head_dim must be 32 or 64, strides multiples of 8, mode inputs present");
+  return e == hipSuccess ? CRL_OK : hip_fail("crl_attention", e);
+}
+
+int crl_attn_bias_slot(int query, int key) {
+  if (query < 0 || query > 63 || key < 0 || key > 63) return -1;
+  return attn_bias_slot_host(query, key);
+}
+
+int crl_masked_softmax(const float* logits, int64_t ldl, const uint8_t* mask, int64_t ldm, float* probs, int64_t ldp,
+                       int32_t* argmax, int B, int V, float temperature, void* stream) {
+  if (!logits || B < 0) return arg_fail("crl_masked_softmax: bad arguments");
+  SoftmaxArgs a;
+  std::memset(&a, 0, sizeof(a));
+  a.logits = logits; a.ldl = ldl; a.mask = mask; a.ldm = ldm; a.probs = probs; a.ldp = ldp; a.argmax = argmax;
+  a.B = B; a.V = V; a.temperature = temperature;
+  hipError_t e = launch_masked_softmax(a, (hipStream_t)stream);
+  if (e == hipErrorInvalidValue) return arg_fail("crl_masked_softmax: V must be in 1..2048");
+  return e == hipSuccess ? CRL_OK : hip_fail("crl_masked_softmax", e);
+}
+
+int crl_leela_to_rl(const float* src, int64_t lds, float* dst, int64_t ldd, const uint8_t* white_to_move, int B, void* stream) {
+  if (!src || !dst || !white_to_move || B < 0) return arg_fail("crl_leela_to_rl: bad arguments");
+  // Inverse maps live on the device for the lifetime of the process, one copy per device.
+  static int32_t* inv_dev[16] = {};
+  int dev = 0;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess) return hip_fail("hipGetDevice", e);
+  if (dev < 0 || dev >= 16) return arg_fail("crl_leela_to_rl: device index above 15");
+  if (!inv_dev[dev]) {
+    std::vector<int32_t> inv((size_t)2 * VOCAB_RL, -1);
+    for (int i = 0; i < VOCAB_LEELA; ++i) {
+      inv[leela_to_rl_white()[i]] = i;
+      inv[VOCAB_RL + leela_to_rl_black()[i]] = i;
+    }
+    int32_t* p = nullptr;
+    e = hipMalloc((void**)&p, inv.size() * sizeof(int32_t));
+    if (e != hipSuccess) return hip_fail("hipMalloc", e);
+    e = hipMemcpy(p, inv.data(), inv.size() * sizeof(int32_t), hipMemcpyHostToDevice);
+    if (e != hipSuccess) { (void)hipFree(p); return hip_fail("hipMemcpy", e); }
+    inv_dev[dev] = p;
+  }
+  ScatterArgs a;
+  std::memset(&a, 0, sizeof(a));
+  a.src = src; a.lds = lds; a.dst = dst; a.ldd = ldd; a.inv_white = inv_dev[dev]; a.inv_black = inv_dev[dev] + VOCAB_RL;
+  a.white_to_move = white_to_move; a.B = B; a.nsrc = VOCAB_LEELA; a.ndst = VOCAB_RL;
+  e = launch_leela_to_rl(a, (hipStream_t)stream);
+  return e == hipSuccess ? CRL_OK : hip_fail("crl_leela_to_rl", e);
+}
+
+// ---------------------------------------------------------------------------- models
+struct crl_model { Model impl; explicit crl_model(const crl_model_config& c) : impl(c) {} };
+
+int crl_model_create(const crl_model_config* cfg, crl_model** out) {
+  if (!cfg || !out) return arg_fail("crl_model_create: null argument");
+  if (cfg->arch < 0 || cfg->arch > 2) return arg_fail("crl_model_create: unknown arch");
+  if (cfg->n_layer < 0 || cfg->d_model <= 0 || cfg->n_head <= 0 || cfg->d_ff <= 0) return arg_fail("crl_model_create: non-positive size");
+  if (cfg->d_model % cfg->n_head) return arg_fail("crl_model_create: d_model must be divisible by n_head");
+  const int hs = cfg->d_model / cfg->n_head;
+  if (hs != 32 && hs != 64) return arg_fail("crl_model_create: head dimension must be 32 or 64");
+  if (cfg->d_model % 16 || cfg->d_model > 2048 || cfg->d_ff % 8) return arg_fail("crl_model_create: d_model must be a multiple of 16 up to 2048, d_ff a multiple of 8");
+  if (cfg->arch == CRL_ARCH_BT4CLASS) {
+    const int sg = cfg->smolgen_gen ? cfg->smolgen_gen : 256, sc = cfg->smolgen_compress ? cfg->smolgen_compress : 32;
+    const int sh = cfg->smolgen_hidden ? cfg->smolgen_hidden : 256;
+    if (sg % 8 || sc % 8 || sh % 8 || (long)cfg->n_head * sg > 8192) return arg_fail("crl_model_create: smolgen sizes must be multiples of 8 and n_head*gen <= 8192");
+  }
+  *out = new (std::nothrow) crl_model(*cfg);
+  if (!*out) return arg_fail("crl_model_create: out of host memory");
+  return CRL_OK;
+}
+void crl_model_destroy(crl_model* m) { delete m; }
+int crl_model_set_weight(crl_model* m, const char* key, const float* data, int64_t numel) {
+  if (!m) return arg_fail("null model");
+  return m->impl.set_weight(key, data, (long)numel);
+}
+const char* crl_model_expected_key(crl_model* m, int i, int64_t* numel) {
+  if (!m || i < 0 || i >= (int)m->impl.expected.size()) return nullptr;
+  if (numel) *numel = m->impl.expected[i].second;
+  return m->impl.expected[i].first.c_str();
+}
+int crl_model_finalize(crl_model* m) {
+  if (!m) return arg_fail("null model");
+  return m->impl.finalize();
+}
+int crl_model_calibrate(crl_model* m, const float* planes, int B, void* stream) {
+  if (!m || !planes || B <= 0) return arg_fail("crl_model_calibrate: bad arguments");
+  return m->impl.calibrate(planes, B, (hipStream_t)stream);
+}
+int crl_model_get_amax(crl_model* m, float* out, int n) {
+  if (!m || !out || n != (int)m->impl.amax_host.size()) return arg_fail("crl_model_get_amax: n must be n_layer*4");
+  std::memcpy(out, m->impl.amax_host.data(), sizeof(float) * n);
+  return CRL_OK;
+}
+int crl_model_set_amax(crl_model* m, const float* in, int n) {
+  if (!m || !in || n != (int)m->impl.amax_host.size()) return arg_fail("crl_model_set_amax: n must be n_layer*4");
+  std::memcpy(m->impl.amax_host.data(), in, sizeof(float) * n);
+  return CRL_OK;
+}
+int crl_model_forward(crl_model* m, const float* planes, int B, float* policy_logits, float* wdl_logits, void* stream) {
+  if (!m || !planes) return arg_fail("crl_model_forward: bad arguments");
+  return m->impl.forward(planes, nullptr, nullptr, B, policy_logits, wdl_logits, false, (hipStream_t)stream);
+}
+int crl_model_forward_compact(crl_model* m, const uint8_t* ids, const uint8_t* flags, int B, float* policy_logits,
+                              float* wdl_logits, void* stream) {
+  if (!m || !ids || !flags) return arg_fail("crl_model_forward_compact: bad arguments");
+  return m->impl.forward(nullptr, ids, flags, B, policy_logits, wdl_logits, false, (hipStream_t)stream);
+}
+int crl_model_vocab(const crl_model* m) { return m ? m->impl.vocab : 0; }
+double crl_model_flops_per_position(const crl_model* m) { return m ? m->impl.flops_per_position() : 0.0; }
+int crl_model_set_profiling(crl_model* m, int on) {
+  if (!m) return arg_fail("null model");
+  m->impl.profiling = on != 0;
+  for (int i = 0; i < 5; ++i) { m->impl.prof_ms[i] = 0; m->impl.prof_n[i] = 0; }
+  return CRL_OK;
+}
+int crl_model_get_profile(crl_model* m, double* ms5, int64_t* launches5) {
+  if (!m || !ms5 || !launches5) return arg_fail("crl_model_get_profile: bad arguments");
+  for (int i = 0; i < 5; ++i) { ms5[i] = m->impl.prof_ms[i]; launches5[i] = m->impl.prof_n[i]; }
+  return CRL_OK;
+}
+
+}  // extern "C"

@@ -1,0 +1,337 @@
+// Fused 64-token multi-head attention: one 64-lane wave per (position, head).
+//
+// Replaces F.scaled_dot_product_attention(q,k,v,is_causal=True) of model_bis.py:71 and
+// the score/softmax/context chain of RelativeMultiHeadAttention2.forward
+// (new_paradigm/attn.py:507-521), including the pad-and-reshape relative shift of
+// new_paradigm/attn.py:525-533. A third mode adds a generated per-head 64x64 bias
+// before the softmax (the BT4-class configuration).
+//
+// The wave computes the TRANSPOSED score tile S^T[j][i] = K[j]·Q[i] with 32x32x16
+// MFMAs whose operands are 16-byte row segments read straight from global memory
+// (both Q and K are head-dim contiguous). In the accumulator layout a lane then owns
+// one query i and 32 of its 64 keys j, so the softmax over keys is a reduction over
+// the lane's own registers plus one exchange with lane^32. The probabilities are
+// re-used in place as the column operand of the second product O^T = V^T · P^T; only V
+// needs a transpose, which goes through a wave-private LDS patch.
+#include "common.hpp"
+
+namespace crl {
+
+constexpr int VT_STRIDE = 72;   // bf16 elements per V^T row (64 keys + 8 padding)
+constexpr int SP_STRIDE = 65;   // floats per row of the positional score patch
+
+// Storage order of a 64x64 bias tile so that each lane reads its accumulator
+// registers as 16-byte vectors: element (query i, key j) lives at
+//   ((((i/32)*2 + j/32)*2 + rh)*64 + lane)*8 + e
+// with lane = (i%32) + 32*g, j%32 = 8*(2*rh + e/4) + 4*g + e%4.
+__host__ __device__ inline int attn_bias_slot(int i, int j) {
+  const int it = i >> 5, jt = j >> 5, jj = j & 31;
+  const int q4 = jj >> 3, g = (jj >> 2) & 1, e0 = jj & 3;
+  const int rh = q4 >> 1, e = ((q4 & 1) << 2) | e0;
+  const int lane = (i & 31) + 32 * g;
+  return ((((it * 2 + jt) * 2 + rh) * 64 + lane) << 3) + e;
+}
+
+__device__ __forceinline__ bf16x8_t add_bias_bf16(bf16x8_t q, const float* bias8) {
+  bf16x8_t r;
+#pragma unroll
+  for (int e = 0; e < 8; ++e) r[e] = (__bf16)((float)q[e] + bias8[e]);
+  return r;
+}
+
+// Waves per workgroup: the relative-shift mode needs a 16.6 KB score patch per wave,
+// so it runs two waves per workgroup to stay inside 64 KB of static LDS.
+template <int MODE>
+struct AttnWaves { static constexpr int N = MODE == ATTN_RELSHIFT ? 2 : 4; };
+
+template <int HS, int MODE, int OUT_DT>
+__global__ void __launch_bounds__(64 * AttnWaves<MODE>::N) attention_kernel(const AttnArgs a) {
+  constexpr int KS = HS / 16;   // k-steps of the score product
+  constexpr int DT_TILES = HS / 32;
+  constexpr int NW = AttnWaves<MODE>::N;
+  __shared__ __align__(16) uint16_t s_vt[NW][HS * VT_STRIDE];
+  __shared__ float s_sp[MODE == ATTN_RELSHIFT ? NW : 1][MODE == ATTN_RELSHIFT ? 64 * SP_STRIDE : 1];
+
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  const int lr = lane & 31, g = lane >> 5;
+  const int unit = blockIdx.x * NW + wave;
+  if (unit >= a.B * a.H) return;
+  const int b = unit / a.H, h = unit - b * a.H;
+
+  const uint16_t* qp = reinterpret_cast<const uint16_t*>(a.q) + (long)b * 64 * a.ldq + h * HS;
+  const uint16_t* kp = reinterpret_cast<const uint16_t*>(a.k) + (long)b * 64 * a.ldk + h * HS;
+  const uint16_t* vp = reinterpret_cast<const uint16_t*>(a.v) + (long)b * 64 * a.ldv + h * HS;
+
+  // ---- V -> V^T in LDS ------------------------------------------------------------
+  uint16_t* vt = s_vt[wave];
+  {
+    constexpr int DC = HS / 8;            // 16-byte chunks per V row
+    constexpr int PASSES = (16 * DC) / 64;
+#pragma unroll
+    for (int p = 0; p < PASSES; ++p) {
+      const int id = p * 64 + lane;
+      const int jq = id / DC, dc = id - jq * DC;
+      uint4 rows[4];
+#pragma unroll
+      for (int t = 0; t < 4; ++t) rows[t] = *reinterpret_cast<const uint4*>(vp + (long)(4 * jq + t) * a.ldv + 8 * dc);
+      const uint32_t* w0 = reinterpret_cast<const uint32_t*>(&rows[0]);
+      const uint32_t* w1 = reinterpret_cast<const uint32_t*>(&rows[1]);
+      const uint32_t* w2 = reinterpret_cast<const uint32_t*>(&rows[2]);
+      const uint32_t* w3 = reinterpret_cast<const uint32_t*>(&rows[3]);
+#pragma unroll
+      for (int e2 = 0; e2 < 4; ++e2) {
+        // d = 8dc + 2e2 (low halves) and d+1 (high halves)
+        uint2 lo = make_uint2((w0[e2] & 0xffffu) | (w1[e2] << 16), (w2[e2] & 0xffffu) | (w3[e2] << 16));
+        uint2 hi = make_uint2((w0[e2] >> 16) | (w1[e2] & 0xffff0000u), (w2[e2] >> 16) | (w3[e2] & 0xffff0000u));
+        *reinterpret_cast<uint2*>(vt + (8 * dc + 2 * e2) * VT_STRIDE + 4 * jq) = lo;
+        *reinterpret_cast<uint2*>(vt + (8 * dc + 2 * e2 + 1) * VT_STRIDE + 4 * jq) = hi;
+      }
+    }
+  }
+
+  // ---- scores -----------------------------------------------------------------------
+  bf16x8_t qf[2][KS], kf[2][KS];
+#pragma unroll
+  for (int t = 0; t < 2; ++t)
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) {
+      qf[t][ks] = *reinterpret_cast<const bf16x8_t*>(qp + (long)(32 * t + lr) * a.ldq + 16 * ks + 8 * g);
+      kf[t][ks] = *reinterpret_cast<const bf16x8_t*>(kp + (long)(32 * t + lr) * a.ldk + 16 * ks + 8 * g);
+    }
+
+  f32x16_t s[2][2];  // [jt][it]
+#pragma unroll
+  for (int jt = 0; jt < 2; ++jt)
+#pragma unroll
+    for (int it = 0; it < 2; ++it)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) s[jt][it][r] = 0.f;
+
+  if constexpr (MODE == ATTN_RELSHIFT) {
+    // content = (q+u)·k, position = (q+v)·p, both with the bias folded into the query.
+    const uint16_t* pp = reinterpret_cast<const uint16_t*>(a.pos) + h * HS;
+    const long ldp = (long)a.H * HS;
+    f32x16_t sp[2][2];
+#pragma unroll
+    for (int jt = 0; jt < 2; ++jt)
+#pragma unroll
+      for (int it = 0; it < 2; ++it)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) sp[jt][it][r] = 0.f;
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) {
+      float ub[8], vb[8];
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        ub[e] = a.u_bias[h * HS + 16 * ks + 8 * g + e];
+        vb[e] = a.v_bias[h * HS + 16 * ks + 8 * g + e];
+      }
+      bf16x8_t pf[2];
+#pragma unroll
+      for (int t = 0; t < 2; ++t) pf[t] = *reinterpret_cast<const bf16x8_t*>(pp + (long)(32 * t + lr) * ldp + 16 * ks + 8 * g);
+#pragma unroll
+      for (int it = 0; it < 2; ++it) {
+        const bf16x8_t qu = add_bias_bf16(qf[it][ks], ub);
+        const bf16x8_t qv = add_bias_bf16(qf[it][ks], vb);
+#pragma unroll
+        for (int jt = 0; jt < 2; ++jt) {
+          s[jt][it] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf[jt][ks], qu, s[jt][it], 0, 0, 0);
+          sp[jt][it] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(pf[jt], qv, sp[jt][it], 0, 0, 0);
+        }
+      }
+    }
+    // Shifted read-back (new_paradigm/attn.py:525-533): with T=64,
+    //   out[i][j] = P[i][63-i+j] (j<=i), 0 (j==i+1), P[i+1][j-i-2] (j>i+1).
+    float* spm = s_sp[wave];
+#pragma unroll
+    for (int jt = 0; jt < 2; ++jt)
+#pragma unroll
+      for (int it = 0; it < 2; ++it)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+          const int m = 32 * jt + 8 * (r >> 2) + 4 * g + (r & 3);
+          spm[(32 * it + lr) * SP_STRIDE + m] = sp[jt][it][r];
+        }
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+#pragma unroll
+    for (int jt = 0; jt < 2; ++jt)
+#pragma unroll
+      for (int it = 0; it < 2; ++it)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+          const int j = 32 * jt + 8 * (r >> 2) + 4 * g + (r & 3);
+          const int i = 32 * it + lr;
+          float pv;
+          if (j <= i) pv = spm[i * SP_STRIDE + (63 - i + j)];
+          else if (j == i + 1) pv = 0.f;
+          else pv = spm[(i + 1) * SP_STRIDE + (j - i - 2)];
+          s[jt][it][r] = (s[jt][it][r] + pv) * a.scale;
+        }
+  } else {
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks)
+#pragma unroll
+      for (int jt = 0; jt < 2; ++jt)
+#pragma unroll
+        for (int it = 0; it < 2; ++it)
+          s[jt][it] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf[jt][ks], qf[it][ks], s[jt][it], 0, 0, 0);
+
+    if constexpr (MODE == ATTN_BIAS) {
+      const uint16_t* bp = reinterpret_cast<const uint16_t*>(a.bias) + (long)unit * 4096;
+#pragma unroll
+      for (int it = 0; it < 2; ++it)
+#pragma unroll
+        for (int jt = 0; jt < 2; ++jt)
+#pragma unroll
+          for (int rh = 0; rh < 2; ++rh) {
+            const uint4 u = *reinterpret_cast<const uint4*>(bp + ((((it * 2 + jt) * 2 + rh) * 64 + lane) << 3));
+            const uint32_t w[4] = {u.x, u.y, u.z, u.w};
+#pragma unroll
+            for (int e = 0; e < 8; ++e) {
+              const float bv = bf16_bits_to_f32((uint16_t)((e & 1) ? (w[e >> 1] >> 16) : (w[e >> 1] & 0xffff)));
+              s[jt][it][8 * rh + e] = s[jt][it][8 * rh + e] * a.scale + bv;
+            }
+          }
+    } else {
+#pragma unroll
+      for (int jt = 0; jt < 2; ++jt)
+#pragma unroll
+        for (int it = 0; it < 2; ++it)
+#pragma unroll
+          for (int r = 0; r < 16; ++r) {
+            float x = s[jt][it][r] * a.scale;
+            if constexpr (MODE == ATTN_CAUSAL) {
+              const int j = 32 * jt + 8 * (r >> 2) + 4 * g + (r & 3);
+              const int i = 32 * it + lr;
+              if (j > i) x = -INFINITY;
+            }
+            s[jt][it][r] = x;
+          }
+    }
+  }
+
+  // ---- softmax over keys (registers + lane^32) ------------------------------------------
+  float inv_l[2];
+#pragma unroll
+  for (int it = 0; it < 2; ++it) {
+    float mx = -INFINITY;
+#pragma unroll
+    for (int jt = 0; jt < 2; ++jt)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) mx = fmaxf(mx, s[jt][it][r]);
+    mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+    float sum = 0.f;
+#pragma unroll
+    for (int jt = 0; jt < 2; ++jt)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        const float p = __expf(s[jt][it][r] - mx);
+        s[jt][it][r] = p;
+        sum += p;
+      }
+    sum += __shfl_xor(sum, 32, 64);
+    inv_l[it] = 1.0f / sum;
+  }
+
+  // ---- O^T = V^T · P^T ------------------------------------------------------------------
+  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+  __builtin_amdgcn_wave_barrier();
+  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+  f32x16_t o[DT_TILES][2];
+#pragma unroll
+  for (int dt = 0; dt < DT_TILES; ++dt)
+#pragma unroll
+    for (int it = 0; it < 2; ++it)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) o[dt][it][r] = 0.f;
+
+#pragma unroll
+  for (int kb = 0; kb < 4; ++kb) {
+    const int jt = kb >> 1, kh = kb & 1;
+    bf16x8_t pf[2];
+#pragma unroll
+    for (int it = 0; it < 2; ++it)
+#pragma unroll
+      for (int e = 0; e < 8; ++e) pf[it][e] = (__bf16)s[jt][it][8 * kh + e];
+#pragma unroll
+    for (int dt = 0; dt < DT_TILES; ++dt) {
+      const uint16_t* vrow = vt + (32 * dt + lr) * VT_STRIDE + 16 * kb + 4 * g;
+      const uint2 lo = *reinterpret_cast<const uint2*>(vrow);
+      const uint2 hi = *reinterpret_cast<const uint2*>(vrow + 8);
+      const uint4 packed = make_uint4(lo.x, lo.y, hi.x, hi.y);
+      const bf16x8_t vf = __builtin_bit_cast(bf16x8_t, packed);
+#pragma unroll
+      for (int it = 0; it < 2; ++it) o[dt][it] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vf, pf[it], o[dt][it], 0, 0, 0);
+    }
+  }
+
+  // ---- normalise and store ----------------------------------------------------------------
+  float am = 0.f;
+#pragma unroll
+  for (int it = 0; it < 2; ++it) {
+    const long row = (long)b * 64 + 32 * it + lr;
+#pragma unroll
+    for (int dt = 0; dt < DT_TILES; ++dt)
+#pragma unroll
+      for (int rq = 0; rq < 4; ++rq) {
+        const int d = 32 * dt + 8 * rq + 4 * g;
+        float v[4];
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          v[e] = o[dt][it][4 * rq + e] * inv_l[it];
+          am = fmaxf(am, fabsf(v[e]));
+        }
+        const long off = row * a.ldo + h * HS + d;
+        if constexpr (OUT_DT == DT_FP8) {
+          *reinterpret_cast<uint32_t*>(reinterpret_cast<uint8_t*>(a.out) + off) =
+              pack_fp8x4(v[0] * a.out_scale, v[1] * a.out_scale, v[2] * a.out_scale, v[3] * a.out_scale);
+        } else {
+          *reinterpret_cast<uint2*>(reinterpret_cast<uint16_t*>(a.out) + off) = make_uint2(pack_bf16x2(v[0], v[1]), pack_bf16x2(v[2], v[3]));
+        }
+      }
+  }
+  if (a.amax) {
+    am = wave_max(am);
+    if (lane == 0) atomic_amax(a.amax, am);
+  }
+}
+
+template <int HS, int MODE>
+static hipError_t launch_attn_mode(const AttnArgs& a, hipStream_t st) {
+  constexpr int NW = AttnWaves<MODE>::N;
+  const dim3 grid((a.B * a.H + NW - 1) / NW), block(64 * NW);
+  if (a.out_dtype == DT_FP8) hipLaunchKernelGGL((attention_kernel<HS, MODE, DT_FP8>), grid, block, 0, st, a);
+  else if (a.out_dtype == DT_BF16) hipLaunchKernelGGL((attention_kernel<HS, MODE, DT_BF16>), grid, block, 0, st, a);
+  else return hipErrorInvalidValue;
+  return hipGetLastError();
+}
+
+template <int HS>
+static hipError_t launch_attn_hs(const AttnArgs& a, hipStream_t st) {
+  switch (a.mode) {
+    case ATTN_PLAIN: return launch_attn_mode<HS, ATTN_PLAIN>(a, st);
+    case ATTN_CAUSAL: return launch_attn_mode<HS, ATTN_CAUSAL>(a, st);
+    case ATTN_BIAS: return launch_attn_mode<HS, ATTN_BIAS>(a, st);
+    case ATTN_RELSHIFT: return launch_attn_mode<HS, ATTN_RELSHIFT>(a, st);
+  }
+  return hipErrorInvalidValue;
+}
+
+hipError_t launch_attention(const AttnArgs& a, int head_dim, hipStream_t st) {
+  if (a.B <= 0) return hipSuccess;
+  // 16-byte row-segment loads: strides and bases must be multiples of 8 elements.
+  if (a.ldq % 8 || a.ldk % 8 || a.ldv % 8 || a.ldo % 4 ||
+      (reinterpret_cast<uintptr_t>(a.q) & 15) || (reinterpret_cast<uintptr_t>(a.k) & 15) || (reinterpret_cast<uintptr_t>(a.v) & 15))
+    return hipErrorInvalidValue;
+  if (a.mode == ATTN_BIAS && !a.bias) return hipErrorInvalidValue;
+  if (a.mode == ATTN_RELSHIFT && (!a.pos || !a.u_bias || !a.v_bias)) return hipErrorInvalidValue;
+  if (head_dim == 32) return launch_attn_hs<32>(a, st);
+  if (head_dim == 64) return launch_attn_hs<64>(a, st);
+  return hipErrorInvalidValue;
+}
+
+int attn_bias_slot_host(int i, int j) { return attn_bias_slot(i, j); }
+
+}  // namespace crl

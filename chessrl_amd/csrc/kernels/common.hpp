@@ -1,0 +1,212 @@
+// Shared device helpers for the gfx950 kernels: element types, vector aliases,
+// conversions, activations, 64-lane wave reductions and the kernel argument blocks.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace crl {
+
+typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
+typedef _Float16 f16x8_t __attribute__((ext_vector_type(8)));
+typedef float f32x16_t __attribute__((ext_vector_type(16)));
+typedef float f32x4_t __attribute__((ext_vector_type(4)));
+typedef int i32x8_t __attribute__((ext_vector_type(8)));
+typedef int i32x4_t __attribute__((ext_vector_type(4)));
+
+// Element type codes used across the C ABI.
+enum DType : int { DT_F32 = 0, DT_BF16 = 1, DT_F16 = 2, DT_FP8 = 3 };
+enum Act : int { ACT_NONE = 0, ACT_GELU = 1, ACT_MISH = 2, ACT_SWISH = 3 };
+
+__host__ __device__ inline int dtype_size(int dt) { return dt == DT_F32 ? 4 : dt == DT_FP8 ? 1 : 2; }
+
+// ---- scalar conversions ------------------------------------------------------
+__device__ __forceinline__ float bf16_bits_to_f32(uint16_t b) { return __uint_as_float(((uint32_t)b) << 16); }
+// Round-to-nearest-even, NaN kept quiet.
+__device__ __forceinline__ uint16_t f32_to_bf16_bits(float f) {
+  uint32_t u = __float_as_uint(f);
+  if ((u & 0x7fffffffu) > 0x7f800000u) return (uint16_t)((u >> 16) | 0x40);
+  u += 0x7fffu + ((u >> 16) & 1u);
+  return (uint16_t)(u >> 16);
+}
+__device__ __forceinline__ uint32_t pack_bf16x2(float lo, float hi) {
+  return (uint32_t)f32_to_bf16_bits(lo) | ((uint32_t)f32_to_bf16_bits(hi) << 16);
+}
+__device__ __forceinline__ uint16_t f32_to_f16_bits(float f) {
+  _Float16 h = (_Float16)f;
+  return __builtin_bit_cast(uint16_t, h);
+}
+__device__ __forceinline__ float f16_bits_to_f32(uint16_t b) { return (float)__builtin_bit_cast(_Float16, b); }
+
+// OCP e4m3fn: 4 values -> 4 bytes with hardware saturating conversion (max 448).
+__device__ __forceinline__ uint32_t pack_fp8x4(float a, float b, float c, float d) {
+  a = fminf(fmaxf(a, -448.f), 448.f);
+  b = fminf(fmaxf(b, -448.f), 448.f);
+  c = fminf(fmaxf(c, -448.f), 448.f);
+  d = fminf(fmaxf(d, -448.f), 448.f);
+  int v = 0;
+  v = __builtin_amdgcn_cvt_pk_fp8_f32(a, b, v, false);
+  v = __builtin_amdgcn_cvt_pk_fp8_f32(c, d, v, true);
+  return (uint32_t)v;
+}
+__device__ __forceinline__ uint8_t f32_to_fp8(float a) {
+  a = fminf(fmaxf(a, -448.f), 448.f);
+  int v = __builtin_amdgcn_cvt_pk_fp8_f32(a, a, 0, false);
+  return (uint8_t)(v & 0xff);
+}
+__device__ __forceinline__ float fp8_to_f32(uint8_t b) { return __builtin_amdgcn_cvt_f32_fp8((int)b, 0); }
+
+// ---- activations ---------------------------------------------------------------
+__device__ __forceinline__ float act_gelu(float x) { return 0.5f * x * (1.0f + erff(x * 0.70710678118654752f)); }
+// mish(x) = x * tanh(softplus(x)); with n = e^x, tanh(log(1+n)) = (n^2+2n)/(n^2+2n+2).
+__device__ __forceinline__ float act_mish(float x) {
+  if (x > 20.f) return x;
+  float n = __expf(x);
+  float t = n * (n + 2.f);
+  return x * (t / (t + 2.f));
+}
+__device__ __forceinline__ float act_swish(float x) { return x / (1.0f + __expf(-x)); }
+__device__ __forceinline__ float apply_act(float x, int act) {
+  switch (act) {
+    case ACT_GELU: return act_gelu(x);
+    case ACT_MISH: return act_mish(x);
+    case ACT_SWISH: return act_swish(x);
+    default: return x;
+  }
+}
+
+// ---- wave reductions (64 lanes) ---------------------------------------------------
+__device__ __forceinline__ float wave_sum(float v) {
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, 64);
+  return v;
+}
+__device__ __forceinline__ float wave_max(float v) {
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) v = fmaxf(v, __shfl_xor(v, o, 64));
+  return v;
+}
+
+// amax is kept as the bit pattern of a non-negative float so integer max orders it.
+__device__ __forceinline__ void atomic_amax(float* slot, float v) {
+  atomicMax(reinterpret_cast<unsigned int*>(slot), __float_as_uint(v));
+}
+
+// ---- argument blocks ---------------------------------------------------------------
+struct GemmArgs {
+  const void* A;      // activations [M,K], row stride lda elements
+  const void* W;      // weights [N,K] (nn.Linear layout), row stride ldw elements
+  void* C;            // output [M,N], row stride ldc elements
+  void* C2;           // optional second output for columns >= nsplit (written at column n-nsplit)
+  const float* bias;  // [N] fp32 or null
+  const void* res;    // optional residual [M,N], row stride ldr elements
+  float* amax;        // optional: max |output| is accumulated here
+  long lda, ldw, ldc, ldc2, ldr;
+  int M, N, K;
+  int nsplit;         // N if unused
+  int act;            // Act
+  int res_dtype;      // DType of res (bf16 or f32)
+  float descale;      // multiplies the accumulator (1/(scale_a*scale_w) for fp8 inputs)
+  float alpha;        // multiplies act(acc*descale+bias) before the residual is added
+  float out_scale;    // multiplies the final value before an fp8 store
+  int vec_ok;         // 1 if 4-wide stores/loads along N are aligned for C, C2 and res
+  int res_rows;       // >0: the residual has this many rows and row m reads row m % res_rows
+};
+
+struct LayerNormArgs {
+  const void* x;        // [rows, C]
+  const float* gamma;   // [C]
+  const float* beta;    // [C] or null
+  void* out;            // optional [rows, C] in out_dtype
+  uint8_t* out_fp8;     // optional [rows, C] e4m3, value*fp8_scale
+  float* amax;          // optional
+  long ldx, ldo;        // row strides in elements
+  int rows, C;
+  int in_dtype, out_dtype;
+  float eps, fp8_scale;
+};
+
+struct EmbedArgs {
+  const float* planes;  // [B*64, 19] or null when ids are given
+  const uint8_t* ids;   // [B,64] piece codes 0..12 (token order), with flags
+  const uint8_t* flags; // [B,4]
+  const float* w1t;     // [19, C] (transposed linear1.weight)
+  const float* b1;      // [C]
+  const float* ln_g; const float* ln_b;   // [C]
+  const float* gate_a_exp;  // [64, C] = exp(ma_gating.a)
+  const float* gate_b;      // [64, C]
+  const float* pe;          // optional [64, C] added after gating
+  void* out;            // [B*64, C] in out_dtype
+  uint8_t* out_fp8;     // optional
+  float* amax;
+  int tokens, C, out_dtype, act;
+  float eps, fp8_scale;
+};
+
+enum AttnMode : int { ATTN_PLAIN = 0, ATTN_CAUSAL = 1, ATTN_BIAS = 2, ATTN_RELSHIFT = 3 };
+
+struct AttnArgs {
+  const void* q; const void* k; const void* v;  // bf16, [B*64, ld*] with head h at column h*HS
+  long ldq, ldk, ldv;
+  const void* bias;     // ATTN_BIAS: bf16 [B,H,4096] in the kernel's register order
+  const void* pos;      // ATTN_RELSHIFT: bf16 [64, H*HS] projected positional table
+  const float* u_bias;  // ATTN_RELSHIFT: [H*HS]
+  const float* v_bias;  // ATTN_RELSHIFT: [H*HS]
+  void* out;            // [B*64, ldo] bf16 or fp8
+  long ldo;
+  float* amax;
+  int B, H, mode, out_dtype;
+  float scale, out_scale;
+};
+
+struct PolicyQKArgs {
+  const void* q; const void* k;   // bf16/f16 [B*64, ld], d_model contiguous
+  long ldq, ldk;
+  int in_dtype;                   // DT_BF16 or DT_F16
+  int B, C;
+  float scale;
+  // dense mode
+  void* dense; int dense_dtype; long ldd;   // [B, 4096], index = query*64 + key
+  // gather mode
+  float* logits; long ldl;                  // [B, 1858]
+  const int16_t* gidx;                      // [2][1858] (black-to-move table first, then white): from_token*64+to_token
+  const int8_t* gpromo;                     // [1858]: -1, or to_file*4 + piece (0 q, 1 r, 2 b)
+  const float* wpromo;                      // [4, C] promotion offset weights (q, r, b, n)
+  const uint8_t* white_to_move;             // [B]
+  int nmoves;
+};
+
+struct SoftmaxArgs {
+  const float* logits; long ldl;   // [B, V]
+  const uint8_t* mask; long ldm;   // optional [B, V], 1 = legal
+  float* probs; long ldp;          // optional [B, V]
+  int32_t* argmax;                 // optional [B]
+  int B, V;
+  float temperature;               // 0 -> one-hot at the arg-max
+};
+
+struct ScatterArgs {
+  const float* src; long lds;       // [B, 1858]
+  float* dst; long ldd;             // [B, 1929], fully written (zeros where no source)
+  const int32_t* inv_white;         // [1929]: source index for a white row, or -1
+  const int32_t* inv_black;         // [1929]: source index for a black row, or -1
+  const uint8_t* white_to_move;     // [B]
+  int B, nsrc, ndst;
+};
+
+// ---- launchers (one per kernel family) -------------------------------------------------
+// in_dt: element type of A and W; out_dt: element type of C/C2; tile: 0 auto, 1 = 64x64,
+// 2 = 128x128, 3 = 256x256 workgroup tile.
+hipError_t launch_gemm(GemmArgs a, int in_dt, int out_dt, int tile, hipStream_t st);
+hipError_t launch_layernorm(const LayerNormArgs& a, hipStream_t st);
+hipError_t launch_embed(const EmbedArgs& a, hipStream_t st);
+hipError_t launch_attention(const AttnArgs& a, int head_dim, hipStream_t st);
+hipError_t launch_policy_qk(const PolicyQKArgs& a, hipStream_t st);
+hipError_t launch_masked_softmax(const SoftmaxArgs& a, hipStream_t st);
+hipError_t launch_leela_to_rl(const ScatterArgs& a, hipStream_t st);
+hipError_t launch_extract_stm(const float* planes, uint8_t* white_to_move, int B, hipStream_t st);
+hipError_t launch_fill_f32(float* p, float v, long n, hipStream_t st);
+hipError_t launch_convert(const float* src, void* dst, long n, int dt, float scale, hipStream_t st);
+// Slot of (query i, key j) inside a 4096-element attention bias tile.
+int attn_bias_slot_host(int i, int j);
+
+}  // namespace crl

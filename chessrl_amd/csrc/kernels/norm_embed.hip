@@ -1,0 +1,242 @@
+// Row-wise LayerNorm and the board-token embedding.
+//
+// LayerNorm replaces F.layer_norm / nn.LayerNorm (eps 1e-5, affine) at
+// model_bis.py:34, new_paradigm/value.py:36-37,134 and utils/fen_encoder.py:57; the
+// residual sum it normalises is produced by the preceding GEMM's epilogue. It can
+// also emit an e4m3 copy of its output (value * scale) so the next fp8 GEMM needs no
+// separate quantise pass.
+//
+// The embedding kernel is FenEncoder.forward (utils/fen_encoder.py:61-67) and the
+// identical stem of BT4.forward (new_paradigm/value.py:159-167): Linear(19->C), GELU,
+// LayerNorm, x*exp(a)+b gating, plus the fixed sinusoid rows of model_bis.py:362-366
+// when a table is supplied.
+//
+// One 64-lane wave owns one row; a lane keeps VPL vectors of 8 consecutive columns in
+// registers, so a row is read once and the statistics are two wave reductions.
+#include "common.hpp"
+
+namespace crl {
+
+template <int DT>
+__device__ __forceinline__ void load8(const void* base, long off, float v[8]) {
+  if constexpr (DT == DT_F32) {
+    const float4* p = reinterpret_cast<const float4*>(reinterpret_cast<const float*>(base) + off);
+    float4 a = p[0], b = p[1];
+    v[0] = a.x; v[1] = a.y; v[2] = a.z; v[3] = a.w; v[4] = b.x; v[5] = b.y; v[6] = b.z; v[7] = b.w;
+  } else {
+    uint4 u = *reinterpret_cast<const uint4*>(reinterpret_cast<const uint16_t*>(base) + off);
+    const uint32_t w[4] = {u.x, u.y, u.z, u.w};
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      if constexpr (DT == DT_BF16) {
+        v[2 * i] = bf16_bits_to_f32((uint16_t)(w[i] & 0xffff));
+        v[2 * i + 1] = bf16_bits_to_f32((uint16_t)(w[i] >> 16));
+      } else {
+        v[2 * i] = f16_bits_to_f32((uint16_t)(w[i] & 0xffff));
+        v[2 * i + 1] = f16_bits_to_f32((uint16_t)(w[i] >> 16));
+      }
+    }
+  }
+}
+
+__device__ __forceinline__ void store8(void* base, long off, const float v[8], int dt) {
+  if (dt == DT_F32) {
+    float4* p = reinterpret_cast<float4*>(reinterpret_cast<float*>(base) + off);
+    p[0] = make_float4(v[0], v[1], v[2], v[3]);
+    p[1] = make_float4(v[4], v[5], v[6], v[7]);
+  } else if (dt == DT_BF16) {
+    uint4 u = make_uint4(pack_bf16x2(v[0], v[1]), pack_bf16x2(v[2], v[3]), pack_bf16x2(v[4], v[5]), pack_bf16x2(v[6], v[7]));
+    *reinterpret_cast<uint4*>(reinterpret_cast<uint16_t*>(base) + off) = u;
+  } else {
+    uint32_t w[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) w[i] = (uint32_t)f32_to_f16_bits(v[2 * i]) | ((uint32_t)f32_to_f16_bits(v[2 * i + 1]) << 16);
+    *reinterpret_cast<uint4*>(reinterpret_cast<uint16_t*>(base) + off) = make_uint4(w[0], w[1], w[2], w[3]);
+  }
+}
+
+__device__ __forceinline__ void store8_fp8(uint8_t* base, long off, const float v[8], float scale) {
+  uint2 u = make_uint2(pack_fp8x4(v[0] * scale, v[1] * scale, v[2] * scale, v[3] * scale),
+                       pack_fp8x4(v[4] * scale, v[5] * scale, v[6] * scale, v[7] * scale));
+  *reinterpret_cast<uint2*>(base + off) = u;
+}
+
+// Normalise the VPL*8 values a lane holds (columns col0(i) = (i*64+lane)*8) and write them.
+template <int VPL>
+__device__ __forceinline__ void ln_finish(float (&x)[VPL][8], int lane, int C, const float* gamma, const float* beta,
+                                           float eps, float (&y)[VPL][8]) {
+  float s = 0.f;
+#pragma unroll
+  for (int i = 0; i < VPL; ++i) {
+    if ((i * 64 + lane) * 8 < C) {
+#pragma unroll
+      for (int e = 0; e < 8; ++e) s += x[i][e];
+    }
+  }
+  const float mean = wave_sum(s) / (float)C;
+  float q = 0.f;
+#pragma unroll
+  for (int i = 0; i < VPL; ++i) {
+    if ((i * 64 + lane) * 8 < C) {
+#pragma unroll
+      for (int e = 0; e < 8; ++e) { const float d = x[i][e] - mean; q += d * d; }
+    }
+  }
+  const float rstd = rsqrtf(wave_sum(q) / (float)C + eps);
+#pragma unroll
+  for (int i = 0; i < VPL; ++i) {
+    const int col = (i * 64 + lane) * 8;
+    if (col < C) {
+      float gv[8], bv[8];
+      load8<DT_F32>(gamma, col, gv);
+      if (beta) load8<DT_F32>(beta, col, bv);
+#pragma unroll
+      for (int e = 0; e < 8; ++e) y[i][e] = (x[i][e] - mean) * rstd * gv[e] + (beta ? bv[e] : 0.f);
+    }
+  }
+}
+
+template <int IN_DT, int VPL>
+__global__ void __launch_bounds__(256) layernorm_kernel(const LayerNormArgs a) {
+  const int lane = threadIdx.x & 63;
+  const int row = blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (row >= a.rows) return;
+  float x[VPL][8], y[VPL][8];
+#pragma unroll
+  for (int i = 0; i < VPL; ++i) {
+    const int col = (i * 64 + lane) * 8;
+    if (col < a.C) load8<IN_DT>(a.x, (long)row * a.ldx + col, x[i]);
+  }
+  ln_finish<VPL>(x, lane, a.C, a.gamma, a.beta, a.eps, y);
+  float am = 0.f;
+#pragma unroll
+  for (int i = 0; i < VPL; ++i) {
+    const int col = (i * 64 + lane) * 8;
+    if (col < a.C) {
+      if (a.out) store8(a.out, (long)row * a.ldo + col, y[i], a.out_dtype);
+      if (a.out_fp8) store8_fp8(a.out_fp8, (long)row * a.ldo + col, y[i], a.fp8_scale);
+      if (a.amax) {
+#pragma unroll
+        for (int e = 0; e < 8; ++e) am = fmaxf(am, fabsf(y[i][e]));
+      }
+    }
+  }
+  if (a.amax) {
+    am = wave_max(am);
+    if (lane == 0) atomic_amax(a.amax, am);
+  }
+}
+
+template <int IN_DT>
+static hipError_t launch_ln_dt(const LayerNormArgs& a, hipStream_t st) {
+  const dim3 grid((a.rows + 3) / 4), block(256);
+  const int vecs = (a.C / 8 + 63) / 64;
+  if (vecs <= 1) hipLaunchKernelGGL((layernorm_kernel<IN_DT, 1>), grid, block, 0, st, a);
+  else if (vecs <= 2) hipLaunchKernelGGL((layernorm_kernel<IN_DT, 2>), grid, block, 0, st, a);
+  else if (vecs <= 4) hipLaunchKernelGGL((layernorm_kernel<IN_DT, 4>), grid, block, 0, st, a);
+  else if (vecs <= 16) hipLaunchKernelGGL((layernorm_kernel<IN_DT, 16>), grid, block, 0, st, a);
+  else return hipErrorInvalidValue;
+  return hipGetLastError();
+}
+
+hipError_t launch_layernorm(const LayerNormArgs& a, hipStream_t st) {
+  if (a.rows <= 0) return hipSuccess;
+  if (a.C % 8 || a.ldx % 8 || a.ldo % 8 || a.C > 8192) return hipErrorInvalidValue;
+  switch (a.in_dtype) {
+    case DT_F32: return launch_ln_dt<DT_F32>(a, st);
+    case DT_BF16: return launch_ln_dt<DT_BF16>(a, st);
+    case DT_F16: return launch_ln_dt<DT_F16>(a, st);
+  }
+  return hipErrorInvalidValue;
+}
+
+// ---- embedding ------------------------------------------------------------------------
+template <int VPL>
+__global__ void __launch_bounds__(256) embed_kernel(const EmbedArgs a) {
+  const int lane = threadIdx.x & 63;
+  const int tok = blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (tok >= a.tokens) return;
+  const int sqr = tok & 63;
+
+  // The 19 input features of this token (uniform across the wave).
+  float f[19];
+  if (a.planes) {
+#pragma unroll
+    for (int p = 0; p < 19; ++p) f[p] = a.planes[(long)tok * 19 + p];
+  } else {
+    const int b = tok >> 6;
+    const int id = a.ids[tok];
+    const uint8_t* fl = a.flags + b * 4;
+#pragma unroll
+    for (int p = 0; p < 12; ++p) f[p] = (id == p + 1) ? 1.f : 0.f;
+    f[12] = fl[0] ? 1.f : 0.f;
+    f[13] = (fl[2] == sqr) ? 1.f : 0.f;
+    f[14] = (fl[1] & 1) ? 1.f : 0.f;
+    f[15] = (fl[1] & 2) ? 1.f : 0.f;
+    f[16] = (fl[1] & 4) ? 1.f : 0.f;
+    f[17] = (fl[1] & 8) ? 1.f : 0.f;
+    f[18] = fminf((float)fl[3] / 100.0f, 1.0f);
+  }
+
+  float x[VPL][8], y[VPL][8];
+#pragma unroll
+  for (int i = 0; i < VPL; ++i) {
+    const int col = (i * 64 + lane) * 8;
+    if (col < a.C) {
+      load8<DT_F32>(a.b1, col, x[i]);
+#pragma unroll
+      for (int p = 0; p < 19; ++p) {
+        if (f[p] != 0.f) {  // uniform branch: most planes are zero for a given token
+          float w[8];
+          load8<DT_F32>(a.w1t, (long)p * a.C + col, w);
+#pragma unroll
+          for (int e = 0; e < 8; ++e) x[i][e] = fmaf(f[p], w[e], x[i][e]);
+        }
+      }
+#pragma unroll
+      for (int e = 0; e < 8; ++e) x[i][e] = apply_act(x[i][e], a.act);
+    }
+  }
+  ln_finish<VPL>(x, lane, a.C, a.ln_g, a.ln_b, a.eps, y);
+  float am = 0.f;
+#pragma unroll
+  for (int i = 0; i < VPL; ++i) {
+    const int col = (i * 64 + lane) * 8;
+    if (col < a.C) {
+      float ga[8], gb[8];
+      load8<DT_F32>(a.gate_a_exp, (long)sqr * a.C + col, ga);
+      load8<DT_F32>(a.gate_b, (long)sqr * a.C + col, gb);
+#pragma unroll
+      for (int e = 0; e < 8; ++e) y[i][e] = y[i][e] * ga[e] + gb[e];
+      if (a.pe) {
+        float pe[8];
+        load8<DT_F32>(a.pe, (long)sqr * a.C + col, pe);
+#pragma unroll
+        for (int e = 0; e < 8; ++e) y[i][e] += pe[e];
+      }
+      store8(a.out, (long)tok * a.C + col, y[i], a.out_dtype);
+      if (a.out_fp8) store8_fp8(a.out_fp8, (long)tok * a.C + col, y[i], a.fp8_scale);
+      if (a.amax) {
+#pragma unroll
+        for (int e = 0; e < 8; ++e) am = fmaxf(am, fabsf(y[i][e]));
+      }
+    }
+  }
+  if (a.amax) {
+    am = wave_max(am);
+    if (lane == 0) atomic_amax(a.amax, am);
+  }
+}
+
+hipError_t launch_embed(const EmbedArgs& a, hipStream_t st) {
+  if (a.tokens <= 0) return hipSuccess;
+  if (a.C % 8 || a.C > 2048) return hipErrorInvalidValue;
+  const dim3 grid((a.tokens + 3) / 4), block(256);
+  const int vecs = (a.C / 8 + 63) / 64;
+  if (vecs <= 1) hipLaunchKernelGGL((embed_kernel<1>), grid, block, 0, st, a);
+  else if (vecs <= 2) hipLaunchKernelGGL((embed_kernel<2>), grid, block, 0, st, a);
+  else hipLaunchKernelGGL((embed_kernel<4>), grid, block, 0, st, a);
+  return hipGetLastError();
+}
+
+}  // namespace crl

@@ -1,0 +1,622 @@
+// Host-side model runner: owns the packed device weights and the workspace of one
+// model and issues the kernel sequence of its forward pass on the caller's stream.
+//
+// Three architectures share the kernels:
+//   GPT64    model_bis.GPT restricted to the 64 board tokens (model_bis.py:358-370):
+//            pre-LN blocks, causal attention, logits of token 63 through lm_head.
+//   BT4      new_paradigm/value.py BT4: post-LN encoder with relative-position attention,
+//            attention-policy head with the dense 4096->1929 map, WDL value head.
+//   BT4CLASS the benchmark's BT4-class encoder: post-LN with residual scaling
+//            alpha=(2L)^-1/4, mish FFN, generated attention bias (smolgen), attention
+//            policy gathered to the 1858-move list, WDL head. Not present in the
+//            reference repository; defined by this build.
+#include "model.hpp"
+
+#include <cmath>
+#include <cstdio>
+#include <cstring>
+
+namespace crl {
+
+#define HIPCHK(expr)                                                                      \
+  do {                                                                                    \
+    hipError_t e_ = (expr);                                                               \
+    if (e_ != hipSuccess) {                                                               \
+      set_error(std::string(#expr) + ": " + hipGetErrorString(e_));                       \
+      return CRL_ERR_HIP;                                                                 \
+    }                                                                                     \
+  } while (0)
+
+static thread_local std::string g_error;
+void set_error(const std::string& s) { g_error = s; }
+const char* get_error() { return g_error.c_str(); }
+
+static std::string lkey(const char* fmt, int i) {
+  char buf[160];
+  std::snprintf(buf, sizeof(buf), fmt, i);
+  return buf;
+}
+
+Model::Model(const crl_model_config& c) : cfg(c) {
+  if (cfg.eps == 0.f) cfg.eps = 1e-5f;
+  if (cfg.smolgen_compress == 0) cfg.smolgen_compress = 32;
+  if (cfg.smolgen_hidden == 0) cfg.smolgen_hidden = 256;
+  if (cfg.smolgen_gen == 0) cfg.smolgen_gen = 256;
+  if (cfg.head_dtype != DT_F16) cfg.head_dtype = DT_BF16;
+  if (cfg.micro_batch <= 0) cfg.micro_batch = 1024;
+  vocab = cfg.arch == CRL_ARCH_BT4CLASS ? VOCAB_LEELA : VOCAB_RL;
+  const long C = cfg.d_model, F = cfg.d_ff, L = cfg.n_layer, H = cfg.n_head;
+  auto add = [&](const std::string& k, long n) { expected.push_back({k, n}); };
+  auto lin = [&](const std::string& k, long out, long in, bool bias = true) {
+    add(k + ".weight", out * in);
+    if (bias) add(k + ".bias", out);
+  };
+  auto ln = [&](const std::string& k, long n) { add(k + ".weight", n); add(k + ".bias", n); };
+  if (cfg.arch == CRL_ARCH_GPT64) {
+    lin("FenEncoder.linear1", C, 19); ln("FenEncoder.layernorm1", C);
+    add("FenEncoder.ma_gating.a", 64 * C); add("FenEncoder.ma_gating.b", 64 * C);
+    for (int i = 0; i < L; ++i) {
+      const std::string p = lkey("transformer.h.%d.", i);
+      ln(p + "ln_1", C); lin(p + "attn.c_attn", 3 * C, C); lin(p + "attn.c_proj", C, C);
+      ln(p + "ln_2", C); lin(p + "mlp.c_fc", F, C); lin(p + "mlp.c_proj", C, F);
+    }
+    ln("transformer.ln_f", C);
+    add("lm_head.weight", (long)VOCAB_RL * C);
+    add("pe", 64 * C);
+  } else {
+    lin("linear1", C, 19); ln("layernorm1", C);
+    add("ma_gating.a", 64 * C); add("ma_gating.b", 64 * C);
+    for (int i = 0; i < L; ++i) {
+      const std::string p = lkey("layers.%d.", i);
+      lin(p + "attention.query_proj", C, C); lin(p + "attention.key_proj", C, C);
+      lin(p + "attention.value_proj", C, C); lin(p + "attention.out_proj", C, C);
+      if (cfg.arch == CRL_ARCH_BT4) {
+        add(p + "attention.pos_proj.weight", C * C);
+        add(p + "attention.u_bias", C); add(p + "attention.v_bias", C);
+      } else {
+        const long sc = cfg.smolgen_compress, sh = cfg.smolgen_hidden, sg = cfg.smolgen_gen;
+        add(p + "smolgen.compress.weight", sc * C);
+        lin(p + "smolgen.hidden", sh, 64 * sc); ln(p + "smolgen.hidden_ln", sh);
+        lin(p + "smolgen.gen_from", H * sg, sh); ln(p + "smolgen.gen_from_ln", H * sg);
+      }
+      ln(p + "norm1", C); ln(p + "norm2", C);
+      lin(p + "ff1", F, C); lin(p + "ff2", C, F);
+    }
+    lin("policy_tokens_lin", C, C); lin("queries_pol", C, C); lin("keys_pol", C, C);
+    if (cfg.arch == CRL_ARCH_BT4) add("policy_head.weight", (long)VOCAB_RL * 4096);
+    else {
+      add("smol_weight_gen.weight", 4096L * cfg.smolgen_gen);
+      add("promotion_offsets.weight", 4 * C);
+    }
+    lin("value_head.dense1", 128, C); lin("value_head.dense2", 128, 128 * 64); lin("value_head.dense3", 3, 128);
+  }
+  amax_host.assign((size_t)L * 4, 0.f);
+}
+
+Model::~Model() {
+  for (void* p : allocs) (void)hipFree(p);
+  for (void* p : ws_allocs) (void)hipFree(p);
+  for (auto& e : prof_events) { (void)hipEventDestroy(e.a); (void)hipEventDestroy(e.b); }
+}
+
+int Model::set_weight(const char* key, const float* data, long numel) {
+  if (!key || !data) { set_error("set_weight: null argument"); return CRL_ERR_ARG; }
+  std::string k = key;
+  if (k == "transformer.wte.weight") return CRL_OK;  // tied to lm_head.weight (model_bis.py:148)
+  for (auto& e : expected) {
+    if (e.first != k) continue;
+    const bool ok = (k == "pe") ? numel >= e.second : numel == e.second;
+    if (!ok) { set_error("set_weight: " + k + " has " + std::to_string(numel) + " elements, expected " + std::to_string(e.second)); return CRL_ERR_ARG; }
+    host[k].assign(data, data + e.second);
+    finalized = false;
+    return CRL_OK;
+  }
+  set_error("set_weight: unexpected key " + k);
+  return CRL_ERR_ARG;
+}
+
+// ---- device packing ---------------------------------------------------------------------
+int Model::dev_alloc(void** p, size_t bytes, bool ws) {
+  HIPCHK(hipMalloc(p, bytes ? bytes : 16));
+  (ws ? ws_allocs : allocs).push_back(*p);
+  return CRL_OK;
+}
+
+int Model::upload(const std::vector<float>& v, int dt, float scale, void** out) {
+  float* tmp = nullptr;
+  HIPCHK(hipMalloc((void**)&tmp, v.size() * sizeof(float)));
+  hipError_t e = hipMemcpy(tmp, v.data(), v.size() * sizeof(float), hipMemcpyHostToDevice);
+  if (e == hipSuccess) {
+    int rc = dev_alloc(out, v.size() * dtype_size(dt), false);
+    if (rc) { (void)hipFree(tmp); return rc; }
+    e = launch_convert(tmp, *out, (long)v.size(), dt, scale, nullptr);
+    if (e == hipSuccess) e = hipDeviceSynchronize();
+  }
+  (void)hipFree(tmp);
+  HIPCHK(e);
+  return CRL_OK;
+}
+
+const std::vector<float>& Model::w(const std::string& k) { return host.at(k); }
+
+int Model::make_lin(Lin& L, const std::vector<float>& W, const std::vector<float>* bias, int N, int K, int dt16, bool fp8) {
+  L.N = N; L.K = K; L.dt = dt16;
+  int rc = upload(W, dt16, 1.f, &L.w);
+  if (rc) return rc;
+  if (fp8) {
+    float am = 0.f;
+    for (float x : W) am = std::fmax(am, std::fabs(x));
+    L.wscale = am > 0.f ? 448.f / am : 1.f;
+    rc = upload(W, DT_FP8, L.wscale, &L.w8);
+    if (rc) return rc;
+  }
+  if (bias) {
+    rc = upload(*bias, DT_F32, 1.f, (void**)&L.b);
+    if (rc) return rc;
+  }
+  return CRL_OK;
+}
+
+static std::vector<float> cat(std::initializer_list<const std::vector<float>*> parts) {
+  std::vector<float> r;
+  for (auto* p : parts) r.insert(r.end(), p->begin(), p->end());
+  return r;
+}
+
+int Model::finalize() {
+  for (auto& e : expected)
+    if (!host.count(e.first)) { set_error("finalize: missing weight " + e.first); return CRL_ERR_STATE; }
+  for (void* p : allocs) (void)hipFree(p);
+  allocs.clear();
+  layers.assign(cfg.n_layer, Layer());
+  const int C = cfg.d_model, F = cfg.d_ff, H = cfg.n_head;
+  const bool f8 = cfg.fp8 != 0;
+  const int hd = cfg.head_dtype;
+  int rc;
+#define UP(vec, dt, out) do { rc = upload(vec, dt, 1.f, (void**)&(out)); if (rc) return rc; } while (0)
+#define LIN(L, W, B, N, K, dt, f) do { rc = make_lin(L, W, B, N, K, dt, f); if (rc) return rc; } while (0)
+  const std::string pre = cfg.arch == CRL_ARCH_GPT64 ? "FenEncoder." : "";
+  {
+    const auto& w1 = w(pre + "linear1.weight");  // [C,19] -> [19,C]
+    std::vector<float> w1t((size_t)19 * C);
+    for (int c = 0; c < C; ++c)
+      for (int p = 0; p < 19; ++p) w1t[(size_t)p * C + c] = w1[(size_t)c * 19 + p];
+    UP(w1t, DT_F32, emb_w1t);
+    UP(w(pre + "linear1.bias"), DT_F32, emb_b1);
+    UP(w(pre + "layernorm1.weight"), DT_F32, emb_g);
+    UP(w(pre + "layernorm1.bias"), DT_F32, emb_b);
+    std::vector<float> ea = w(pre + "ma_gating.a");
+    for (float& x : ea) x = std::exp(x);
+    UP(ea, DT_F32, gate_a_exp);
+    UP(w(pre + "ma_gating.b"), DT_F32, gate_b);
+  }
+  if (cfg.arch == CRL_ARCH_GPT64) {
+    UP(w("pe"), DT_F32, pe_f32);
+    for (int i = 0; i < cfg.n_layer; ++i) {
+      Layer& ly = layers[i];
+      const std::string p = lkey("transformer.h.%d.", i);
+      UP(w(p + "ln_1.weight"), DT_F32, ly.ln1_g); UP(w(p + "ln_1.bias"), DT_F32, ly.ln1_b);
+      UP(w(p + "ln_2.weight"), DT_F32, ly.ln2_g); UP(w(p + "ln_2.bias"), DT_F32, ly.ln2_b);
+      LIN(ly.qkv, w(p + "attn.c_attn.weight"), &w(p + "attn.c_attn.bias"), 3 * C, C, DT_BF16, f8);
+      LIN(ly.proj, w(p + "attn.c_proj.weight"), &w(p + "attn.c_proj.bias"), C, C, DT_BF16, f8);
+      LIN(ly.ff1, w(p + "mlp.c_fc.weight"), &w(p + "mlp.c_fc.bias"), F, C, DT_BF16, f8);
+      LIN(ly.ff2, w(p + "mlp.c_proj.weight"), &w(p + "mlp.c_proj.bias"), C, F, DT_BF16, f8);
+    }
+    UP(w("transformer.ln_f.weight"), DT_F32, lnf_g); UP(w("transformer.ln_f.bias"), DT_F32, lnf_b);
+    LIN(lm_head, w("lm_head.weight"), nullptr, VOCAB_RL, C, hd, false);
+  } else {
+    // Absolute sinusoid table of new_paradigm/value.py:77-93.
+    std::vector<float> pe((size_t)64 * C);
+    for (int p = 0; p < 64; ++p)
+      for (int i = 0; i < C; i += 2) {
+        const float d = std::pow(10000.0f, (float)i / (float)C);
+        pe[(size_t)p * C + i] = std::sin((float)p / d);
+        if (i + 1 < C) pe[(size_t)p * C + i + 1] = std::cos((float)p / d);
+      }
+    UP(pe, hd, pe_head);
+    for (int i = 0; i < cfg.n_layer; ++i) {
+      Layer& ly = layers[i];
+      const std::string p = lkey("layers.%d.", i);
+      std::vector<float> wq = cat({&w(p + "attention.query_proj.weight"), &w(p + "attention.key_proj.weight"), &w(p + "attention.value_proj.weight")});
+      std::vector<float> bq = cat({&w(p + "attention.query_proj.bias"), &w(p + "attention.key_proj.bias"), &w(p + "attention.value_proj.bias")});
+      int nq = 3 * C;
+      if (cfg.arch == CRL_ARCH_BT4CLASS) {
+        const auto& cw = w(p + "smolgen.compress.weight");
+        wq.insert(wq.end(), cw.begin(), cw.end());
+        bq.insert(bq.end(), (size_t)cfg.smolgen_compress, 0.f);
+        nq += cfg.smolgen_compress;
+      }
+      LIN(ly.qkv, wq, &bq, nq, C, DT_BF16, f8);
+      LIN(ly.proj, w(p + "attention.out_proj.weight"), &w(p + "attention.out_proj.bias"), C, C, DT_BF16, f8);
+      LIN(ly.ff1, w(p + "ff1.weight"), &w(p + "ff1.bias"), F, C, DT_BF16, f8);
+      LIN(ly.ff2, w(p + "ff2.weight"), &w(p + "ff2.bias"), C, F, DT_BF16, f8);
+      UP(w(p + "norm1.weight"), DT_F32, ly.ln1_g); UP(w(p + "norm1.bias"), DT_F32, ly.ln1_b);
+      UP(w(p + "norm2.weight"), DT_F32, ly.ln2_g); UP(w(p + "norm2.bias"), DT_F32, ly.ln2_b);
+      if (cfg.arch == CRL_ARCH_BT4) {
+        // pos_proj(PE) does not depend on the input (new_paradigm/attn.py:505): fold it here.
+        const auto& pw = w(p + "attention.pos_proj.weight");
+        std::vector<float> pt((size_t)64 * C);
+        for (int t = 0; t < 64; ++t)
+          for (int o = 0; o < C; ++o) {
+            double s = 0;
+            for (int c = 0; c < C; ++c) s += (double)pe[(size_t)t * C + c] * pw[(size_t)o * C + c];
+            pt[(size_t)t * C + o] = (float)s;
+          }
+        UP(pt, DT_BF16, ly.pos);
+        UP(w(p + "attention.u_bias"), DT_F32, ly.u_bias);
+        UP(w(p + "attention.v_bias"), DT_F32, ly.v_bias);
+      } else {
+        const int sc = cfg.smolgen_compress, sh = cfg.smolgen_hidden, sg = cfg.smolgen_gen;
+        LIN(ly.sm_hidden, w(p + "smolgen.hidden.weight"), &w(p + "smolgen.hidden.bias"), sh, 64 * sc, DT_BF16, false);
+        LIN(ly.sm_gen, w(p + "smolgen.gen_from.weight"), &w(p + "smolgen.gen_from.bias"), H * sg, sh, DT_BF16, false);
+        UP(w(p + "smolgen.hidden_ln.weight"), DT_F32, ly.sm_ln1_g); UP(w(p + "smolgen.hidden_ln.bias"), DT_F32, ly.sm_ln1_b);
+        UP(w(p + "smolgen.gen_from_ln.weight"), DT_F32, ly.sm_ln2_g); UP(w(p + "smolgen.gen_from_ln.bias"), DT_F32, ly.sm_ln2_b);
+      }
+    }
+    LIN(pol_tok, w("policy_tokens_lin.weight"), &w("policy_tokens_lin.bias"), C, C, hd, false);
+    {
+      std::vector<float> wqk = cat({&w("queries_pol.weight"), &w("keys_pol.weight")});
+      std::vector<float> bqk = cat({&w("queries_pol.bias"), &w("keys_pol.bias")});
+      LIN(pol_qk, wqk, &bqk, 2 * C, C, hd, false);
+    }
+    if (cfg.arch == CRL_ARCH_BT4) {
+      LIN(pol_head, w("policy_head.weight"), nullptr, VOCAB_RL, 4096, hd, false);
+    } else {
+      // Rows of the shared bias generator are stored in the order the attention kernel
+      // reads its accumulator registers, so the generated tile needs no transpose.
+      const int sg = cfg.smolgen_gen;
+      const auto& gw = w("smol_weight_gen.weight");
+      std::vector<float> perm((size_t)4096 * sg);
+      for (int i = 0; i < 64; ++i)
+        for (int j = 0; j < 64; ++j)
+          std::memcpy(&perm[(size_t)attn_bias_slot_host(i, j) * sg], &gw[(size_t)(i * 64 + j) * sg], sizeof(float) * sg);
+      LIN(sm_weight_gen, perm, nullptr, 4096, sg, DT_BF16, false);
+      UP(w("promotion_offsets.weight"), DT_F32, promo_w);
+      // Gather tables: Leela move v -> (from_token*64+to_token) for black / white rows.
+      std::vector<int16_t> gi((size_t)2 * VOCAB_LEELA);
+      std::vector<int8_t> gp(VOCAB_LEELA);
+      const auto& names = policy_leela();
+      for (int v = 0; v < VOCAB_LEELA; ++v) {
+        const std::string& s = names[v];
+        const int ff = s[0] - 'a', fr = s[1] - '1', tf = s[2] - 'a', tr = s[3] - '1';
+        // white row: squares as written; black row: ranks mirrored back to the real board.
+        gi[VOCAB_LEELA + v] = (int16_t)(((7 - fr) * 8 + ff) * 64 + ((7 - tr) * 8 + tf));
+        gi[v] = (int16_t)((fr * 8 + ff) * 64 + (tr * 8 + tf));
+        gp[v] = s.size() == 5 ? (int8_t)(tf * 4 + (s[4] == 'q' ? 0 : s[4] == 'r' ? 1 : 2)) : (int8_t)-1;
+      }
+      rc = dev_alloc((void**)&gidx, gi.size() * 2, false); if (rc) return rc;
+      rc = dev_alloc((void**)&gpromo, gp.size(), false); if (rc) return rc;
+      HIPCHK(hipMemcpy(gidx, gi.data(), gi.size() * 2, hipMemcpyHostToDevice));
+      HIPCHK(hipMemcpy(gpromo, gp.data(), gp.size(), hipMemcpyHostToDevice));
+    }
+    LIN(val1, w("value_head.dense1.weight"), &w("value_head.dense1.bias"), 128, C, hd, false);
+    LIN(val2, w("value_head.dense2.weight"), &w("value_head.dense2.bias"), 128, 8192, hd, false);
+    LIN(val3, w("value_head.dense3.weight"), &w("value_head.dense3.bias"), 3, 128, hd, false);
+  }
+  rc = dev_alloc((void**)&amax_dev, sizeof(float) * amax_host.size(), false);
+  if (rc) return rc;
+  HIPCHK(hipMemset(amax_dev, 0, sizeof(float) * amax_host.size()));
+#undef UP
+#undef LIN
+  finalized = true;
+  return CRL_OK;
+}
+
+// ---- workspace ------------------------------------------------------------------------------
+int Model::ensure_ws(int mb) {
+  if (mb <= ws_mb) return CRL_OK;
+  for (void* p : ws_allocs) (void)hipFree(p);
+  ws_allocs.clear();
+  ws_mb = 0;
+  const size_t M = (size_t)mb * 64, C = cfg.d_model, F = cfg.d_ff, H = cfg.n_head;
+  int rc;
+#define WS(ptr, bytes) do { rc = dev_alloc((void**)&(ptr), (bytes), true); if (rc) return rc; } while (0)
+  WS(ws.x, M * C * 4);        // residual stream (fp32 for GPT64 with stream_f32, else 16-bit)
+  WS(ws.x8, M * C);
+  WS(ws.t, M * C * 2);
+  WS(ws.h, M * C * 2);
+  WS(ws.h8, M * C);
+  WS(ws.qkv, M * 3 * C * 2);
+  WS(ws.ao, M * C * 2);
+  WS(ws.ao8, M * C);
+  WS(ws.f, M * F * 2);
+  WS(ws.f8, M * F);
+  WS(ws.stm, (size_t)mb);
+  if (cfg.arch == CRL_ARCH_BT4CLASS) {
+    WS(ws.comp, M * cfg.smolgen_compress * 2);
+    WS(ws.sh1, (size_t)mb * cfg.smolgen_hidden * 2);
+    WS(ws.sh2, (size_t)mb * cfg.smolgen_hidden * 2);
+    WS(ws.sg1, (size_t)mb * H * cfg.smolgen_gen * 2);
+    WS(ws.sg2, (size_t)mb * H * cfg.smolgen_gen * 2);
+    WS(ws.bias, (size_t)mb * H * 4096 * 2);
+  }
+  if (cfg.arch == CRL_ARCH_GPT64) {
+    WS(ws.hl, (size_t)mb * C * 2);
+  } else {
+    WS(ws.tok, M * C * 2);
+    WS(ws.pqk, M * 2 * C * 2);
+    WS(ws.v1, M * 128 * 2);
+    WS(ws.v2, (size_t)mb * 128 * 2);
+    WS(ws.dense, (size_t)mb * 4096 * 2);
+  }
+#undef WS
+  ws_mb = mb;
+  return CRL_OK;
+}
+
+// ---- profiling helpers ------------------------------------------------------------------------
+void Model::prof_begin(int fam, hipStream_t st) {
+  if (!profiling) return;
+  if (prof_used == prof_events.size()) {
+    ProfEvent e;
+    (void)hipEventCreate(&e.a);
+    (void)hipEventCreate(&e.b);
+    prof_events.push_back(e);
+  }
+  prof_events[prof_used].fam = fam;
+  (void)hipEventRecord(prof_events[prof_used].a, st);
+}
+void Model::prof_end(hipStream_t st) {
+  if (!profiling) return;
+  (void)hipEventRecord(prof_events[prof_used].b, st);
+  ++prof_used;
+}
+void Model::prof_collect(hipStream_t st) {
+  if (!profiling) return;
+  (void)hipStreamSynchronize(st);
+  for (size_t i = 0; i < prof_used; ++i) {
+    float ms = 0.f;
+    if (hipEventElapsedTime(&ms, prof_events[i].a, prof_events[i].b) == hipSuccess) {
+      prof_ms[prof_events[i].fam] += ms;
+      prof_n[prof_events[i].fam] += 1;
+    }
+  }
+  prof_used = 0;
+}
+
+// ---- launch helpers ------------------------------------------------------------------------------
+struct GOpt {
+  int act = ACT_NONE;
+  float alpha = 1.f;
+  const void* res = nullptr; long ldr = 0; int res_dt = DT_BF16; int res_rows = 0;
+  float a_scale = 1.f;     // scale the fp8 A operand was quantised with
+  float out_scale = 1.f;
+  float* amax = nullptr;
+  void* C2 = nullptr; long ldc2 = 0; int nsplit = 0;
+};
+
+int Model::gemm(const Lin& L, const void* A, long lda, int in_dt, void* C, long ldc, int out_dt, int M, const GOpt& o, hipStream_t st) {
+  GemmArgs g;
+  std::memset(&g, 0, sizeof(g));
+  g.A = A; g.lda = lda;
+  g.W = in_dt == DT_FP8 ? L.w8 : L.w; g.ldw = L.K;
+  if (!g.W) { set_error("gemm: weight copy for the requested element type is missing"); return CRL_ERR_STATE; }
+  g.C = C; g.ldc = ldc; g.C2 = o.C2; g.ldc2 = o.ldc2; g.nsplit = o.nsplit > 0 ? o.nsplit : L.N;
+  g.bias = L.b; g.res = o.res; g.ldr = o.ldr; g.res_dtype = o.res_dt; g.res_rows = o.res_rows;
+  g.amax = o.amax; g.M = M; g.N = L.N; g.K = L.K; g.act = o.act;
+  g.descale = in_dt == DT_FP8 ? 1.f / (o.a_scale * L.wscale) : 1.f;
+  g.alpha = o.alpha; g.out_scale = o.out_scale;
+  prof_begin(0, st);
+  hipError_t e = launch_gemm(g, in_dt == DT_FP8 ? DT_FP8 : L.dt, out_dt, 0, st);
+  prof_end(st);
+  HIPCHK(e);
+  return CRL_OK;
+}
+
+int Model::lnorm(const void* x, long ldx, int in_dt, const float* g, const float* b, void* out, int out_dt, uint8_t* out8,
+                 float scale8, long ldo, int rows, int C, float* amax, hipStream_t st) {
+  LayerNormArgs a;
+  std::memset(&a, 0, sizeof(a));
+  a.x = x; a.ldx = ldx; a.in_dtype = in_dt; a.gamma = g; a.beta = b; a.out = out; a.out_dtype = out_dt;
+  a.out_fp8 = out8; a.fp8_scale = scale8; a.ldo = ldo; a.rows = rows; a.C = C; a.eps = cfg.eps; a.amax = amax;
+  prof_begin(2, st);
+  hipError_t e = launch_layernorm(a, st);
+  prof_end(st);
+  HIPCHK(e);
+  return CRL_OK;
+}
+
+float Model::act_scale(int layer, int slot) const {
+  const float am = amax_host[(size_t)layer * 4 + slot];
+  return am > 0.f ? 448.f / am : 1.f;
+}
+
+int Model::forward(const float* planes, const uint8_t* ids, const uint8_t* flags, int B, float* policy, float* wdl,
+                   bool calibrate, hipStream_t st) {
+  if (!finalized) { set_error("forward: call crl_model_finalize first"); return CRL_ERR_STATE; }
+  if (B < 0 || (!planes && !(ids && flags)) || !policy) { set_error("forward: bad arguments"); return CRL_ERR_ARG; }
+  const int mbmax = cfg.micro_batch;
+  int rc = ensure_ws(B < mbmax ? B : mbmax);
+  if (rc) return rc;
+  for (int b0 = 0; b0 < B; b0 += mbmax) {
+    const int mb = (B - b0) < mbmax ? (B - b0) : mbmax;
+    rc = forward_chunk(planes ? planes + (size_t)b0 * 64 * 19 : nullptr, ids ? ids + (size_t)b0 * 64 : nullptr,
+                       flags ? flags + (size_t)b0 * 4 : nullptr, mb, policy + (size_t)b0 * vocab, wdl ? wdl + (size_t)b0 * 3 : nullptr,
+                       calibrate, st);
+    if (rc) return rc;
+  }
+  prof_collect(st);
+  return CRL_OK;
+}
+
+int Model::forward_chunk(const float* planes, const uint8_t* ids, const uint8_t* flags, int mb, float* policy, float* wdl,
+                         bool calibrate, hipStream_t st) {
+  const int C = cfg.d_model, F = cfg.d_ff, H = cfg.n_head, L = cfg.n_layer, hs = C / H;
+  const int M = mb * 64;
+  const bool f8 = cfg.fp8 && !calibrate;
+  const int hd = cfg.head_dtype;
+  const bool gpt = cfg.arch == CRL_ARCH_GPT64;
+  const bool sf32 = gpt && cfg.stream_f32;
+  const int xdt = sf32 ? DT_F32 : DT_BF16;
+  auto am = [&](int l, int slot) -> float* { return calibrate ? amax_dev + (size_t)l * 4 + slot : nullptr; };
+  int rc;
+#define RUN(call) do { rc = (call); if (rc) return rc; } while (0)
+
+  // ---- embedding
+  {
+    EmbedArgs e;
+    std::memset(&e, 0, sizeof(e));
+    e.planes = planes; e.ids = ids; e.flags = flags;
+    e.w1t = emb_w1t; e.b1 = emb_b1; e.ln_g = emb_g; e.ln_b = emb_b; e.gate_a_exp = gate_a_exp; e.gate_b = gate_b;
+    e.pe = gpt ? pe_f32 : nullptr;
+    e.out = ws.x; e.out_dtype = (L == 0 && !gpt) ? hd : xdt; e.tokens = M; e.C = C; e.act = ACT_GELU; e.eps = cfg.eps;
+    if (!gpt && L > 0) { e.out_fp8 = f8 ? ws.x8 : nullptr; e.fp8_scale = f8 ? act_scale(0, 0) : 1.f; e.amax = am(0, 0); }
+    prof_begin(3, st);
+    hipError_t he = launch_embed(e, st);
+    prof_end(st);
+    HIPCHK(he);
+  }
+  if (cfg.arch == CRL_ARCH_BT4CLASS) {
+    if (planes) HIPCHK(launch_extract_stm(planes, ws.stm, mb, st));
+    else HIPCHK(hipMemcpy2DAsync(ws.stm, 1, flags, 4, 1, mb, hipMemcpyDeviceToDevice, st));
+  }
+
+  const float attn_scale = cfg.arch == CRL_ARCH_BT4 ? 1.0f / std::sqrt((float)C) : 1.0f / std::sqrt((float)hs);
+  const float alpha = cfg.arch == CRL_ARCH_BT4CLASS ? std::pow(2.0f * (float)L, -0.25f) : 1.0f;
+
+  for (int l = 0; l < L; ++l) {
+    const Layer& ly = layers[l];
+    const bool last = l + 1 == L;
+    const void* a_in; int a_dt; float a_sc = 1.f;
+    if (gpt) {
+      // h = LN1(x)
+      RUN(lnorm(ws.x, C, xdt, ly.ln1_g, ly.ln1_b, f8 ? nullptr : ws.h, DT_BF16, f8 ? ws.h8 : nullptr, f8 ? act_scale(l, 0) : 1.f, C, M, C, am(l, 0), st));
+      a_in = f8 ? (const void*)ws.h8 : (const void*)ws.h; a_dt = f8 ? DT_FP8 : DT_BF16; a_sc = f8 ? act_scale(l, 0) : 1.f;
+    } else {
+      a_in = f8 ? (const void*)ws.x8 : (const void*)ws.x; a_dt = f8 ? DT_FP8 : DT_BF16; a_sc = f8 ? act_scale(l, 0) : 1.f;
+    }
+    // q|k|v (and the smolgen compression for BT4-class) in one GEMM
+    {
+      GOpt o; o.a_scale = a_sc;
+      if (cfg.arch == CRL_ARCH_BT4CLASS) { o.C2 = ws.comp; o.ldc2 = cfg.smolgen_compress; o.nsplit = 3 * C; }
+      RUN(gemm(ly.qkv, a_in, C, a_dt, ws.qkv, 3 * C, DT_BF16, M, o, st));
+    }
+    const void* bias_tile = nullptr;
+    if (cfg.arch == CRL_ARCH_BT4CLASS) {
+      const int sc = cfg.smolgen_compress, sh = cfg.smolgen_hidden, sg = cfg.smolgen_gen;
+      GOpt o; o.act = ACT_SWISH;
+      RUN(gemm(ly.sm_hidden, ws.comp, 64 * sc, DT_BF16, ws.sh1, sh, DT_BF16, mb, o, st));
+      RUN(lnorm(ws.sh1, sh, DT_BF16, ly.sm_ln1_g, ly.sm_ln1_b, ws.sh2, DT_BF16, nullptr, 1.f, sh, mb, sh, nullptr, st));
+      RUN(gemm(ly.sm_gen, ws.sh2, sh, DT_BF16, ws.sg1, H * sg, DT_BF16, mb, o, st));
+      RUN(lnorm(ws.sg1, H * sg, DT_BF16, ly.sm_ln2_g, ly.sm_ln2_b, ws.sg2, DT_BF16, nullptr, 1.f, H * sg, mb, H * sg, nullptr, st));
+      GOpt o2;
+      RUN(gemm(sm_weight_gen, ws.sg2, sg, DT_BF16, ws.bias, 4096, DT_BF16, mb * H, o2, st));
+      bias_tile = ws.bias;
+    }
+    // attention
+    {
+      AttnArgs a;
+      std::memset(&a, 0, sizeof(a));
+      const uint16_t* base = reinterpret_cast<const uint16_t*>(ws.qkv);
+      a.q = base; a.k = base + C; a.v = base + 2 * C; a.ldq = a.ldk = a.ldv = 3 * C;
+      a.bias = bias_tile; a.pos = ly.pos; a.u_bias = ly.u_bias; a.v_bias = ly.v_bias;
+      a.out = f8 ? (void*)ws.ao8 : (void*)ws.ao; a.ldo = C; a.out_dtype = f8 ? DT_FP8 : DT_BF16;
+      a.out_scale = f8 ? act_scale(l, 1) : 1.f; a.amax = am(l, 1);
+      a.B = mb; a.H = H; a.scale = attn_scale;
+      a.mode = gpt ? ATTN_CAUSAL : cfg.arch == CRL_ARCH_BT4 ? ATTN_RELSHIFT : ATTN_BIAS;
+      prof_begin(1, st);
+      hipError_t he = launch_attention(a, hs, st);
+      prof_end(st);
+      HIPCHK(he);
+    }
+    const void* ao_in = f8 ? (const void*)ws.ao8 : (const void*)ws.ao;
+    const int ao_dt = f8 ? DT_FP8 : DT_BF16;
+    if (gpt) {
+      // x += proj(ao);  h = LN2(x);  x += proj2(gelu(fc(h)))
+      { GOpt o; o.res = ws.x; o.ldr = C; o.res_dt = xdt; o.a_scale = f8 ? act_scale(l, 1) : 1.f;
+        RUN(gemm(ly.proj, ao_in, C, ao_dt, ws.x, C, xdt, M, o, st)); }
+      RUN(lnorm(ws.x, C, xdt, ly.ln2_g, ly.ln2_b, f8 ? nullptr : ws.h, DT_BF16, f8 ? ws.h8 : nullptr, f8 ? act_scale(l, 2) : 1.f, C, M, C, am(l, 2), st));
+      { GOpt o; o.act = ACT_GELU; o.a_scale = f8 ? act_scale(l, 2) : 1.f; o.out_scale = f8 ? act_scale(l, 3) : 1.f; o.amax = am(l, 3);
+        RUN(gemm(ly.ff1, f8 ? (const void*)ws.h8 : (const void*)ws.h, C, ao_dt, f8 ? (void*)ws.f8 : (void*)ws.f, F, ao_dt, M, o, st)); }
+      { GOpt o; o.res = ws.x; o.ldr = C; o.res_dt = xdt; o.a_scale = f8 ? act_scale(l, 3) : 1.f;
+        RUN(gemm(ly.ff2, f8 ? (const void*)ws.f8 : (const void*)ws.f, F, ao_dt, ws.x, C, xdt, M, o, st)); }
+    } else {
+      // t = x + alpha*proj(ao);  h = LN1(t)
+      { GOpt o; o.res = ws.x; o.ldr = C; o.res_dt = DT_BF16; o.alpha = alpha; o.a_scale = f8 ? act_scale(l, 1) : 1.f;
+        RUN(gemm(ly.proj, ao_in, C, ao_dt, ws.t, C, DT_BF16, M, o, st)); }
+      RUN(lnorm(ws.t, C, DT_BF16, ly.ln1_g, ly.ln1_b, ws.h, DT_BF16, f8 ? ws.h8 : nullptr, f8 ? act_scale(l, 2) : 1.f, C, M, C, am(l, 2), st));
+      const void* h_in = f8 ? (const void*)ws.h8 : (const void*)ws.h;
+      if (cfg.arch == CRL_ARCH_BT4) {
+        // y = ff2(ff1(h)) with no activation in between; t = gelu(y) + h (new_paradigm/value.py:65-70)
+        { GOpt o; o.a_scale = f8 ? act_scale(l, 2) : 1.f; o.out_scale = f8 ? act_scale(l, 3) : 1.f; o.amax = am(l, 3);
+          RUN(gemm(ly.ff1, h_in, C, ao_dt, f8 ? (void*)ws.f8 : (void*)ws.f, F, ao_dt, M, o, st)); }
+        { GOpt o; o.act = ACT_GELU; o.res = ws.h; o.ldr = C; o.res_dt = DT_BF16; o.a_scale = f8 ? act_scale(l, 3) : 1.f;
+          RUN(gemm(ly.ff2, f8 ? (const void*)ws.f8 : (const void*)ws.f, F, ao_dt, ws.t, C, DT_BF16, M, o, st)); }
+      } else {
+        { GOpt o; o.act = ACT_MISH; o.a_scale = f8 ? act_scale(l, 2) : 1.f; o.out_scale = f8 ? act_scale(l, 3) : 1.f; o.amax = am(l, 3);
+          RUN(gemm(ly.ff1, h_in, C, ao_dt, f8 ? (void*)ws.f8 : (void*)ws.f, F, ao_dt, M, o, st)); }
+        { GOpt o; o.res = ws.h; o.ldr = C; o.res_dt = DT_BF16; o.alpha = alpha; o.a_scale = f8 ? act_scale(l, 3) : 1.f;
+          RUN(gemm(ly.ff2, f8 ? (const void*)ws.f8 : (const void*)ws.f, F, ao_dt, ws.t, C, DT_BF16, M, o, st)); }
+      }
+      // x = LN2(t); the last layer's output feeds only the heads.
+      RUN(lnorm(ws.t, C, DT_BF16, ly.ln2_g, ly.ln2_b, ws.x, last ? hd : DT_BF16, (f8 && !last) ? ws.x8 : nullptr,
+                (f8 && !last) ? act_scale(l + 1, 0) : 1.f, C, M, C, last ? nullptr : am(l + 1, 0), st));
+    }
+  }
+
+  // ---- heads
+  if (gpt) {
+    // ln_f and lm_head on token 63 only (model_bis.py:369-370).
+    const char* last_tok = reinterpret_cast<const char*>(ws.x) + (size_t)63 * C * dtype_size(xdt);
+    RUN(lnorm(last_tok, 64L * C, xdt, lnf_g, lnf_b, ws.hl, hd, nullptr, 1.f, C, mb, C, nullptr, st));
+    GOpt o;
+    RUN(gemm(lm_head, ws.hl, C, hd, policy, VOCAB_RL, DT_F32, mb, o, st));
+    return CRL_OK;
+  }
+  const int hact = cfg.arch == CRL_ARCH_BT4 ? ACT_GELU : ACT_MISH;
+  if (wdl) {
+    { GOpt o; o.act = hact; RUN(gemm(val1, ws.x, C, hd, ws.v1, 128, hd, M, o, st)); }
+    { GOpt o; o.act = hact; RUN(gemm(val2, ws.v1, 8192, hd, ws.v2, 128, hd, mb, o, st)); }
+    { GOpt o; RUN(gemm(val3, ws.v2, 128, hd, wdl, 3, DT_F32, mb, o, st)); }
+  }
+  {
+    GOpt o; o.act = hact;
+    if (cfg.arch == CRL_ARCH_BT4) { o.res = pe_head; o.ldr = C; o.res_dt = hd; o.res_rows = 64; }
+    RUN(gemm(pol_tok, ws.x, C, hd, ws.tok, C, hd, M, o, st));
+  }
+  { GOpt o; RUN(gemm(pol_qk, ws.tok, C, hd, ws.pqk, 2 * C, hd, M, o, st)); }
+  {
+    PolicyQKArgs p;
+    std::memset(&p, 0, sizeof(p));
+    const uint16_t* base = reinterpret_cast<const uint16_t*>(ws.pqk);
+    p.q = base; p.k = base + C; p.ldq = p.ldk = 2 * C; p.in_dtype = hd; p.B = mb; p.C = C;
+    p.scale = 1.0f / std::sqrt((float)C);
+    if (cfg.arch == CRL_ARCH_BT4) { p.dense = ws.dense; p.dense_dtype = hd; p.ldd = 4096; }
+    else { p.logits = policy; p.ldl = VOCAB_LEELA; p.gidx = gidx; p.gpromo = gpromo; p.wpromo = promo_w; p.white_to_move = ws.stm; p.nmoves = VOCAB_LEELA; }
+    prof_begin(4, st);
+    hipError_t he = launch_policy_qk(p, st);
+    prof_end(st);
+    HIPCHK(he);
+  }
+  if (cfg.arch == CRL_ARCH_BT4) { GOpt o; RUN(gemm(pol_head, ws.dense, 4096, hd, policy, VOCAB_RL, DT_F32, mb, o, st)); }
+#undef RUN
+  return CRL_OK;
+}
+
+int Model::calibrate(const float* planes, int B, hipStream_t st) {
+  if (!finalized) { set_error("calibrate: call crl_model_finalize first"); return CRL_ERR_STATE; }
+  HIPCHK(launch_fill_f32(amax_dev, 0.f, (long)amax_host.size(), st));
+  float* pol = nullptr;
+  HIPCHK(hipMalloc((void**)&pol, (size_t)B * vocab * sizeof(float)));
+  int rc = forward(planes, nullptr, nullptr, B, pol, nullptr, true, st);
+  hipError_t e = hipStreamSynchronize(st);
+  if (rc == CRL_OK && e == hipSuccess) e = hipMemcpy(amax_host.data(), amax_dev, sizeof(float) * amax_host.size(), hipMemcpyDeviceToHost);
+  (void)hipFree(pol);
+  if (rc) return rc;
+  HIPCHK(e);
+  return CRL_OK;
+}
+
+double Model::flops_per_position() const {
+  const double T = 64, C = cfg.d_model, F = cfg.d_ff, L = cfg.n_layer, H = cfg.n_head;
+  if (cfg.arch == CRL_ARCH_GPT64)
+    return L * (8 * T * C * C + 4 * T * C * F + 2 * T * (T + 1) * C) + 2 * T * 19 * C + 2 * C * VOCAB_RL;
+  const double heads_common = 2 * T * C * 128 + 2 * 8192.0 * 128 + 2 * 128 * 3 + 2 * T * 19 * C;
+  if (cfg.arch == CRL_ARCH_BT4)
+    return L * (8 * T * C * C + 6 * T * T * C + 4 * T * C * F) + 6 * T * C * C + 2 * T * T * C + 2 * 4096.0 * VOCAB_RL + heads_common;
+  const double sc = cfg.smolgen_compress, sh = cfg.smolgen_hidden, sg = cfg.smolgen_gen;
+  const double smol = 2 * T * C * sc + 2 * 64 * sc * sh + 2 * sh * H * sg + 2 * H * sg * 4096;
+  return L * (8 * T * C * C + 4 * T * T * C + 4 * T * C * F + smol) + 6 * T * C * C + 2 * T * T * C + 2 * 8 * 4 * C + heads_common;
+}
+
+}  // namespace crl

@@ -1,0 +1,95 @@
+// Host-side model runner (see model.hip).
+#pragma once
+#include <map>
+#include <string>
+#include <utility>
+#include <vector>
+
+#include "../../include/chessrl_amd.h"
+#include "host/chess.hpp"
+#include "kernels/common.hpp"
+
+namespace crl {
+
+void set_error(const std::string& s);
+const char* get_error();
+
+// One linear layer on the device: a 16-bit copy, an optional e4m3 copy (value*wscale)
+// and an fp32 bias.
+struct Lin {
+  void* w = nullptr;
+  void* w8 = nullptr;
+  float* b = nullptr;
+  int N = 0, K = 0, dt = DT_BF16;
+  float wscale = 1.f;
+};
+
+struct Layer {
+  Lin qkv, proj, ff1, ff2, sm_hidden, sm_gen;
+  float *ln1_g = nullptr, *ln1_b = nullptr, *ln2_g = nullptr, *ln2_b = nullptr;
+  float *sm_ln1_g = nullptr, *sm_ln1_b = nullptr, *sm_ln2_g = nullptr, *sm_ln2_b = nullptr;
+  void* pos = nullptr;
+  float *u_bias = nullptr, *v_bias = nullptr;
+};
+
+struct Workspace {
+  void *x = nullptr, *t = nullptr, *h = nullptr, *qkv = nullptr, *ao = nullptr, *f = nullptr;
+  uint8_t *x8 = nullptr, *h8 = nullptr, *ao8 = nullptr, *f8 = nullptr, *stm = nullptr;
+  void *comp = nullptr, *sh1 = nullptr, *sh2 = nullptr, *sg1 = nullptr, *sg2 = nullptr, *bias = nullptr;
+  void *hl = nullptr, *tok = nullptr, *pqk = nullptr, *v1 = nullptr, *v2 = nullptr, *dense = nullptr;
+};
+
+struct GOpt;
+
+struct Model {
+  crl_model_config cfg;
+  int vocab = 0;
+  bool finalized = false;
+  std::vector<std::pair<std::string, long>> expected;
+  std::map<std::string, std::vector<float>> host;
+
+  std::vector<void*> allocs, ws_allocs;
+  std::vector<Layer> layers;
+  float *emb_w1t = nullptr, *emb_b1 = nullptr, *emb_g = nullptr, *emb_b = nullptr, *gate_a_exp = nullptr, *gate_b = nullptr;
+  float *pe_f32 = nullptr, *lnf_g = nullptr, *lnf_b = nullptr, *promo_w = nullptr;
+  void* pe_head = nullptr;
+  Lin lm_head, pol_tok, pol_qk, pol_head, val1, val2, val3, sm_weight_gen;
+  int16_t* gidx = nullptr;
+  int8_t* gpromo = nullptr;
+  float* amax_dev = nullptr;
+  std::vector<float> amax_host;
+  Workspace ws;
+  int ws_mb = 0;
+
+  struct ProfEvent { hipEvent_t a, b; int fam; };
+  bool profiling = false;
+  std::vector<ProfEvent> prof_events;
+  size_t prof_used = 0;
+  double prof_ms[5] = {0, 0, 0, 0, 0};
+  long prof_n[5] = {0, 0, 0, 0, 0};
+
+  explicit Model(const crl_model_config& c);
+  ~Model();
+  int set_weight(const char* key, const float* data, long numel);
+  int finalize();
+  int forward(const float* planes, const uint8_t* ids, const uint8_t* flags, int B, float* policy, float* wdl, bool calibrate, hipStream_t st);
+  int calibrate(const float* planes, int B, hipStream_t st);
+  double flops_per_position() const;
+
+ private:
+  const std::vector<float>& w(const std::string& k);
+  int dev_alloc(void** p, size_t bytes, bool ws);
+  int upload(const std::vector<float>& v, int dt, float scale, void** out);
+  int make_lin(Lin& L, const std::vector<float>& W, const std::vector<float>* bias, int N, int K, int dt16, bool fp8);
+  int ensure_ws(int mb);
+  int forward_chunk(const float* planes, const uint8_t* ids, const uint8_t* flags, int mb, float* policy, float* wdl, bool calibrate, hipStream_t st);
+  int gemm(const Lin& L, const void* A, long lda, int in_dt, void* C, long ldc, int out_dt, int M, const GOpt& o, hipStream_t st);
+  int lnorm(const void* x, long ldx, int in_dt, const float* g, const float* b, void* out, int out_dt, uint8_t* out8, float scale8,
+            long ldo, int rows, int C, float* amax, hipStream_t st);
+  float act_scale(int layer, int slot) const;
+  void prof_begin(int fam, hipStream_t st);
+  void prof_end(hipStream_t st);
+  void prof_collect(hipStream_t st);
+};
+
+}  // namespace crl

@@ -1,0 +1,183 @@
+/* chessrl_amd — C ABI of the MI355X (gfx950) policy/value forward path.
+ *
+ * The reference (maxlegrec1/ChessRL) has no FFI layer: its boundary for this path is
+ * the Python nn.Module surface plus the state-dict. Every entry point below therefore
+ * cites the reference Python interface it stands in for; chessrl_amd/models.py is the
+ * ctypes binding that rebuilds that surface on top of this header.
+ *
+ * Conventions: every function returns 0 on success and a negative code on failure
+ * (crl_last_error() gives the message for the calling thread). No exception crosses
+ * the boundary. "device" pointers are HIP device pointers owned by the caller (for
+ * example torch tensors' data_ptr()); "stream" is a hipStream_t passed as void*
+ * (NULL = the default stream). The library never synchronises the stream unless the
+ * function says so. Host-only functions touch no GPU state and work without a GPU.
+ */
+#ifndef CHESSRL_AMD_H
+#define CHESSRL_AMD_H
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define CRL_OK 0
+#define CRL_ERR_ARG (-1)      /* bad argument / shape / alignment */
+#define CRL_ERR_HIP (-2)      /* a HIP call failed */
+#define CRL_ERR_STATE (-3)    /* call order (e.g. forward before finalize, missing weight) */
+#define CRL_ERR_FEN (-4)      /* malformed FEN */
+
+#define CRL_VOCAB_RL 1929     /* utils/vocab.py:9-227   policy_index */
+#define CRL_VOCAB_LEELA 1858  /* utils/vocab.py:229-438 policy_leela */
+#define CRL_NUM_PLANES 19     /* utils/fen_encoder.py:7 */
+
+/* element types */
+#define CRL_F32 0
+#define CRL_BF16 1
+#define CRL_F16 2
+#define CRL_FP8 3             /* OCP e4m3fn */
+/* activations */
+#define CRL_ACT_NONE 0
+#define CRL_ACT_GELU 1        /* erf form, nn.GELU() */
+#define CRL_ACT_MISH 2
+#define CRL_ACT_SWISH 3
+/* attention modes */
+#define CRL_ATTN_PLAIN 0
+#define CRL_ATTN_CAUSAL 1     /* model_bis.py:71 */
+#define CRL_ATTN_BIAS 2       /* generated per-head 64x64 bias (BT4-class) */
+#define CRL_ATTN_RELSHIFT 3   /* new_paradigm/attn.py:507-533 */
+/* model architectures */
+#define CRL_ARCH_GPT64 0      /* model_bis.GPT, 64-token forward (model_bis.py:358-370) */
+#define CRL_ARCH_BT4 1        /* new_paradigm/value.py BT4 */
+#define CRL_ARCH_BT4CLASS 2   /* BT4-class encoder of the benchmark configuration */
+
+const char* crl_last_error(void);
+const char* crl_version(void);
+
+/* ------------------------------------------------------------------ host: vocabulary */
+/* utils/vocab.py:9-227 / :229-438 — i-th move string (static storage), NULL if out of range. */
+const char* crl_policy_index(int i);
+const char* crl_policy_leela(int i);
+/* policy_index.index(uci) with the reference's trailing-'n' strip (model_bis.py:376-380); -1 if absent. */
+int crl_move_to_index(const char* uci);
+/* Leela/compare_policy.py:470-491 — mapping_white / mapping_black, int32[1858] each. */
+int crl_leela_to_rl_maps(int32_t* white_out, int32_t* black_out);
+
+/* ------------------------------------------------------------------ host: boards */
+/* utils/fen_encoder.py:5-38 fen_to_tensor: float32[64*19] in token order t=(7-rank)*8+file. */
+int crl_fen_to_planes(const char* fen, float* out_planes);
+/* utils/parse.py:71-75 encode_fens: n FENs -> float32[n,64,19]; threads<=0 picks a default. */
+int crl_encode_fens(const char* const* fens, int n, float* out_planes, int threads);
+/* Compact form of the same information: uint8[n,64] piece codes (0 empty, 1..6 PNBRQK,
+ * 7..12 pnbrqk) and uint8[n,4] {white_to_move, castling bits WK|WQ<<1|BK<<2|BQ<<3,
+ * en-passant token or 255, min(halfmove,100)}. */
+int crl_encode_fens_compact(const char* const* fens, int n, uint8_t* out_ids, uint8_t* out_flags, int threads);
+/* model_bis.py:373-380 (same code grpo_refactored.py:374-384, new_paradigm/value.py:222-231):
+ * uint8[n,1929] legal-move masks; out_counts (optional) gets len(list(board.legal_moves)). */
+int crl_legal_masks(const char* const* fens, int n, uint8_t* out_masks, int32_t* out_counts, int threads);
+/* Same for the 1858-entry side-to-move frame (black rows rank-mirrored, Leela/compare_policy.py:437-463). */
+int crl_legal_masks_leela(const char* const* fens, int n, uint8_t* out_masks, int32_t* out_counts, int threads);
+/* Legal moves of one position as UCI strings, 6 bytes each (NUL padded), in generation
+ * order; returns the count (<= max_moves) or a negative code. new_paradigm/value.py:331. */
+int crl_legal_moves(const char* fen, char* out_uci6, int max_moves);
+/* board.push(move); board.fen() for every legal move (new_paradigm/value.py:336-340):
+ * writes child FENs (96 bytes each, NUL terminated) and the moves (6 bytes each). */
+int crl_child_fens(const char* fen, char* out_fens96, char* out_uci6, int max_moves);
+uint64_t crl_perft(const char* fen, int depth);
+/* Seeded uniform-random legal playouts from the start position (splitmix64): position k
+ * gets U{0..max_plies} plies; when late_fraction>0 that share of positions is instead
+ * played on until at most late_max_pieces pieces remain. Outputs (each optional):
+ * float32[n,64,19] planes, uint8[n,1929] masks, uint8[n,1858] masks, FENs (96 bytes each). */
+int crl_random_positions(uint64_t seed, int n, int max_plies, double late_fraction, int late_max_pieces,
+                         float* out_planes, uint8_t* out_masks_rl, uint8_t* out_masks_leela, char* out_fens96);
+
+/* ------------------------------------------------------------------ device: operators */
+/* nn.Linear / te.Linear (model_bis.py:42-44,89-91,139; model_fp8.py:43-45,90-92,140;
+ * new_paradigm/value.py:39-40,129-152): C = res + alpha*act(descale*(A·W^T) + bias).
+ * A [M,K] (lda), W [N,K] (ldw) of in_dtype (bf16/f16/fp8); C [M,N] (ldc) of out_dtype;
+ * bias fp32[N] or NULL; res [M,N] of res_dtype (f32/bf16) or NULL; for an fp8 output the
+ * value is multiplied by out_scale before conversion; amax (device float, optional)
+ * accumulates max|value|. tile: 0 = automatic. */
+int crl_gemm(const void* A, int64_t lda, const void* W, int64_t ldw, void* C, int64_t ldc,
+             int M, int N, int K, int in_dtype, int out_dtype,
+             const float* bias, int act, float descale, float alpha,
+             const void* res, int64_t ldr, int res_dtype, float out_scale, float* amax,
+             int tile, void* stream);
+/* F.layer_norm(x,(C,),gamma,beta,eps) (model_bis.py:34). out (out_dtype) and/or out_fp8
+ * (value*fp8_scale, e4m3) may be given. */
+int crl_layernorm(const void* x, int64_t ldx, int in_dtype, const float* gamma, const float* beta,
+                  void* out, int out_dtype, uint8_t* out_fp8, float fp8_scale, int64_t ldo,
+                  int rows, int C, float eps, float* amax, void* stream);
+/* Attention over 64 tokens per position, bf16 q/k/v with head h at columns [h*head_dim, ...).
+ * mode CAUSAL: model_bis.py:71; RELSHIFT: new_paradigm/attn.py:507-521 with pos = pos_proj(PE)
+ * (bf16 [64,H*head_dim]) and u_bias/v_bias fp32[H*head_dim]; BIAS: bias bf16 [B,H,64,64] in the
+ * order crl_attn_bias_slot defines. out is bf16 or fp8 (value*out_scale) [B*64, ldo]. */
+int crl_attention(const void* q, int64_t ldq, const void* k, int64_t ldk, const void* v, int64_t ldv,
+                  void* out, int64_t ldo, int out_dtype, float out_scale,
+                  int B, int H, int head_dim, int mode, float scale,
+                  const void* bias, const void* pos, const float* u_bias, const float* v_bias,
+                  float* amax, void* stream);
+int crl_attn_bias_slot(int query, int key);
+/* logits + (1-mask)*(-999); softmax(./T); T==0 -> one-hot arg-max (model_bis.py:382-392).
+ * logits f32 [B,V] (ldl), mask uint8 [B,V] or NULL, probs f32 [B,V] or NULL, argmax int32[B] or NULL. */
+int crl_masked_softmax(const float* logits, int64_t ldl, const uint8_t* mask, int64_t ldm,
+                       float* probs, int64_t ldp, int32_t* argmax, int B, int V, float temperature, void* stream);
+/* Leela/compare_policy.py:493-523 map_leela_to_rl on device: src f32 [B,1858] -> dst f32 [B,1929];
+ * white_to_move uint8[B] selects identity or the rank-mirrored slot. */
+int crl_leela_to_rl(const float* src, int64_t lds, float* dst, int64_t ldd, const uint8_t* white_to_move, int B, void* stream);
+
+/* ------------------------------------------------------------------ device: models */
+typedef struct crl_model crl_model;
+
+typedef struct crl_model_config {
+  int32_t arch;           /* CRL_ARCH_* */
+  int32_t n_layer;
+  int32_t d_model;
+  int32_t n_head;
+  int32_t d_ff;
+  int32_t fp8;            /* 1: trunk linears (qkv, out-proj, ffn) run in e4m3 with static per-tensor scales */
+  int32_t micro_batch;    /* positions per pass through the trunk; 0 = default */
+  int32_t stream_f32;     /* GPT64 only: keep the residual stream in fp32 (default 1) */
+  int32_t head_dtype;     /* CRL_BF16 or CRL_F16: element type of the policy/value head GEMM inputs */
+  int32_t smolgen_compress, smolgen_hidden, smolgen_gen;  /* BT4-class; 0 = 32/256/256 */
+  float eps;              /* LayerNorm epsilon; 0 = 1e-5 */
+  int32_t reserved[4];
+} crl_model_config;
+
+/* GPT(config) / BT4(...) constructors (model_bis.py:127-157, new_paradigm/value.py:122-152). */
+int crl_model_create(const crl_model_config* cfg, crl_model** out);
+void crl_model_destroy(crl_model* m);
+/* load_state_dict(): hand over one tensor by its state-dict key as host fp32 (the library
+ * keeps its own converted copy). Keys are listed by crl_model_expected_key(). */
+int crl_model_set_weight(crl_model* m, const char* key, const float* data, int64_t numel);
+/* i-th expected state-dict key and its element count; NULL when i is out of range. */
+const char* crl_model_expected_key(crl_model* m, int i, int64_t* numel);
+/* Convert/pack weights to device (bf16, fp8 and re-ordered copies). Needs a GPU. */
+int crl_model_finalize(crl_model* m);
+/* fp8 only: run the bf16 path on calibration positions and derive the static activation
+ * scales 448/amax (pretrain_fp8.py:75-79 uses DelayedScaling amax history; here the history
+ * is one calibration batch). Synchronises the stream. */
+int crl_model_calibrate(crl_model* m, const float* planes, int B, void* stream);
+/* Read / overwrite the activation amax table (float[n_layer*4]). */
+int crl_model_get_amax(crl_model* m, float* out, int n);
+int crl_model_set_amax(crl_model* m, const float* in, int n);
+/* The forward pass. planes: device f32 [B,64,19] (GPT.forward batch[0] / BT4.forward inp[0]).
+ * policy_logits: device f32 [B, vocab] with vocab = 1929 (GPT64: logits of token 63,
+ * model_bis.py:370; BT4: value.py:187) or 1858 (BT4-class). wdl_logits: device f32 [B,3]
+ * in the order [black win, draw, white win] (value.py:248), NULL for GPT64 or to skip. */
+int crl_model_forward(crl_model* m, const float* planes, int B, float* policy_logits, float* wdl_logits, void* stream);
+/* Same from the compact board form (device uint8[B,64] ids + uint8[B,4] flags). */
+int crl_model_forward_compact(crl_model* m, const uint8_t* ids, const uint8_t* flags, int B,
+                              float* policy_logits, float* wdl_logits, void* stream);
+int crl_model_vocab(const crl_model* m);
+/* 2*MAC count of one position through this model (for roofline accounting). */
+double crl_model_flops_per_position(const crl_model* m);
+/* Per-call switch: wrap every kernel family in HIP events on the call's stream and return
+ * the accumulated milliseconds per family (gemm, attention, layernorm, embed, heads). */
+int crl_model_set_profiling(crl_model* m, int on);
+int crl_model_get_profile(crl_model* m, double* ms5, int64_t* launches5);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* CHESSRL_AMD_H */
