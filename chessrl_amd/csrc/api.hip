@@ -336,12 +336,16 @@ double crl_model_flops_per_position(const crl_model* m) { return m ? m->impl.flo
 int crl_model_set_profiling(crl_model* m, int on) {
   if (!m) return arg_fail("null model");
   m->impl.profiling = on != 0;
-  for (int i = 0; i < 5; ++i) { m->impl.prof_ms[i] = 0; m->impl.prof_n[i] = 0; }
+  for (int i = 0; i < 6; ++i) { m->impl.prof_ms[i] = 0; m->impl.prof_n[i] = 0; m->impl.prof_flops[i] = 0; }
   return CRL_OK;
 }
-int crl_model_get_profile(crl_model* m, double* ms5, int64_t* launches5) {
-  if (!m || !ms5 || !launches5) return arg_fail("crl_model_get_profile: bad arguments");
-  for (int i = 0; i < 5; ++i) { ms5[i] = m->impl.prof_ms[i]; launches5[i] = m->impl.prof_n[i]; }
+int crl_model_get_profile(crl_model* m, double* ms6, int64_t* launches6, double* flops6) {
+  if (!m || !ms6 || !launches6) return arg_fail("crl_model_get_profile: bad arguments");
+  for (int i = 0; i < 6; ++i) {
+    ms6[i] = m->impl.prof_ms[i];
+    launches6[i] = m->impl.prof_n[i];
+    if (flops6) flops6[i] = m->impl.prof_flops[i];
+  }
   return CRL_OK;
 }
 

@@ -203,7 +203,7 @@ hipError_t launch_attention(const AttnArgs& a, int head_dim, hipStream_t st);
 hipError_t launch_policy_qk(const PolicyQKArgs& a, hipStream_t st);
 hipError_t launch_masked_softmax(const SoftmaxArgs& a, hipStream_t st);
 hipError_t launch_leela_to_rl(const ScatterArgs& a, hipStream_t st);
-hipError_t launch_extract_stm(const float* planes, uint8_t* white_to_move, int B, hipStream_t st);
+hipError_t launch_extract_stm(const float* planes, const uint8_t* flags, uint8_t* white_to_move, int B, hipStream_t st);
 hipError_t launch_fill_f32(float* p, float v, long n, hipStream_t st);
 hipError_t launch_convert(const float* src, void* dst, long n, int dt, float scale, hipStream_t st);
 // Slot of (query i, key j) inside a 4096-element attention bias tile.

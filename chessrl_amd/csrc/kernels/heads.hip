@@ -204,13 +204,15 @@ hipError_t launch_leela_to_rl(const ScatterArgs& a, hipStream_t st) {
 
 
 // Side to move of each position: plane 12 of its first token (utils/fen_encoder.py:22).
-__global__ void extract_stm_kernel(const float* planes, uint8_t* out, int B) {
+// With the compact board form it is byte 0 of the position's four flag bytes.
+__global__ void extract_stm_kernel(const float* planes, const uint8_t* flags, uint8_t* out, int B) {
   const int b = blockIdx.x * blockDim.x + threadIdx.x;
-  if (b < B) out[b] = planes[(long)b * 64 * 19 + 12] > 0.5f ? 1 : 0;
+  if (b >= B) return;
+  out[b] = planes ? (planes[(long)b * 64 * 19 + 12] > 0.5f ? 1 : 0) : (flags[(long)b * 4] ? 1 : 0);
 }
-hipError_t launch_extract_stm(const float* planes, uint8_t* white_to_move, int B, hipStream_t st) {
+hipError_t launch_extract_stm(const float* planes, const uint8_t* flags, uint8_t* white_to_move, int B, hipStream_t st) {
   if (B <= 0) return hipSuccess;
-  hipLaunchKernelGGL(extract_stm_kernel, dim3((B + 255) / 256), dim3(256), 0, st, planes, white_to_move, B);
+  hipLaunchKernelGGL(extract_stm_kernel, dim3((B + 255) / 256), dim3(256), 0, st, planes, flags, white_to_move, B);
   return hipGetLastError();
 }
 

@@ -396,7 +396,9 @@ int Model::gemm(const Lin& L, const void* A, long lda, int in_dt, void* C, long 
   g.amax = o.amax; g.M = M; g.N = L.N; g.K = L.K; g.act = o.act;
   g.descale = in_dt == DT_FP8 ? 1.f / (o.a_scale * L.wscale) : 1.f;
   g.alpha = o.alpha; g.out_scale = o.out_scale;
-  prof_begin(0, st);
+  const int fam = in_dt == DT_FP8 ? 0 : 5;
+  if (profiling) prof_flops[fam] += 2.0 * M * (double)L.N * L.K;
+  prof_begin(fam, st);
   hipError_t e = launch_gemm(g, in_dt == DT_FP8 ? DT_FP8 : L.dt, out_dt, 0, st);
   prof_end(st);
   HIPCHK(e);
@@ -467,8 +469,7 @@ int Model::forward_chunk(const float* planes, const uint8_t* ids, const uint8_t*
     HIPCHK(he);
   }
   if (cfg.arch == CRL_ARCH_BT4CLASS) {
-    if (planes) HIPCHK(launch_extract_stm(planes, ws.stm, mb, st));
-    else HIPCHK(hipMemcpy2DAsync(ws.stm, 1, flags, 4, 1, mb, hipMemcpyDeviceToDevice, st));
+    HIPCHK(launch_extract_stm(planes, flags, ws.stm, mb, st));
   }
 
   const float attn_scale = cfg.arch == CRL_ARCH_BT4 ? 1.0f / std::sqrt((float)C) : 1.0f / std::sqrt((float)hs);

@@ -65,8 +65,9 @@ struct Model {
   bool profiling = false;
   std::vector<ProfEvent> prof_events;
   size_t prof_used = 0;
-  double prof_ms[5] = {0, 0, 0, 0, 0};
-  long prof_n[5] = {0, 0, 0, 0, 0};
+  double prof_ms[6] = {0, 0, 0, 0, 0, 0};
+  double prof_flops[6] = {0, 0, 0, 0, 0, 0};
+  long prof_n[6] = {0, 0, 0, 0, 0, 0};
 
   explicit Model(const crl_model_config& c);
   ~Model();

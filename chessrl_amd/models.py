@@ -1,0 +1,478 @@
+"""Python surface of the reference models on top of the HIP library.
+
+GPTConfig / GPT keep the constructor, state-dict keys and inference methods of
+model_bis.py:115-398 for the 64-token ("no thinking") forward; BT4 keeps those of
+new_paradigm/value.py:121-400; BT4Class is the benchmark's BT4-class encoder. All
+compute runs in libchessrl_amd.so; torch only owns device memory and streams.
+"""
+import ctypes as C
+import math
+from collections import OrderedDict
+from dataclasses import dataclass
+
+import numpy as np
+import torch
+
+from . import _lib, board
+from ._lib import check, lib
+from .vocab import policy_index, policy_leela
+
+VOCAB_RL, VOCAB_LEELA = _lib.VOCAB_RL, _lib.VOCAB_LEELA
+
+
+def _stream_ptr():
+    return C.c_void_p(torch.cuda.current_stream().cuda_stream)
+
+
+def _ptr(t):
+    return C.c_void_p(t.data_ptr()) if t is not None else None
+
+
+def _lin_shapes(d, name, out, inp, bias=True):
+    d[name + ".weight"] = (out, inp)
+    if bias:
+        d[name + ".bias"] = (out,)
+
+
+def _ln_shapes(d, name, n):
+    d[name + ".weight"] = (n,)
+    d[name + ".bias"] = (n,)
+
+
+def gpt_shapes(n_layer, n_embd, block_size=256, vocab_size=VOCAB_RL):
+    """State-dict keys and shapes of model_bis.GPT (model_bis.py:132-146)."""
+    C_ = n_embd
+    d = OrderedDict()
+    _lin_shapes(d, "FenEncoder.linear1", C_, 19)
+    _ln_shapes(d, "FenEncoder.layernorm1", C_)
+    d["FenEncoder.ma_gating.a"] = (64, C_)
+    d["FenEncoder.ma_gating.b"] = (64, C_)
+    d["transformer.wte.weight"] = (vocab_size, C_)
+    for i in range(n_layer):
+        p = "transformer.h.%d." % i
+        _ln_shapes(d, p + "ln_1", C_)
+        _lin_shapes(d, p + "attn.c_attn", 3 * C_, C_)
+        _lin_shapes(d, p + "attn.c_proj", C_, C_)
+        _ln_shapes(d, p + "ln_2", C_)
+        _lin_shapes(d, p + "mlp.c_fc", 4 * C_, C_)
+        _lin_shapes(d, p + "mlp.c_proj", C_, 4 * C_)
+    _ln_shapes(d, "transformer.ln_f", C_)
+    d["lm_head.weight"] = (vocab_size, C_)
+    d["pe"] = (block_size, C_)
+    return d
+
+
+def bt4_shapes(num_layers, d_model, d_ff, num_heads, bt4class=False, compress=32, hidden=256, gen=256):
+    """State-dict keys and shapes of new_paradigm/value.py BT4 (value.py:129-152,423-425);
+    with bt4class=True the BT4-class extension (smolgen, promotion offsets, no dense policy map)."""
+    C_, F_, H = d_model, d_ff, num_heads
+    d = OrderedDict()
+    for i in range(num_layers):
+        p = "layers.%d." % i
+        for n in ("query_proj", "key_proj", "value_proj"):
+            _lin_shapes(d, p + "attention." + n, C_, C_)
+        if not bt4class:
+            d[p + "attention.pos_proj.weight"] = (C_, C_)
+            d[p + "attention.u_bias"] = (H, C_ // H)
+            d[p + "attention.v_bias"] = (H, C_ // H)
+        _lin_shapes(d, p + "attention.out_proj", C_, C_)
+        if bt4class:
+            d[p + "smolgen.compress.weight"] = (compress, C_)
+            _lin_shapes(d, p + "smolgen.hidden", hidden, 64 * compress)
+            _ln_shapes(d, p + "smolgen.hidden_ln", hidden)
+            _lin_shapes(d, p + "smolgen.gen_from", H * gen, hidden)
+            _ln_shapes(d, p + "smolgen.gen_from_ln", H * gen)
+        _ln_shapes(d, p + "norm1", C_)
+        _ln_shapes(d, p + "norm2", C_)
+        _lin_shapes(d, p + "ff1", F_, C_)
+        _lin_shapes(d, p + "ff2", C_, F_)
+    if bt4class:
+        d["smol_weight_gen.weight"] = (4096, gen)
+    _lin_shapes(d, "linear1", C_, 19)
+    _ln_shapes(d, "layernorm1", C_)
+    _lin_shapes(d, "policy_tokens_lin", C_, C_)
+    _lin_shapes(d, "queries_pol", C_, C_)
+    _lin_shapes(d, "keys_pol", C_, C_)
+    d["ma_gating.a"] = (64, C_)
+    d["ma_gating.b"] = (64, C_)
+    if bt4class:
+        d["promotion_offsets.weight"] = (4, C_)
+    else:
+        d["policy_head.weight"] = (VOCAB_RL, 4096)
+    _lin_shapes(d, "value_head.dense1", 128, C_)
+    _lin_shapes(d, "value_head.dense2", 128, 128 * 64)
+    _lin_shapes(d, "value_head.dense3", 3, 128)
+    return d
+
+
+def _default_init(shapes, seed, n_layer=None):
+    """normal(0, 0.02) weights, zero biases, LayerNorm at identity, gating a=0/b=1
+    (model_bis.py:163-169); c_proj weights use std 0.02/sqrt(2L) (model_bis.py:153-155)."""
+    g = torch.Generator().manual_seed(seed)
+    sd = OrderedDict()
+    for k, shp in shapes.items():
+        if k == "pe":
+            continue
+        if k.endswith("ma_gating.a"):
+            t = torch.zeros(shp)
+        elif k.endswith("ma_gating.b"):
+            t = torch.ones(shp)
+        elif k.endswith("u_bias") or k.endswith("v_bias"):
+            bound = math.sqrt(6.0 / (shp[0] + shp[1]))
+            t = torch.empty(shp).uniform_(-bound, bound, generator=g)
+        elif len(shp) == 2:
+            std = 0.02 / math.sqrt(2 * n_layer) if (k.endswith("c_proj.weight") and n_layer) else 0.02
+            t = torch.empty(shp).normal_(0.0, std, generator=g)
+        elif k.endswith(".bias"):
+            t = torch.zeros(shp)
+        else:
+            t = torch.ones(shp)
+        sd[k] = t
+    return sd
+
+
+class _Engine:
+    """Owns one crl_model handle."""
+
+    def __init__(self, arch, n_layer, d_model, n_head, d_ff, fp8=False, micro_batch=0, stream_f32=True,
+                 head_dtype="bf16", compress=32, hidden=256, gen=256):
+        cfg = _lib.ModelConfig()
+        cfg.arch, cfg.n_layer, cfg.d_model, cfg.n_head, cfg.d_ff = arch, n_layer, d_model, n_head, d_ff
+        cfg.fp8 = 1 if fp8 else 0
+        cfg.micro_batch = micro_batch
+        cfg.stream_f32 = 1 if stream_f32 else 0
+        cfg.head_dtype = _lib.F16 if head_dtype in ("f16", "fp16") else _lib.BF16
+        cfg.smolgen_compress, cfg.smolgen_hidden, cfg.smolgen_gen = compress, hidden, gen
+        self.cfg = cfg
+        self.n_layer = n_layer
+        self.fp8 = bool(fp8)
+        h = C.c_void_p()
+        check(lib().crl_model_create(C.byref(cfg), C.byref(h)), "crl_model_create")
+        self.handle = h
+        self.vocab = lib().crl_model_vocab(h)
+        self.ready = False
+
+    def __del__(self):
+        h = getattr(self, "handle", None)
+        if h:
+            try:
+                lib().crl_model_destroy(h)
+            except Exception:
+                pass
+            self.handle = None
+
+    def expected_keys(self):
+        out, i, n = [], 0, C.c_int64()
+        while True:
+            k = lib().crl_model_expected_key(self.handle, i, C.byref(n))
+            if k is None:
+                return out
+            out.append((k.decode(), n.value))
+            i += 1
+
+    def load(self, sd):
+        for k, _ in self.expected_keys():
+            if k not in sd:
+                raise KeyError("state dict lacks %r" % k)
+            t = sd[k].detach().to("cpu", torch.float32).contiguous()
+            check(lib().crl_model_set_weight(self.handle, k.encode(), C.c_void_p(t.data_ptr()), t.numel()), "crl_model_set_weight(%s)" % k)
+        self.ready = False
+
+    def finalize(self):
+        if not torch.cuda.is_available():
+            raise _lib.CrlError("no GPU: the forward pass has no CPU fallback")
+        check(lib().crl_model_finalize(self.handle), "crl_model_finalize")
+        self.ready = True
+
+    def calibrate(self, planes):
+        if not self.ready:
+            self.finalize()
+        planes = _as_planes(planes)
+        check(lib().crl_model_calibrate(self.handle, _ptr(planes), planes.shape[0], _stream_ptr()), "crl_model_calibrate")
+
+    def get_amax(self):
+        a = np.zeros(self.n_layer * 4, np.float32)
+        check(lib().crl_model_get_amax(self.handle, a.ctypes.data, a.size), "crl_model_get_amax")
+        return a.reshape(self.n_layer, 4)
+
+    def set_amax(self, a):
+        a = np.ascontiguousarray(np.asarray(a, np.float32).reshape(-1))
+        check(lib().crl_model_set_amax(self.handle, a.ctypes.data, a.size), "crl_model_set_amax")
+
+    def forward(self, planes, want_wdl=True, out_policy=None, out_wdl=None):
+        """planes: cuda float32 [B,64,19] (any shape with 64*19 trailing elements per position)."""
+        if not self.ready:
+            self.finalize()
+        planes = _as_planes(planes)
+        B = planes.shape[0]
+        pol = out_policy if out_policy is not None else torch.empty((B, self.vocab), dtype=torch.float32, device=planes.device)
+        wdl = None
+        if want_wdl and self.cfg.arch != _lib.ARCH_GPT64:
+            wdl = out_wdl if out_wdl is not None else torch.empty((B, 3), dtype=torch.float32, device=planes.device)
+        check(lib().crl_model_forward(self.handle, _ptr(planes), B, _ptr(pol), _ptr(wdl), _stream_ptr()), "crl_model_forward")
+        return pol, wdl
+
+    def forward_compact(self, ids, flags, want_wdl=True):
+        if not self.ready:
+            self.finalize()
+        B = ids.shape[0]
+        pol = torch.empty((B, self.vocab), dtype=torch.float32, device=ids.device)
+        wdl = torch.empty((B, 3), dtype=torch.float32, device=ids.device) if (want_wdl and self.cfg.arch != _lib.ARCH_GPT64) else None
+        check(lib().crl_model_forward_compact(self.handle, _ptr(ids.contiguous()), _ptr(flags.contiguous()), B, _ptr(pol), _ptr(wdl), _stream_ptr()),
+              "crl_model_forward_compact")
+        return pol, wdl
+
+    def flops_per_position(self):
+        return lib().crl_model_flops_per_position(self.handle)
+
+    def set_profiling(self, on):
+        check(lib().crl_model_set_profiling(self.handle, 1 if on else 0), "crl_model_set_profiling")
+
+    def get_profile(self):
+        ms = (C.c_double * 6)()
+        n = (C.c_int64 * 6)()
+        fl = (C.c_double * 6)()
+        check(lib().crl_model_get_profile(self.handle, ms, n, fl), "crl_model_get_profile")
+        names = ("gemm_fp8", "attention", "layernorm", "embed", "policy_qk", "gemm_16bit")
+        return {k: {"ms": ms[i], "launches": n[i], "flops": fl[i]} for i, k in enumerate(names)}
+
+
+def _as_planes(planes):
+    if not planes.is_cuda:
+        raise _lib.CrlError("planes must live on the GPU (the forward pass has no CPU path)")
+    if planes.dtype != torch.float32:
+        planes = planes.float()
+    return planes.reshape(-1, 64, 19).contiguous()
+
+
+def masked_softmax(logits, mask=None, temperature=1.0, want_probs=True):
+    """softmax((logits + (1-mask)*-999)/T) and the arg-max, on the GPU (model_bis.py:382-392)."""
+    logits = logits.contiguous()
+    B, V = logits.shape
+    probs = torch.empty_like(logits) if want_probs else None
+    am = torch.empty((B,), dtype=torch.int32, device=logits.device)
+    if mask is not None:
+        mask = mask.to(torch.uint8).contiguous()
+    check(lib().crl_masked_softmax(_ptr(logits), V, _ptr(mask), V, _ptr(probs), V, _ptr(am), B, V, float(temperature), _stream_ptr()),
+          "crl_masked_softmax")
+    return probs, am
+
+
+def leela_to_rl(logits1858, white_to_move):
+    """[B,1858] side-to-move-frame values -> [B,1929] policy_index slots (Leela/compare_policy.py:493-523)."""
+    src = logits1858.contiguous()
+    B = src.shape[0]
+    dst = torch.empty((B, VOCAB_RL), dtype=torch.float32, device=src.device)
+    wtm = white_to_move.to(torch.uint8).contiguous()
+    check(lib().crl_leela_to_rl(_ptr(src), VOCAB_LEELA, _ptr(dst), VOCAB_RL, _ptr(wtm), B, _stream_ptr()), "crl_leela_to_rl")
+    return dst
+
+
+class _ModelBase:
+    """Shared state-dict plumbing and the batched leaf-evaluation entry."""
+
+    is_thinking_model = False
+
+    def state_dict(self):
+        return OrderedDict((k, v.clone()) for k, v in self._sd.items())
+
+    def load_state_dict(self, sd, strict=True):
+        missing = [k for k in self._shapes if k not in sd and k != "transformer.wte.weight"]
+        unexpected = [k for k in sd if k not in self._shapes]
+        if strict and (missing or unexpected):
+            raise RuntimeError("load_state_dict: missing %s, unexpected %s" % (missing, unexpected))
+        for k, shp in self._shapes.items():
+            if k in sd:
+                t = sd[k].detach().to("cpu", torch.float32)
+                if tuple(t.shape) != tuple(shp) and not (k == "pe" and t.shape[0] >= 64 and t.shape[1] == shp[1]):
+                    raise RuntimeError("load_state_dict: %s has shape %s, expected %s" % (k, tuple(t.shape), tuple(shp)))
+                self._sd[k] = t.clone()
+        if "lm_head.weight" in self._sd:
+            self._sd["transformer.wte.weight"] = self._sd["lm_head.weight"]
+        self._engine.load(self._sd)
+        return self
+
+    def to(self, *a, **k):
+        return self
+
+    def eval(self):
+        return self
+
+    def parameters(self):
+        return [v for k, v in self._sd.items() if k != "pe"]
+
+    def calibrate(self, planes):
+        """fp8: derive the static activation scales from a calibration batch."""
+        self._engine.calibrate(planes)
+
+    @torch.no_grad()
+    def evaluate(self, planes, legal_mask=None, T=1.0, want_probs=False):
+        """Batched leaf evaluation: planes [B,8,8,19] (cuda) -> (policy_logits [B,V], wdl_logits [B,3] or None).
+        With want_probs the legal-masked softmax(./T) is returned in place of the raw logits."""
+        pol, wdl = self._engine.forward(planes)
+        if want_probs:
+            pol, _ = masked_softmax(pol, legal_mask, T)
+        return pol, wdl
+
+    def _sample(self, logits_row, mask_row, T):
+        probs, am = masked_softmax(logits_row, mask_row, T, want_probs=True)
+        if T == 0:
+            return int(am.item()), probs
+        return int(torch.multinomial(probs, num_samples=1).item()), probs
+
+
+@dataclass
+class GPTConfig:
+    block_size: int = 1024
+    vocab_size: int = 50304
+    n_layer: int = 6
+    n_head: int = 12
+    n_embd: int = 768
+    dropout: float = 0.0
+    bias: bool = True
+
+
+class GPT(_ModelBase):
+    """model_bis.GPT for the 64 board tokens (model_bis.py:125-199, 358-398)."""
+
+    def __init__(self, config, fp8=False, micro_batch=0, stream_f32=True, head_dtype="bf16", seed=0):
+        if config.vocab_size != VOCAB_RL:
+            raise ValueError("vocab_size must be %d (utils/vocab.py)" % VOCAB_RL)
+        if not config.bias:
+            raise ValueError("bias=False is not supported")
+        self.config = config
+        self._shapes = gpt_shapes(config.n_layer, config.n_embd, config.block_size, config.vocab_size)
+        self._sd = _default_init(self._shapes, seed, config.n_layer)
+        self._sd["transformer.wte.weight"] = self._sd["lm_head.weight"]
+        from_pe = torch.zeros(config.block_size, config.n_embd)
+        pos = torch.arange(config.block_size).unsqueeze(1)
+        div = torch.exp(torch.arange(0, config.n_embd, 2).float() * (-math.log(10000.0) / config.n_embd))
+        from_pe[:, 0::2] = torch.sin(pos * div)
+        from_pe[:, 1::2] = torch.cos(pos * div)
+        self._sd["pe"] = from_pe
+        self._engine = _Engine(_lib.ARCH_GPT64, config.n_layer, config.n_embd, config.n_head, 4 * config.n_embd,
+                               fp8=fp8, micro_batch=micro_batch, stream_f32=stream_f32, head_dtype=head_dtype)
+        self._engine.load(self._sd)
+
+    def get_num_params(self, non_embedding=True):
+        return sum(v.numel() for k, v in self._sd.items() if k not in ("pe", "transformer.wte.weight"))
+
+    @torch.no_grad()
+    def forward(self, batch, compute_loss=False):
+        """batch = (planes [B,8,8,19], idx [B,t]); only t == 0 (the 64-token forward) runs here.
+        Returns (logits [B,1,1929], None, targets) like model_bis.py:196-199."""
+        planes, idx = batch[0], batch[1]
+        if compute_loss or (idx is not None and idx.numel() > 0):
+            raise NotImplementedError("only the 64-token forward (no move tokens, no loss) is implemented")
+        pol, _ = self._engine.forward(planes)
+        targets = torch.full((pol.shape[0], 64), 1928, device=pol.device, dtype=torch.int64)
+        return pol.unsqueeze(1), None, targets
+
+    __call__ = forward
+
+    @torch.no_grad()
+    def get_move_from_fen_no_thinking(self, fen, T=1, device="cuda", force_legal=True, return_probs=False):
+        planes = board.encode_fens([fen]).to(device)
+        logits, _ = self._engine.forward(planes)
+        mask = torch.from_numpy(board.legal_move_mask(fen)).to(device).unsqueeze(0) if force_legal else None
+        idx, probs = self._sample(logits, mask, T)
+        move = policy_index[idx]
+        return (move, probs[0]) if return_probs else move
+
+
+class BT4(_ModelBase):
+    """new_paradigm/value.py BT4 (value.py:121-400)."""
+
+    def __init__(self, num_layers=10, d_model=512, d_ff=736, num_heads=8, fp8=False, micro_batch=0, head_dtype="bf16", seed=0):
+        self.num_layers, self.d_model = num_layers, d_model
+        self._shapes = bt4_shapes(num_layers, d_model, d_ff, num_heads)
+        self._sd = _default_init(self._shapes, seed)
+        self._engine = _Engine(_lib.ARCH_BT4, num_layers, d_model, num_heads, d_ff, fp8=fp8, micro_batch=micro_batch, head_dtype=head_dtype)
+        self._engine.load(self._sd)
+
+    @torch.no_grad()
+    def forward(self, inp, compute_loss=False):
+        """inp[0]: [b, seq_len, 8, 8, 19] -> policy [b, seq_len, 1929] (value.py:155-212)."""
+        if compute_loss:
+            raise NotImplementedError("losses are not part of the forward path")
+        x = inp[0]
+        b, s = x.shape[0], x.shape[1]
+        pol, _ = self._engine.forward(x, want_wdl=False)
+        return pol.view(b, s, VOCAB_RL)
+
+    __call__ = forward
+
+    @torch.no_grad()
+    def get_move_from_fen_no_thinking(self, fen, T=1, device="cuda", force_legal=True, return_probs=False):
+        planes = board.encode_fens([fen]).to(device)
+        logits, _ = self._engine.forward(planes, want_wdl=False)
+        mask = torch.from_numpy(board.legal_move_mask(fen)).to(device).unsqueeze(0) if force_legal else None
+        idx, _ = self._sample(logits, mask, T)
+        return policy_index[idx]
+
+    @torch.no_grad()
+    def get_batch_position_values(self, fens, device="cuda"):
+        """[N,3] probabilities [black win, draw, white win] (value.py:275-317)."""
+        if len(fens) == 0:
+            return torch.empty(0, 3, device=device)
+        planes = board.encode_fens(fens).to(device)
+        _, wdl = self._engine.forward(planes)
+        return torch.softmax(wdl, dim=-1)
+
+    def get_position_value(self, fen, device="cuda"):
+        return self.get_batch_position_values([fen], device)[0]
+
+    def calculate_move_values(self, fen, device="cuda"):
+        """(moves, value of each child for the side to move) (value.py:319-354)."""
+        moves, fens = board.child_fens(fen)
+        if not moves:
+            return [], torch.empty(0, device=device)
+        p = self.get_batch_position_values(fens, device)
+        vals = 0.5 * p[:, 1] + (p[:, 2] if board.white_to_move(fen) else p[:, 0])
+        return moves, vals
+
+    @torch.no_grad()
+    def get_best_move_value(self, fen, T=1, device="cuda", return_probs=False):
+        moves, vals = self.calculate_move_values(fen, device)
+        if not moves:
+            raise ValueError("No legal moves available")
+        if T == 0:
+            best = int(torch.argmax(vals).item())
+            probs = torch.zeros_like(vals)
+            probs[best] = 1.0
+        else:
+            probs = torch.softmax(vals / T, dim=0)
+            best = int(torch.multinomial(probs, num_samples=1).item())
+        return (moves[best], probs.cpu().numpy()) if return_probs else moves[best]
+
+
+class BT4Class(_ModelBase):
+    """BT4-class encoder: post-LN with residual scaling, mish FFN, generated attention bias,
+    attention policy gathered to the 1858 side-to-move-frame moves, WDL head."""
+
+    def __init__(self, num_layers=15, d_model=1024, d_ff=1536, num_heads=32, fp8=False, micro_batch=0,
+                 head_dtype="bf16", compress=32, hidden=256, gen=256, seed=0):
+        self.num_layers, self.d_model = num_layers, d_model
+        self._shapes = bt4_shapes(num_layers, d_model, d_ff, num_heads, True, compress, hidden, gen)
+        self._sd = _default_init(self._shapes, seed)
+        self._engine = _Engine(_lib.ARCH_BT4CLASS, num_layers, d_model, num_heads, d_ff, fp8=fp8, micro_batch=micro_batch,
+                               head_dtype=head_dtype, compress=compress, hidden=hidden, gen=gen)
+        self._engine.load(self._sd)
+
+    @torch.no_grad()
+    def forward(self, board_tokens):
+        """board_tokens [B,8,8,19] -> (policy_logits [B,1858], wdl [B,3])."""
+        return self._engine.forward(board_tokens)
+
+    __call__ = forward
+
+    @torch.no_grad()
+    def get_move_from_fen_no_thinking(self, fen, T=1, device="cuda", force_legal=True, return_probs=False):
+        planes = board.encode_fens([fen]).to(device)
+        logits, _ = self._engine.forward(planes, want_wdl=False)
+        mask = torch.from_numpy(board.legal_move_mask(fen, leela=True)).to(device).unsqueeze(0) if force_legal else None
+        idx, probs = self._sample(logits, mask, T)
+        move = policy_leela[idx]
+        if not board.white_to_move(fen):
+            move = move[0] + str(9 - int(move[1])) + move[2] + str(9 - int(move[3])) + move[4:]
+        return (move, probs[0]) if return_probs else move

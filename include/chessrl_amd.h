@@ -172,10 +172,12 @@ int crl_model_forward_compact(crl_model* m, const uint8_t* ids, const uint8_t* f
 int crl_model_vocab(const crl_model* m);
 /* 2*MAC count of one position through this model (for roofline accounting). */
 double crl_model_flops_per_position(const crl_model* m);
-/* Per-call switch: wrap every kernel family in HIP events on the call's stream and return
- * the accumulated milliseconds per family (gemm, attention, layernorm, embed, heads). */
+/* Switch: bracket every kernel launch with HIP events on the call's stream; each forward then
+ * ends with a stream synchronise and accumulates, per kernel family, the elapsed milliseconds,
+ * the launch count and (GEMMs) the 2*M*N*K work. Families: 0 fp8 GEMM, 1 attention,
+ * 2 LayerNorm, 3 embedding, 4 policy QK^T, 5 16-bit GEMM. flops6 may be NULL. */
 int crl_model_set_profiling(crl_model* m, int on);
-int crl_model_get_profile(crl_model* m, double* ms5, int64_t* launches5);
+int crl_model_get_profile(crl_model* m, double* ms6, int64_t* launches6, double* flops6);
 
 #ifdef __cplusplus
 }

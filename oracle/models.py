@@ -1,0 +1,440 @@
+"""CPU fp32 restatement of the reference forward passes. TEST INFRASTRUCTURE ONLY.
+
+Only tests/, __graft_entry__.smoke() and bench.py's cpu_baseline leg may import this
+package; the product path (chessrl_amd) never does.
+
+What each class follows (reference file:line):
+  GPTOracle      model_bis.py:25-34 (LayerNorm), :59-83 (causal attention), :94-99 (MLP),
+                 :110-113 (pre-LN block), :127-157 (module tree, tied embedding, sinusoid
+                 buffer), :358-370 (64-token forward, logits of token 63);
+                 utils/fen_encoder.py:41-67 (gating, stem).
+  BT4Oracle      new_paradigm/value.py:22-75 (gating, post-LN layer with GELU after ff2),
+                 :77-93 (absolute sinusoid table), :121-212 (forward, attention-policy head),
+                 :402-435 (value head); new_paradigm/attn.py:445-533 (relative attention).
+  BT4ClassOracle the BT4-class configuration of the benchmark (15x1024x32h, mish FFN 1536,
+                 generated attention bias, gathered 1858-move policy, WDL head). It is NOT in
+                 the reference repository; this module is its definition. PARITY UNPINNED:
+                 self-consistency only.
+  fp8 emulation  model_fp8.py:43,45,90,92,140 + pretrain_fp8.py:75-79 run the linears through
+                 transformer_engine (not vendored, not installable here): per-tensor e4m3
+                 scaling of input and weight, high-precision accumulate. Restated as
+                 quantise->dequantise->F.linear. PARITY UNPINNED against transformer_engine.
+
+Pins: library routines (F.layer_norm, F.gelu, F.scaled_dot_product_attention) are used
+directly; the relative shift is pinned in tests/test_oracle.py against the pad/reshape
+formulation and a brute-force definition; the move lists are pinned by SHA-256.
+"""
+import math
+
+import torch
+import torch.nn as nn
+import torch.nn.functional as F
+
+VOCAB_RL = 1929
+VOCAB_LEELA = 1858
+FP8_MAX = 448.0
+
+
+# ------------------------------------------------------------------ fp8 emulation
+def fp8_quant_dequant(x, scale):
+    """Round x*scale to OCP e4m3fn (saturating at +-448) and scale back."""
+    q = (x * scale).clamp(-FP8_MAX, FP8_MAX).to(torch.float8_e4m3fn).to(torch.float32)
+    return q / scale
+
+
+def amax_scale(amax):
+    return FP8_MAX / amax if amax > 0 else 1.0
+
+
+class Fp8Plan:
+    """Activation amax table [n_layer, 4]: slot 0 = input of the q/k/v linear, 1 = attention
+    output, 2 = input of the first FFN linear, 3 = input of the second FFN linear."""
+
+    def __init__(self, n_layer):
+        self.amax = torch.zeros(n_layer, 4)
+        self.recording = False
+
+    def lin(self, x, layer, slot, weight, bias):
+        if self.recording:
+            self.amax[layer, slot] = max(self.amax[layer, slot].item(), x.abs().max().item())
+            return F.linear(x, weight, bias)
+        sx = amax_scale(self.amax[layer, slot].item())
+        sw = amax_scale(weight.abs().max().item())
+        return F.linear(fp8_quant_dequant(x, sx), fp8_quant_dequant(weight, sw), bias)
+
+
+def _lin(plan, x, layer, slot, mod):
+    if plan is None:
+        return mod(x)
+    return plan.lin(x, layer, slot, mod.weight, mod.bias)
+
+
+# ------------------------------------------------------------------ shared pieces
+class MaGating(nn.Module):
+    def __init__(self, d_model):
+        super().__init__()
+        self.a = nn.Parameter(torch.zeros(64, d_model))
+        self.b = nn.Parameter(torch.ones(64, d_model))
+
+    def forward(self, x):
+        return x * torch.exp(self.a) + self.b
+
+
+class Stem(nn.Module):
+    """Linear(19->C) -> GELU -> LayerNorm -> gating (utils/fen_encoder.py:61-67)."""
+
+    def __init__(self, d_model):
+        super().__init__()
+        self.linear1 = nn.Linear(19, d_model)
+        self.layernorm1 = nn.LayerNorm(d_model)
+        self.ma_gating = MaGating(d_model)
+
+    def forward(self, planes):
+        x = planes.reshape(-1, 64, 19)
+        return self.ma_gating(self.layernorm1(F.gelu(self.linear1(x))))
+
+
+def sinusoid_gpt(rows, d_model):
+    """model_bis.py:141-145."""
+    pos = torch.arange(rows).unsqueeze(1)
+    div = torch.exp(torch.arange(0, d_model, 2).float() * (-math.log(10000.0) / d_model))
+    pe = torch.zeros(rows, d_model)
+    pe[:, 0::2] = torch.sin(pos * div)
+    pe[:, 1::2] = torch.cos(pos * div)
+    return pe
+
+
+def sinusoid_bt4(d_model):
+    """new_paradigm/value.py:80-89."""
+    pos = torch.arange(64).unsqueeze(1)
+    two_i = torch.arange(0, d_model, 2).float()
+    pe = torch.zeros(64, d_model)
+    pe[:, 0::2] = torch.sin(pos / (10000 ** (two_i / d_model)))
+    pe[:, 1::2] = torch.cos(pos / (10000 ** (two_i / d_model)))
+    return pe
+
+
+# ------------------------------------------------------------------ Model A
+class _AffineLN(nn.Module):
+    def __init__(self, n):
+        super().__init__()
+        self.weight = nn.Parameter(torch.ones(n))
+        self.bias = nn.Parameter(torch.zeros(n))
+
+    def forward(self, x):
+        return F.layer_norm(x, self.weight.shape, self.weight, self.bias, 1e-5)
+
+
+class _GPTAttn(nn.Module):
+    def __init__(self, C, H):
+        super().__init__()
+        self.c_attn = nn.Linear(C, 3 * C)
+        self.c_proj = nn.Linear(C, C)
+        self.n_head = H
+
+
+class _GPTMlp(nn.Module):
+    def __init__(self, C):
+        super().__init__()
+        self.c_fc = nn.Linear(C, 4 * C)
+        self.c_proj = nn.Linear(4 * C, C)
+
+
+class _GPTBlock(nn.Module):
+    def __init__(self, C, H):
+        super().__init__()
+        self.ln_1 = _AffineLN(C)
+        self.attn = _GPTAttn(C, H)
+        self.ln_2 = _AffineLN(C)
+        self.mlp = _GPTMlp(C)
+
+
+class GPTOracle(nn.Module):
+    def __init__(self, n_layer=6, n_head=8, n_embd=256, block_size=256, vocab_size=VOCAB_RL):
+        super().__init__()
+        self.n_layer, self.n_head, self.n_embd = n_layer, n_head, n_embd
+        self.FenEncoder = Stem(n_embd)
+        self.transformer = nn.ModuleDict(dict(
+            wte=nn.Embedding(vocab_size, n_embd),
+            h=nn.ModuleList([_GPTBlock(n_embd, n_head) for _ in range(n_layer)]),
+            ln_f=_AffineLN(n_embd)))
+        self.lm_head = nn.Linear(n_embd, vocab_size, bias=False)
+        self.register_buffer("pe", sinusoid_gpt(block_size, n_embd))
+        self.transformer.wte.weight = self.lm_head.weight
+
+    @torch.no_grad()
+    def forward_last(self, planes, plan=None):
+        """planes [B,8,8,19] -> logits [B,1929] of token 63 (model_bis.py:360-370)."""
+        x = self.FenEncoder(planes) + self.pe[:64]
+        B, T, C = x.shape
+        H = self.n_head
+        for li, blk in enumerate(self.transformer.h):
+            h = blk.ln_1(x)
+            q, k, v = _lin(plan, h, li, 0, blk.attn.c_attn).split(C, dim=2)
+            q, k, v = (t.view(B, T, H, C // H).transpose(1, 2) for t in (q, k, v))
+            y = F.scaled_dot_product_attention(q, k, v, is_causal=True)
+            y = y.transpose(1, 2).reshape(B, T, C)
+            x = x + _lin(plan, y, li, 1, blk.attn.c_proj)
+            h = blk.ln_2(x)
+            f = F.gelu(_lin(plan, h, li, 2, blk.mlp.c_fc))
+            x = x + _lin(plan, f, li, 3, blk.mlp.c_proj)
+        x = self.transformer.ln_f(x)
+        return self.lm_head(x[:, -1, :])
+
+
+# ------------------------------------------------------------------ Model B
+def rel_shift(s):
+    """new_paradigm/attn.py:525-533 in closed form for a [..., T, T] score:
+    out[i][j] = s[i][T-1-i+j] (j<=i), 0 (j==i+1), s[i+1][j-i-2] (j>i+1)."""
+    T = s.shape[-1]
+    i = torch.arange(T).unsqueeze(1)
+    j = torch.arange(T).unsqueeze(0)
+    low = j <= i
+    zero = j == i + 1
+    src_row = torch.where(low, i, (i + 1).clamp(max=T - 1)).expand(T, T)
+    src_col = torch.where(low, T - 1 - i + j, (j - i - 2).clamp(min=0))
+    out = s[..., src_row, src_col]
+    return out.masked_fill(zero, 0.0)
+
+
+class _RelAttn(nn.Module):
+    def __init__(self, C, H):
+        super().__init__()
+        self.query_proj = nn.Linear(C, C)
+        self.key_proj = nn.Linear(C, C)
+        self.value_proj = nn.Linear(C, C)
+        self.pos_proj = nn.Linear(C, C, bias=False)
+        self.u_bias = nn.Parameter(torch.empty(H, C // H))
+        self.v_bias = nn.Parameter(torch.empty(H, C // H))
+        nn.init.xavier_uniform_(self.u_bias)
+        nn.init.xavier_uniform_(self.v_bias)
+        self.out_proj = nn.Linear(C, C)
+
+
+class _BT4Layer(nn.Module):
+    def __init__(self, C, F_, H):
+        super().__init__()
+        self.attention = _RelAttn(C, H)
+        self.norm1 = nn.LayerNorm(C)
+        self.norm2 = nn.LayerNorm(C)
+        self.ff1 = nn.Linear(C, F_)
+        self.ff2 = nn.Linear(F_, C)
+
+
+class _ValueHead(nn.Module):
+    def __init__(self, C):
+        super().__init__()
+        self.dense1 = nn.Linear(C, 128)
+        self.dense2 = nn.Linear(128 * 64, 128)
+        self.dense3 = nn.Linear(128, 3)
+
+    def forward(self, x, act):
+        b = x.shape[0]
+        x = act(self.dense1(x)).reshape(b, -1)
+        return self.dense3(act(self.dense2(x)))
+
+
+class BT4Oracle(nn.Module):
+    def __init__(self, num_layers=10, d_model=512, d_ff=736, num_heads=8):
+        super().__init__()
+        self.num_layers, self.d_model, self.num_heads = num_layers, d_model, num_heads
+        self.layers = nn.ModuleList([_BT4Layer(d_model, d_ff, num_heads) for _ in range(num_layers)])
+        self.linear1 = nn.Linear(19, d_model)
+        self.layernorm1 = nn.LayerNorm(d_model)
+        self.policy_tokens_lin = nn.Linear(d_model, d_model)
+        self.queries_pol = nn.Linear(d_model, d_model)
+        self.keys_pol = nn.Linear(d_model, d_model)
+        self.ma_gating = MaGating(d_model)
+        self.policy_head = nn.Linear(64 * 64, VOCAB_RL, bias=False)
+        self.value_head = _ValueHead(d_model)
+        self.pe = sinusoid_bt4(d_model)  # plain attribute, absent from the state dict (value.py:82)
+
+    @torch.no_grad()
+    def forward_pv(self, planes):
+        """planes [B,8,8,19] -> (policy logits [B,1929], wdl logits [B,3])."""
+        x = planes.reshape(-1, 64, 19)
+        x = self.ma_gating(self.layernorm1(F.gelu(self.linear1(x))))
+        B, T, C = x.shape
+        H = self.num_heads
+        hs = C // H
+        pe = self.pe
+        for ly in self.layers:
+            at = ly.attention
+            q = at.query_proj(x).view(B, T, H, hs)
+            k = at.key_proj(x).view(B, T, H, hs).permute(0, 2, 1, 3)
+            v = at.value_proj(x).view(B, T, H, hs).permute(0, 2, 1, 3)
+            p = at.pos_proj(pe).view(T, H, hs)
+            content = torch.matmul((q + at.u_bias).transpose(1, 2), k.transpose(2, 3))
+            pos = torch.matmul((q + at.v_bias).transpose(1, 2), p.permute(1, 2, 0))
+            score = (content + rel_shift(pos)) / math.sqrt(C)
+            ctx = torch.matmul(F.softmax(score, -1), v).transpose(1, 2).reshape(B, T, C)
+            x = ly.norm1(at.out_proj(ctx) + x)
+            y = F.gelu(ly.ff2(ly.ff1(x)))
+            x = ly.norm2(y + x)
+        wdl = self.value_head(x, F.gelu)
+        pt = F.gelu(self.policy_tokens_lin(x)) + pe
+        qk = torch.matmul(self.queries_pol(pt), self.keys_pol(pt).transpose(-2, -1)) / math.sqrt(C)
+        return self.policy_head(qk.reshape(B, 64 * 64)), wdl
+
+
+# ------------------------------------------------------------------ Model C
+class _Smolgen(nn.Module):
+    def __init__(self, C, H, compress, hidden, gen):
+        super().__init__()
+        self.compress = nn.Linear(C, compress, bias=False)
+        self.hidden = nn.Linear(64 * compress, hidden)
+        self.hidden_ln = nn.LayerNorm(hidden)
+        self.gen_from = nn.Linear(hidden, H * gen)
+        self.gen_from_ln = nn.LayerNorm(H * gen)
+
+
+class _BT4ClassAttn(nn.Module):
+    def __init__(self, C):
+        super().__init__()
+        self.query_proj = nn.Linear(C, C)
+        self.key_proj = nn.Linear(C, C)
+        self.value_proj = nn.Linear(C, C)
+        self.out_proj = nn.Linear(C, C)
+
+
+class _BT4ClassLayer(nn.Module):
+    def __init__(self, C, F_, H, compress, hidden, gen):
+        super().__init__()
+        self.attention = _BT4ClassAttn(C)
+        self.smolgen = _Smolgen(C, H, compress, hidden, gen)
+        self.norm1 = nn.LayerNorm(C)
+        self.norm2 = nn.LayerNorm(C)
+        self.ff1 = nn.Linear(C, F_)
+        self.ff2 = nn.Linear(F_, C)
+
+
+def leela_gather_tables(policy_leela):
+    """For each Leela move: (from_token, to_token) on the real board for white rows and
+    for black rows (ranks mirrored back), plus (to_file, piece) for promotions."""
+    w_from, w_to, b_from, b_to, promo = [], [], [], [], []
+    for s in policy_leela:
+        ff, fr, tf, tr = ord(s[0]) - 97, int(s[1]) - 1, ord(s[2]) - 97, int(s[3]) - 1
+        w_from.append((7 - fr) * 8 + ff)
+        w_to.append((7 - tr) * 8 + tf)
+        b_from.append(fr * 8 + ff)
+        b_to.append(tr * 8 + tf)
+        promo.append(-1 if len(s) == 4 else tf * 4 + "qrb".index(s[4]))
+    t = lambda v: torch.tensor(v, dtype=torch.long)
+    return t(w_from), t(w_to), t(b_from), t(b_to), t(promo)
+
+
+class BT4ClassOracle(nn.Module):
+    def __init__(self, policy_leela, num_layers=15, d_model=1024, d_ff=1536, num_heads=32,
+                 compress=32, hidden=256, gen=256):
+        super().__init__()
+        self.num_layers, self.d_model, self.num_heads = num_layers, d_model, num_heads
+        self.layers = nn.ModuleList([_BT4ClassLayer(d_model, d_ff, num_heads, compress, hidden, gen)
+                                     for _ in range(num_layers)])
+        self.smol_weight_gen = nn.Linear(gen, 64 * 64, bias=False)
+        self.linear1 = nn.Linear(19, d_model)
+        self.layernorm1 = nn.LayerNorm(d_model)
+        self.ma_gating = MaGating(d_model)
+        self.policy_tokens_lin = nn.Linear(d_model, d_model)
+        self.queries_pol = nn.Linear(d_model, d_model)
+        self.keys_pol = nn.Linear(d_model, d_model)
+        self.promotion_offsets = nn.Linear(d_model, 4, bias=False)
+        self.value_head = _ValueHead(d_model)
+        self.tables = leela_gather_tables(policy_leela)
+
+    @torch.no_grad()
+    def forward_pv(self, planes, plan=None):
+        """planes [B,8,8,19] -> (policy logits [B,1858] in the side-to-move frame, wdl logits [B,3])."""
+        planes = planes.reshape(-1, 64, 19)
+        white = planes[:, 0, 12] > 0.5
+        x = self.ma_gating(self.layernorm1(F.gelu(self.linear1(planes))))
+        B, T, C = x.shape
+        H = self.num_heads
+        hs = C // H
+        alpha = (2.0 * self.num_layers) ** -0.25
+        for li, ly in enumerate(self.layers):
+            at, sm = ly.attention, ly.smolgen
+            if plan is None:
+                q, k, v, comp = at.query_proj(x), at.key_proj(x), at.value_proj(x), sm.compress(x)
+            else:
+                # one fused linear over [q;k;v;compress] with a single weight scale
+                w = torch.cat([at.query_proj.weight, at.key_proj.weight, at.value_proj.weight, sm.compress.weight])
+                b = torch.cat([at.query_proj.bias, at.key_proj.bias, at.value_proj.bias, torch.zeros(sm.compress.weight.shape[0])])
+                out = plan.lin(x, li, 0, w, b)
+                q, k, v, comp = out.split([C, C, C, sm.compress.weight.shape[0]], dim=-1)
+            hid = sm.hidden_ln(F.silu(sm.hidden(comp.reshape(B, -1))))
+            gen = sm.gen_from_ln(F.silu(sm.gen_from(hid))).view(B, H, -1)
+            bias = self.smol_weight_gen(gen).view(B, H, 64, 64)
+            q, k, v = (t.view(B, T, H, hs).transpose(1, 2) for t in (q, k, v))
+            score = torch.matmul(q, k.transpose(-2, -1)) / math.sqrt(hs) + bias
+            ctx = torch.matmul(F.softmax(score, -1), v).transpose(1, 2).reshape(B, T, C)
+            x = ly.norm1(x + alpha * _lin(plan, ctx, li, 1, at.out_proj))
+            f = F.mish(_lin(plan, x, li, 2, ly.ff1))
+            x = ly.norm2(x + alpha * _lin(plan, f, li, 3, ly.ff2))
+        wdl = self.value_head(x, F.mish)
+        tok = F.mish(self.policy_tokens_lin(x))
+        qp, kp = self.queries_pol(tok), self.keys_pol(tok)
+        a = torch.matmul(qp, kp.transpose(-2, -1)) / math.sqrt(C)       # [B, from, to]
+        w_from, w_to, b_from, b_to, promo = self.tables
+        wl = white.unsqueeze(1)
+        frm = torch.where(wl, w_from.unsqueeze(0), b_from.unsqueeze(0))
+        to = torch.where(wl, w_to.unsqueeze(0), b_to.unsqueeze(0))
+        logits = a.reshape(B, 4096).gather(1, frm * 64 + to)
+        # promotion offsets from the keys of the promotion rank (rank 8 for white = tokens
+        # 0..7, rank 1 for black = tokens 56..63): q, r, b each get their own offset plus
+        # the knight one.
+        rank_tok = torch.where(white.unsqueeze(1), torch.arange(8).unsqueeze(0), torch.arange(56, 64).unsqueeze(0))
+        keys = kp.gather(1, rank_tok.unsqueeze(-1).expand(B, 8, C))
+        off = self.promotion_offsets(keys)                                # [B, 8 files, 4]
+        off = off[:, :, :3] + off[:, :, 3:4]
+        is_promo = promo >= 0
+        pidx = promo.clamp(min=0)
+        add = off[:, pidx // 4, pidx % 4] * is_promo
+        return logits + add, wdl
+
+
+# ------------------------------------------------------------------ helpers
+def spec_init_(model, seed=0):
+    """Benchmark initialisation: Linear/Embedding weights normal(0, 0.02), zero biases, LayerNorm
+    at identity, gating a=0/b=1 (model_bis.py:163-169); relative biases keep their xavier draw."""
+    g = torch.Generator().manual_seed(seed)
+    for name, p in model.named_parameters():
+        if name.endswith("u_bias") or name.endswith("v_bias"):
+            p.data.copy_(torch.empty_like(p).uniform_(-0.3, 0.3, generator=g))
+        elif "ma_gating.a" in name:
+            p.data.zero_()
+        elif "ma_gating.b" in name:
+            p.data.fill_(1.0)
+        elif p.dim() >= 2:
+            p.data.copy_(torch.empty_like(p).normal_(0.0, 0.02, generator=g))
+        elif name.endswith("bias"):
+            p.data.zero_()
+        else:
+            p.data.fill_(1.0)
+    return model
+
+
+def test_init_(model, seed=0, wstd=0.02):
+    """Initialisation for parity tests: every parameter (biases, LayerNorm affine, gating)
+    is non-trivial so a dropped or mis-indexed term changes the output."""
+    g = torch.Generator().manual_seed(seed)
+    rnd = lambda p, s: torch.empty_like(p).normal_(0.0, s, generator=g)
+    for name, p in model.named_parameters():
+        if "ma_gating.a" in name:
+            p.data.copy_(rnd(p, 0.1))
+        elif "ma_gating.b" in name:
+            p.data.copy_(1.0 + rnd(p, 0.1))
+        elif name.endswith("u_bias") or name.endswith("v_bias"):
+            p.data.copy_(rnd(p, 0.2))
+        elif p.dim() >= 2:
+            p.data.copy_(rnd(p, wstd))
+        elif name.endswith("bias"):
+            p.data.copy_(rnd(p, 0.05))
+        else:
+            p.data.copy_(1.0 + rnd(p, 0.1))
+    return model
+
+
+def masked_policy(logits, mask, temperature=1.0):
+    """logits + (1-mask)*(-999), softmax(./T) (model_bis.py:382-389)."""
+    x = logits + (1.0 - mask.to(logits.dtype)) * -999.0
+    return F.softmax(x / temperature, dim=-1)
