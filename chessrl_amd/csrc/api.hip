@@ -177,10 +177,14 @@ int crl_random_positions(uint64_t seed, int n, int max_plies, double late_fracti
     SplitMix64 rng(mix.next());
     const bool late = late_fraction > 0 && (double)(rng.next() >> 11) * (1.0 / 9007199254740992.0) < late_fraction;
     Board b = random_playout(rng, max_plies, late ? late_max_pieces : 0);
+    // Positions reach the models as FEN strings, and the FEN of a live board names the
+    // en-passant square only when the capture is legal: encode what that FEN encodes.
+    const std::string fen = b.fen(true);
+    b.set_fen(fen.c_str());
     if (out_planes) b.planes(out_planes + (size_t)i * 64 * NUM_PLANES);
     if (out_masks_rl) legal_mask_rl(b, out_masks_rl + (size_t)i * VOCAB_RL);
     if (out_masks_leela) legal_mask_leela(b, out_masks_leela + (size_t)i * VOCAB_LEELA);
-    if (out_fens96) put_str(out_fens96 + (size_t)i * 96, 96, b.fen(true));
+    if (out_fens96) put_str(out_fens96 + (size_t)i * 96, 96, fen);
     return 0;
   });
 }

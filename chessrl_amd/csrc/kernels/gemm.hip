@@ -10,39 +10,60 @@
 //    kernel is written on bytes: one code path serves 2-byte and 1-byte element types.
 //  * LDS rows are 128 bytes = 8 chunks of 16 bytes; chunk c of row r is stored at
 //    chunk c ^ ((r ^ (r>>3)) & 7), which keeps both the 16-byte fragment reads and the
-//    row-wise stores free of bank conflicts.
+//    row-wise stores free of bank conflicts (measured: SQ_LDS_BANK_CONFLICT = 0).
 //  * Each wave owns a (WM x WN) sub-tile made of 32x32 MFMA tiles. The weight rows are
 //    the MFMA row operand and the activation rows the column operand, so a lane ends
 //    up holding four consecutive output columns of one output row, which the epilogue
 //    moves through LDS as 16-byte chunks.
-//  * Global loads for slab k+1 are issued before the MFMAs of slab k and written to the
-//    other LDS stage afterwards (register double buffering, one barrier per slab).
+//  * Global loads for slab k+1 are issued before the MFMAs of slab k and written to LDS
+//    afterwards (register staging). With two LDS stages that costs one barrier per slab;
+//    the single-stage variant uses two barriers and half the LDS so two workgroups fit
+//    on a CU and cover each other's stalls.
 //  * Workgroup ids are remapped so each XCD (ids round-robin over 8 XCDs) walks a
 //    contiguous range of tiles, N fastest: the weight matrix stays in that XCD's L2
 //    and every activation slab is fetched from HBM by one XCD only.
+#include <type_traits>
+
 #include "common.hpp"
 
 namespace crl {
 
-template <int BM_, int BN_, int WGM_, int WGN_>
+template <int BM_, int BN_, int WGM_, int WGN_, int STAGES_, int FRAG_DB_, int MIN_WAVES_>
 struct GemmCfg {
-  static constexpr int BM = BM_, BN = BN_, WGM = WGM_, WGN = WGN_;
-  static constexpr int NT = 64 * WGM * WGN;
+  static constexpr int BM = BM_, BN = BN_, WGM = WGM_, WGN = WGN_, STAGES = STAGES_, FRAG_DB = FRAG_DB_;
+  static constexpr int MIN_WAVES = MIN_WAVES_;
+  static constexpr int NW = WGM * WGN, NT = 64 * NW;
   static constexpr int WM = BM / WGM, WN = BN / WGN;
   static constexpr int TM = WM / 32, TN = WN / 32;
   static constexpr int ROWS_PER_PASS = NT / 8;
   static constexpr int A_PASSES = BM / ROWS_PER_PASS, W_PASSES = BN / ROWS_PER_PASS;
   static constexpr int STAGE_BYTES = (BM + BN) * 128;
-  static constexpr int LDS_BYTES = 2 * STAGE_BYTES;
+  static constexpr int EPI_BYTES = NW * 32 * WN * 4;
+  static constexpr int LDS_BYTES = STAGES * STAGE_BYTES > EPI_BYTES ? STAGES * STAGE_BYTES : EPI_BYTES;
   static_assert(BM % ROWS_PER_PASS == 0 && BN % ROWS_PER_PASS == 0, "tile/threads mismatch");
+  static_assert(WN >= 32 && WM >= 32, "wave tile too small");
 };
 
 __device__ __forceinline__ int lds_swizzle(int row) { return (row ^ (row >> 3)) & 7; }
+
+// Compile-time loop: f is called with std::integral_constant<int, I> for I in [0, N), so
+// register arrays indexed by I never need dynamic indexing whatever the body size.
+template <int I, int N, typename F>
+__device__ __forceinline__ void static_for(F&& f) {
+  if constexpr (I < N) {
+    f(std::integral_constant<int, I>{});
+    static_for<I + 1, N>(f);
+  }
+}
 
 // One MFMA operand fragment of a lane: 16 bytes (2-byte types, 8 k-elements) or
 // 32 bytes (fp8, 32 k-elements) of one LDS row.
 template <int IN_DT>
 struct Frag {
+  i32x4_t lo;
+};
+template <>
+struct Frag<DT_FP8> {
   i32x4_t lo, hi;
 };
 
@@ -97,8 +118,16 @@ __device__ __forceinline__ void store1(void* base, long off, float v) {
   else reinterpret_cast<uint8_t*>(base)[off] = f32_to_fp8(v);
 }
 
+// Orders this wave's LDS traffic (LDS executes one wave's operations in issue order) and
+// keeps the compiler from moving accesses across the point.
+__device__ __forceinline__ void wave_lds_fence() {
+  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+  __builtin_amdgcn_wave_barrier();
+  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+}
+
 template <typename Cfg, int IN_DT, int OUT_DT>
-__global__ void __launch_bounds__(Cfg::NT) gemm_kernel(const GemmArgs a) {
+__global__ void __launch_bounds__(Cfg::NT, Cfg::MIN_WAVES) gemm_kernel(const GemmArgs a) {
   constexpr int BM = Cfg::BM, BN = Cfg::BN, TM = Cfg::TM, TN = Cfg::TN;
   constexpr int ESZ = (IN_DT == DT_FP8) ? 1 : 2;
   constexpr int KSTEPS = (IN_DT == DT_FP8) ? 2 : 4;
@@ -126,34 +155,51 @@ __global__ void __launch_bounds__(Cfg::NT) gemm_kernel(const GemmArgs a) {
   const long lda_b = a.lda * ESZ, ldw_b = a.ldw * ESZ;
 
   const int lchunk = tid & 7, lrow = tid >> 3;
-  uint4 ra[Cfg::A_PASSES], rw[Cfg::W_PASSES];
+  i32x4_t ra[Cfg::A_PASSES], rw[Cfg::W_PASSES];
 
+  // Rows past M or N are clamped to the last valid row: they only feed output rows or
+  // columns that are never stored, so no zero fill (and no branch) is needed.
+  const uint8_t* aptr[Cfg::A_PASSES];
+  const uint8_t* wptr[Cfg::W_PASSES];
+#pragma unroll
+  for (int i = 0; i < Cfg::A_PASSES; ++i) {
+    int gm = m0 + lrow + i * Cfg::ROWS_PER_PASS;
+    gm = gm < a.M ? gm : a.M - 1;
+    aptr[i] = Ab + (long)gm * lda_b + (lchunk << 4);
+  }
+#pragma unroll
+  for (int i = 0; i < Cfg::W_PASSES; ++i) {
+    int gn = n0 + lrow + i * Cfg::ROWS_PER_PASS;
+    gn = gn < a.N ? gn : a.N - 1;
+    wptr[i] = Wb + (long)gn * ldw_b + (lchunk << 4);
+  }
+  // A K tail shorter than the slab is loaded from a clamped (valid) address and replaced by
+  // zeros when the registers are written to LDS, i.e. after the wait that is needed there
+  // anyway: nothing depends on the loaded data while the MFMAs of the current slab run.
+  const long kmax = kbytes - 16;  // last valid 16-byte chunk offset along K
+  const long kmine = lchunk << 4;
   auto gload = [&](int slab) {
-    const long kb = ((long)slab << 7) + (lchunk << 4);
-    const bool kok = kb < kbytes;
+    const long kb = ((long)slab << 7);
+    const long kofs = (kb + kmine <= kmax) ? kb : kmax - kmine;
 #pragma unroll
-    for (int i = 0; i < Cfg::A_PASSES; ++i) {
-      const int gm = m0 + lrow + i * Cfg::ROWS_PER_PASS;
-      ra[i] = (kok && gm < a.M) ? *reinterpret_cast<const uint4*>(Ab + (long)gm * lda_b + kb) : make_uint4(0, 0, 0, 0);
-    }
+    for (int i = 0; i < Cfg::A_PASSES; ++i) ra[i] = *reinterpret_cast<const i32x4_t*>(aptr[i] + kofs);
 #pragma unroll
-    for (int i = 0; i < Cfg::W_PASSES; ++i) {
-      const int gn = n0 + lrow + i * Cfg::ROWS_PER_PASS;
-      rw[i] = (kok && gn < a.N) ? *reinterpret_cast<const uint4*>(Wb + (long)gn * ldw_b + kb) : make_uint4(0, 0, 0, 0);
-    }
+    for (int i = 0; i < Cfg::W_PASSES; ++i) rw[i] = *reinterpret_cast<const i32x4_t*>(wptr[i] + kofs);
   };
-  auto sstore = [&](int stage) {
+  auto sstore = [&](int stage, int slab) {
     uint8_t* sW = smem + stage * Cfg::STAGE_BYTES;
     uint8_t* sA = sW + BN * 128;
+    const bool kok = ((long)slab << 7) + kmine <= kmax;
+    const i32x4_t z = {0, 0, 0, 0};
 #pragma unroll
     for (int i = 0; i < Cfg::A_PASSES; ++i) {
       const int r = lrow + i * Cfg::ROWS_PER_PASS;
-      *reinterpret_cast<uint4*>(sA + r * 128 + ((lchunk ^ lds_swizzle(r)) << 4)) = ra[i];
+      *reinterpret_cast<i32x4_t*>(sA + r * 128 + ((lchunk ^ lds_swizzle(r)) << 4)) = kok ? ra[i] : z;
     }
 #pragma unroll
     for (int i = 0; i < Cfg::W_PASSES; ++i) {
       const int r = lrow + i * Cfg::ROWS_PER_PASS;
-      *reinterpret_cast<uint4*>(sW + r * 128 + ((lchunk ^ lds_swizzle(r)) << 4)) = rw[i];
+      *reinterpret_cast<i32x4_t*>(sW + r * 128 + ((lchunk ^ lds_swizzle(r)) << 4)) = kok ? rw[i] : z;
     }
   };
 
@@ -165,47 +211,103 @@ __global__ void __launch_bounds__(Cfg::NT) gemm_kernel(const GemmArgs a) {
 #pragma unroll
       for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
 
+  // LDS rows this lane reads its fragments from (fixed for the whole kernel).
+  int wrow_off[TN], wrow_sw[TN], arow_off[TM], arow_sw[TM];
+#pragma unroll
+  for (int tn = 0; tn < TN; ++tn) {
+    const int wr = wn * Cfg::WN + tn * 32 + lr;
+    wrow_off[tn] = wr * 128;
+    wrow_sw[tn] = lds_swizzle(wr);
+  }
+#pragma unroll
+  for (int tm = 0; tm < TM; ++tm) {
+    const int ar = wm * Cfg::WM + tm * 32 + lr;
+    arow_off[tm] = BN * 128 + ar * 128;
+    arow_sw[tm] = lds_swizzle(ar);
+  }
+
   gload(0);
-  sstore(0);
+  sstore(0, 0);
   __syncthreads();
 
+  // With FRAG_DB two fragment sets alternate: while the MFMAs of k-step ks run on one set,
+  // the LDS reads of k-step ks+1 fill the other; the scheduling barriers keep that order
+  // (left alone the compiler reuses one register set and exposes the LDS latency before
+  // every MFMA group). Without it one set is used and a second resident wave hides the latency.
+  // (fp8 fragments are twice as large: two sets would not fit beside 256 accumulators.)
+  constexpr bool FRAG_DB = Cfg::FRAG_DB && IN_DT != DT_FP8;
+  constexpr int NSET = FRAG_DB ? 2 : 1;
+  Frag<IN_DT> wf[NSET][TN], xf[NSET][TM];
+  auto lds_frags = [&](const uint8_t* st, int ks, int set) {
+#pragma unroll
+    for (int tn = 0; tn < TN; ++tn) wf[set][tn] = load_frag<IN_DT>(st + wrow_off[tn], wrow_sw[tn], ks, g);
+#pragma unroll
+    for (int tm = 0; tm < TM; ++tm) xf[set][tm] = load_frag<IN_DT>(st + arow_off[tm], arow_sw[tm], ks, g);
+  };
+  auto mfmas = [&](int set) {
+#pragma unroll
+    for (int tn = 0; tn < TN; ++tn)
+#pragma unroll
+      for (int tm = 0; tm < TM; ++tm) acc[tn][tm] = mfma_frag<IN_DT>(wf[set][tn], xf[set][tm], acc[tn][tm]);
+  };
+
   for (int slab = 0; slab < nslab; ++slab) {
-    const int stage = slab & 1;
-    if (slab + 1 < nslab) gload(slab + 1);
-    const uint8_t* sW = smem + stage * Cfg::STAGE_BYTES;
-    const uint8_t* sA = sW + BN * 128;
+    const int stage = Cfg::STAGES == 2 ? (slab & 1) : 0;
+    const uint8_t* st = smem + stage * Cfg::STAGE_BYTES;
+    const bool more = slab + 1 < nslab;
+    if (more) gload(slab + 1);
+    if constexpr (FRAG_DB) {
+      lds_frags(st, 0, 0);
+      __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-    for (int ks = 0; ks < KSTEPS; ++ks) {
-      Frag<IN_DT> wf[TN], xf[TM];
-#pragma unroll
-      for (int tn = 0; tn < TN; ++tn) {
-        const int wr = wn * Cfg::WN + tn * 32 + lr;
-        wf[tn] = load_frag<IN_DT>(sW + wr * 128, lds_swizzle(wr), ks, g);
+      for (int ks = 0; ks < KSTEPS; ++ks) {
+        if (ks + 1 < KSTEPS) lds_frags(st, ks + 1, (ks + 1) & 1);
+        __builtin_amdgcn_sched_barrier(0);
+        mfmas(ks & 1);
+        __builtin_amdgcn_sched_barrier(0);
       }
+    } else {
 #pragma unroll
-      for (int tm = 0; tm < TM; ++tm) {
-        const int ar = wm * Cfg::WM + tm * 32 + lr;
-        xf[tm] = load_frag<IN_DT>(sA + ar * 128, lds_swizzle(ar), ks, g);
+      for (int ks = 0; ks < KSTEPS; ++ks) {
+        lds_frags(st, ks, 0);
+        mfmas(0);
       }
-#pragma unroll
-      for (int tn = 0; tn < TN; ++tn)
-#pragma unroll
-        for (int tm = 0; tm < TM; ++tm) acc[tn][tm] = mfma_frag<IN_DT>(wf[tn], xf[tm], acc[tn][tm]);
     }
-    if (slab + 1 < nslab) sstore(stage ^ 1);
-    __syncthreads();
+    if constexpr (Cfg::STAGES == 2) {
+      if (more) sstore(stage ^ 1, slab + 1);
+      __syncthreads();
+    } else {
+      __syncthreads();
+      if (more) sstore(0, slab + 1);
+      __syncthreads();
+    }
   }
 
   // Epilogue. acc[tn][tm][r] is output row m = m0 + wm*WM + tm*32 + lr, column
   // n = n0 + wn*WN + tn*32 + 8*(r/4) + 4*g + (r%4). Each wave passes its 32 x WN strip
-  // through a private LDS patch (16-byte chunks XOR-swizzled by row) so that the
-  // bias/activation/residual/quantise code is one compact loop and every store
-  // instruction writes whole contiguous row segments.
-  constexpr int WN = Cfg::WN, CH = WN / 4, ITERS = (32 * CH) / 64;
+  // through a private LDS patch (16-byte chunks XOR-swizzled by row) so that every store
+  // instruction writes whole contiguous row segments. A lane keeps the same four columns
+  // for every row of the strip (64 lanes cover 64/CH rows x CH chunks per step), so its
+  // bias values are loaded once; IU steps are processed together so their LDS reads and
+  // residual loads overlap, and the activation is selected once per group, not per element.
+  constexpr int WN = Cfg::WN, CH = WN / 4, ITERS = (32 * CH) / 64, RSTEP = 64 / CH;
+  constexpr int IU = ITERS < 4 ? ITERS : 4;
   float* sC = reinterpret_cast<float*>(smem) + wave * (32 * WN);
-  float local_amax = 0.f;
+  const int ec = lane % CH, er = lane / CH;
+  const int n = n0 + wn * WN + ec * 4;
+  const bool n_ok = n < a.N;
+  const bool full = a.vec_ok && (n + 3 < a.N) && !(n < a.nsplit && n + 3 >= a.nsplit);
+  float bias4[4] = {0.f, 0.f, 0.f, 0.f};
+  if (a.bias && n_ok) {
 #pragma unroll
-  for (int tm = 0; tm < TM; ++tm) {
+    for (int e = 0; e < 4; ++e) if (n + e < a.N) bias4[e] = a.bias[n + e];
+  }
+  const bool res_f32 = a.res_dtype == DT_F32, res_f16 = a.res_dtype == DT_F16;
+  const float descale = a.descale, alpha = a.alpha;
+  float local_amax = 0.f;
+
+  static_for<0, TM>([&](auto tmc) {
+    constexpr int tm = decltype(tmc)::value;
 #pragma unroll
     for (int tn = 0; tn < TN; ++tn)
 #pragma unroll
@@ -214,69 +316,120 @@ __global__ void __launch_bounds__(Cfg::NT) gemm_kernel(const GemmArgs a) {
         f32x4_t v4 = {acc[tn][tm][4 * rq], acc[tn][tm][4 * rq + 1], acc[tn][tm][4 * rq + 2], acc[tn][tm][4 * rq + 3]};
         *reinterpret_cast<f32x4_t*>(sC + lr * WN + ((chunk ^ (lr & (CH - 1))) << 2)) = v4;
       }
-    __syncthreads();
+    wave_lds_fence();
 #pragma unroll 1
-    for (int it = 0; it < ITERS; ++it) {
-      const int idx = it * 64 + lane;
-      const int r = idx / CH, c = idx - r * CH;
-      const int m = m0 + wm * Cfg::WM + tm * 32 + r;
-      const int n = n0 + wn * WN + c * 4;
-      if (m >= a.M || n >= a.N) continue;
-      const f32x4_t v4 = *reinterpret_cast<const f32x4_t*>(sC + r * WN + ((c ^ (r & (CH - 1))) << 2));
-      float v[4] = {v4[0], v4[1], v4[2], v4[3]};
-      const bool full = a.vec_ok && (n + 3 < a.N) && !(n < a.nsplit && n + 3 >= a.nsplit);
+    for (int ito = 0; ito < ITERS; ito += IU) {
+      const int rbase = er + ito * RSTEP;
+      const int mbase = m0 + wm * Cfg::WM + tm * 32 + rbase;
+      float v[IU][4];
+      f32x4_t lv[IU];
 #pragma unroll
-      for (int e = 0; e < 4; ++e) {
-        float x = v[e] * a.descale;
-        if (a.bias && n + e < a.N) x += a.bias[n + e];
-        v[e] = apply_act(x, a.act) * a.alpha;
+      for (int it = 0; it < IU; ++it) {
+        const int r = rbase + it * RSTEP;
+        lv[it] = *reinterpret_cast<const f32x4_t*>(sC + r * WN + ((ec ^ (r & (CH - 1))) << 2));
+      }
+      float rv[IU][4];
+      if (a.res) {
+#pragma unroll
+        for (int it = 0; it < IU; ++it) {
+          const int m = mbase + it * RSTEP;
+#pragma unroll
+          for (int e = 0; e < 4; ++e) rv[it][e] = 0.f;
+          if (m < a.M && n_ok) {
+            const long ro = (long)(a.res_rows > 0 ? m % a.res_rows : m) * a.ldr + n;
+            if (res_f32) {
+              const float* rp = reinterpret_cast<const float*>(a.res) + ro;
+              if (full) { const float4 r4 = *reinterpret_cast<const float4*>(rp); rv[it][0] = r4.x; rv[it][1] = r4.y; rv[it][2] = r4.z; rv[it][3] = r4.w; }
+              else {
+#pragma unroll
+                for (int e = 0; e < 4; ++e) if (n + e < a.N) rv[it][e] = rp[e];
+              }
+            } else {
+              const uint16_t* rp = reinterpret_cast<const uint16_t*>(a.res) + ro;
+              uint16_t rb[4] = {0, 0, 0, 0};
+              if (full) {
+                const uint2 r2 = *reinterpret_cast<const uint2*>(rp);
+                rb[0] = (uint16_t)(r2.x & 0xffff); rb[1] = (uint16_t)(r2.x >> 16);
+                rb[2] = (uint16_t)(r2.y & 0xffff); rb[3] = (uint16_t)(r2.y >> 16);
+              } else {
+#pragma unroll
+                for (int e = 0; e < 4; ++e) if (n + e < a.N) rb[e] = rp[e];
+              }
+#pragma unroll
+              for (int e = 0; e < 4; ++e) rv[it][e] = res_f16 ? f16_bits_to_f32(rb[e]) : bf16_bits_to_f32(rb[e]);
+            }
+          }
+        }
+      }
+#pragma unroll
+      for (int it = 0; it < IU; ++it)
+#pragma unroll
+        for (int e = 0; e < 4; ++e) v[it][e] = fmaf(lv[it][e], descale, bias4[e]);
+      switch (a.act) {  // uniform
+        case ACT_GELU:
+#pragma unroll
+          for (int it = 0; it < IU; ++it)
+#pragma unroll
+            for (int e = 0; e < 4; ++e) v[it][e] = act_gelu(v[it][e]);
+          break;
+        case ACT_MISH:
+#pragma unroll
+          for (int it = 0; it < IU; ++it)
+#pragma unroll
+            for (int e = 0; e < 4; ++e) v[it][e] = act_mish(v[it][e]);
+          break;
+        case ACT_SWISH:
+#pragma unroll
+          for (int it = 0; it < IU; ++it)
+#pragma unroll
+            for (int e = 0; e < 4; ++e) v[it][e] = act_swish(v[it][e]);
+          break;
+        default: break;
       }
       if (a.res) {
-        const long ro = (long)(a.res_rows > 0 ? m % a.res_rows : m) * a.ldr + n;
-        if (a.res_dtype == DT_F32) {
-          const float* rp = reinterpret_cast<const float*>(a.res) + ro;
-          if (full) { float4 r4 = *reinterpret_cast<const float4*>(rp); v[0] += r4.x; v[1] += r4.y; v[2] += r4.z; v[3] += r4.w; }
-          else {
 #pragma unroll
-            for (int e = 0; e < 4; ++e) if (n + e < a.N) v[e] += rp[e];
-          }
-        } else {
-          const uint16_t* rp = reinterpret_cast<const uint16_t*>(a.res) + ro;
-          uint16_t rb[4] = {0, 0, 0, 0};
-          if (full) {
-            uint2 r2 = *reinterpret_cast<const uint2*>(rp);
-            rb[0] = (uint16_t)(r2.x & 0xffff); rb[1] = (uint16_t)(r2.x >> 16);
-            rb[2] = (uint16_t)(r2.y & 0xffff); rb[3] = (uint16_t)(r2.y >> 16);
-          } else {
+        for (int it = 0; it < IU; ++it)
 #pragma unroll
-            for (int e = 0; e < 4; ++e) if (n + e < a.N) rb[e] = rp[e];
-          }
+          for (int e = 0; e < 4; ++e) v[it][e] = fmaf(v[it][e], alpha, rv[it][e]);
+      } else {
 #pragma unroll
-          for (int e = 0; e < 4; ++e) v[e] += a.res_dtype == DT_F16 ? f16_bits_to_f32(rb[e]) : bf16_bits_to_f32(rb[e]);
-        }
+        for (int it = 0; it < IU; ++it)
+#pragma unroll
+          for (int e = 0; e < 4; ++e) v[it][e] *= alpha;
       }
       if (a.amax) {
 #pragma unroll
-        for (int e = 0; e < 4; ++e) if (n + e < a.N) local_amax = fmaxf(local_amax, fabsf(v[e]));
+        for (int it = 0; it < IU; ++it)
+#pragma unroll
+          for (int e = 0; e < 4; ++e)
+            if (mbase + it * RSTEP < a.M && n + e < a.N) local_amax = fmaxf(local_amax, fabsf(v[it][e]));
       }
       if constexpr (OUT_DT == DT_FP8) {
+        const float os = a.out_scale;
 #pragma unroll
-        for (int e = 0; e < 4; ++e) v[e] *= a.out_scale;
+        for (int it = 0; it < IU; ++it)
+#pragma unroll
+          for (int e = 0; e < 4; ++e) v[it][e] *= os;
       }
-      if (full) {
-        if (n < a.nsplit) store4<OUT_DT>(a.C, (long)m * a.ldc + n, v);
-        else store4<OUT_DT>(a.C2, (long)m * a.ldc2 + (n - a.nsplit), v);
-      } else {
 #pragma unroll
-        for (int e = 0; e < 4; ++e) {
-          if (n + e >= a.N) continue;
-          if (n + e < a.nsplit) store1<OUT_DT>(a.C, (long)m * a.ldc + n + e, v[e]);
-          else store1<OUT_DT>(a.C2, (long)m * a.ldc2 + (n + e - a.nsplit), v[e]);
+      for (int it = 0; it < IU; ++it) {
+        const int m = mbase + it * RSTEP;
+        if (m >= a.M || !n_ok) continue;
+        if (full) {
+          if (n < a.nsplit) store4<OUT_DT>(a.C, (long)m * a.ldc + n, v[it]);
+          else store4<OUT_DT>(a.C2, (long)m * a.ldc2 + (n - a.nsplit), v[it]);
+        } else {
+#pragma unroll
+          for (int e = 0; e < 4; ++e) {
+            if (n + e >= a.N) continue;
+            if (n + e < a.nsplit) store1<OUT_DT>(a.C, (long)m * a.ldc + n + e, v[it][e]);
+            else store1<OUT_DT>(a.C2, (long)m * a.ldc2 + (n + e - a.nsplit), v[it][e]);
+          }
         }
       }
     }
-    __syncthreads();
-  }
+    wave_lds_fence();
+  });
   if (a.amax) {
     local_amax = wave_max(local_amax);
     if (lane == 0) atomic_amax(a.amax, local_amax);
@@ -284,9 +437,14 @@ __global__ void __launch_bounds__(Cfg::NT) gemm_kernel(const GemmArgs a) {
 }
 
 // ---- host-side dispatch -------------------------------------------------------------
-typedef GemmCfg<256, 256, 2, 2> CfgBig;     // 4 waves, 128x128 per wave
-typedef GemmCfg<128, 128, 2, 2> CfgMid;     // 4 waves, 64x64 per wave
-typedef GemmCfg<64, 64, 2, 2> CfgSmall;     // 4 waves, 32x32 per wave
+//                 BM   BN  WGM WGN stages frag_db min_waves
+// Measured on MI355X (M=65536, K=1024..8192): the 8-wave 256x256 tile (two waves per SIMD
+// covering each other's LDS and barrier stalls) beats the 4-wave 256x256 tile with
+// double-buffered fragments, the single-stage 256x128 tile and the 128x128 tile for
+// every trunk shape in both fp8 and bf16.
+typedef GemmCfg<256, 256, 2, 4, 2, 0, 2> CfgBig;    // 8 waves, 128x64 per wave, two waves per SIMD
+typedef GemmCfg<128, 128, 2, 2, 2, 0, 2> CfgMid;    // 4 waves, 64x64 per wave, two workgroups per CU
+typedef GemmCfg<64, 64, 2, 2, 2, 0, 2> CfgSmall;    // 4 waves, 32x32 per wave
 
 template <typename Cfg, int IN_DT, int OUT_DT>
 static hipError_t launch_cfg(const GemmArgs& a, hipStream_t st) {
@@ -294,7 +452,7 @@ static hipError_t launch_cfg(const GemmArgs& a, hipStream_t st) {
   int dev = 0;
   (void)hipGetDevice(&dev);
   auto kern = gemm_kernel<Cfg, IN_DT, OUT_DT>;
-  if (dev < 16 && !attr_set[dev]) {
+  if (dev >= 0 && dev < 16 && !attr_set[dev]) {
     hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, Cfg::LDS_BYTES);
     if (e != hipSuccess) return e;
     attr_set[dev] = true;
@@ -307,10 +465,10 @@ static hipError_t launch_cfg(const GemmArgs& a, hipStream_t st) {
 template <int IN_DT, int OUT_DT>
 static hipError_t launch_in_out(const GemmArgs& a, int tile, hipStream_t st) {
   if (tile == 0) {
-    // Pick the largest tile that still gives every CU work.
+    // Largest tile that still gives every CU a workgroup.
     const long big = (long)((a.M + 255) / 256) * ((a.N + 255) / 256);
     const long mid = (long)((a.M + 127) / 128) * ((a.N + 127) / 128);
-    tile = big >= 256 ? 3 : mid >= 128 ? 2 : 1;
+    tile = big >= 256 ? 3 : mid >= 256 ? 2 : 1;
   }
   if (tile == 3) return launch_cfg<CfgBig, IN_DT, OUT_DT>(a, st);
   if (tile == 2) return launch_cfg<CfgMid, IN_DT, OUT_DT>(a, st);
@@ -328,7 +486,8 @@ static hipError_t launch_in(const GemmArgs& a, int out_dt, int tile, hipStream_t
   return hipErrorInvalidValue;
 }
 
-// in_dt: element type of A and W; out_dt: element type of C/C2; tile: 0 auto, 1..3 fixed.
+// in_dt: element type of A and W; out_dt: element type of C/C2; tile: 0 auto, 1 = 64x64,
+// 2 = 128x128, 3 = 256x256 workgroup tile.
 hipError_t launch_gemm(GemmArgs a, int in_dt, int out_dt, int tile, hipStream_t st) {
   if (a.M <= 0 || a.N <= 0) return hipSuccess;
   const int esz = in_dt == DT_FP8 ? 1 : 2;
