@@ -95,22 +95,6 @@ __device__ __forceinline__ f32x16_t mfma_frag(const Frag<IN_DT>& w, const Frag<I
 }
 
 template <int OUT_DT>
-__device__ __forceinline__ void store4(void* base, long off, const float v[4]) {
-  if constexpr (OUT_DT == DT_F32) {
-    *reinterpret_cast<float4*>(reinterpret_cast<float*>(base) + off) = make_float4(v[0], v[1], v[2], v[3]);
-  } else if constexpr (OUT_DT == DT_BF16) {
-    uint2 p = make_uint2(pack_bf16x2(v[0], v[1]), pack_bf16x2(v[2], v[3]));
-    *reinterpret_cast<uint2*>(reinterpret_cast<uint16_t*>(base) + off) = p;
-  } else if constexpr (OUT_DT == DT_F16) {
-    uint2 p = make_uint2((uint32_t)f32_to_f16_bits(v[0]) | ((uint32_t)f32_to_f16_bits(v[1]) << 16),
-                         (uint32_t)f32_to_f16_bits(v[2]) | ((uint32_t)f32_to_f16_bits(v[3]) << 16));
-    *reinterpret_cast<uint2*>(reinterpret_cast<uint16_t*>(base) + off) = p;
-  } else {
-    *reinterpret_cast<uint32_t*>(reinterpret_cast<uint8_t*>(base) + off) = pack_fp8x4(v[0], v[1], v[2], v[3]);
-  }
-}
-
-template <int OUT_DT>
 __device__ __forceinline__ void store1(void* base, long off, float v) {
   if constexpr (OUT_DT == DT_F32) reinterpret_cast<float*>(base)[off] = v;
   else if constexpr (OUT_DT == DT_BF16) reinterpret_cast<uint16_t*>(base)[off] = f32_to_bf16_bits(v);
@@ -124,6 +108,197 @@ __device__ __forceinline__ void wave_lds_fence() {
   __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
   __builtin_amdgcn_wave_barrier();
   __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+}
+
+template <int OUT_DT>
+__device__ __forceinline__ void store8(void* base, long off, const float v[8]) {
+  if constexpr (OUT_DT == DT_F32) {
+    float4* p = reinterpret_cast<float4*>(reinterpret_cast<float*>(base) + off);
+    p[0] = make_float4(v[0], v[1], v[2], v[3]);
+    p[1] = make_float4(v[4], v[5], v[6], v[7]);
+  } else if constexpr (OUT_DT == DT_BF16) {
+    *reinterpret_cast<uint4*>(reinterpret_cast<uint16_t*>(base) + off) =
+        make_uint4(pack_bf16x2(v[0], v[1]), pack_bf16x2(v[2], v[3]), pack_bf16x2(v[4], v[5]), pack_bf16x2(v[6], v[7]));
+  } else if constexpr (OUT_DT == DT_F16) {
+    uint32_t w[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) w[i] = (uint32_t)f32_to_f16_bits(v[2 * i]) | ((uint32_t)f32_to_f16_bits(v[2 * i + 1]) << 16);
+    *reinterpret_cast<uint4*>(reinterpret_cast<uint16_t*>(base) + off) = make_uint4(w[0], w[1], w[2], w[3]);
+  } else {
+    *reinterpret_cast<uint2*>(reinterpret_cast<uint8_t*>(base) + off) =
+        make_uint2(pack_fp8x4(v[0], v[1], v[2], v[3]), pack_fp8x4(v[4], v[5], v[6], v[7]));
+  }
+}
+
+// Shared epilogue. acc[tn][tm][r] is output row m = mw0 + tm*32 + lr, column
+// n = nw0 + tn*32 + 8*(r/4) + 4*g + (r%4) (lr = lane%32, g = lane/32); sC is this wave's
+// private LDS patch of 32 x WN floats.
+//
+// Each 32 x WN strip of the wave tile goes through the patch (16-byte chunks XOR-swizzled by
+// row) so that a lane ends up with 8 consecutive columns of one row: stores, residual loads
+// and bias loads are 16-byte vectors (32 for fp32) and every store instruction writes whole
+// row segments. A lane keeps the same 8 columns for all rows, so its bias is loaded once. The
+// residual of strip t+1 is requested before strip t is processed (two register sets), which
+// takes its memory latency off the critical path; the activation is selected once per strip.
+template <int WM, int WN, int OUT_DT>
+__device__ __forceinline__ void gemm_epilogue(const GemmArgs& a, f32x16_t (&acc)[WN / 32][WM / 32], float* sC, int mw0, int nw0, int lane) {
+  constexpr int TM = WM / 32, TN = WN / 32, CH4 = WN / 4, CP = WN / 8, RSTEP = 64 / CP, ITERS = 32 / RSTEP;
+  const int lr = lane & 31, g = lane >> 5;
+  const int ec = lane % CP, er = lane / CP;
+  const int n = nw0 + ec * 8;
+  const bool n_ok = n < a.N;
+  const bool full = a.vec_ok && (n + 7 < a.N) && ((n < a.nsplit) == (n + 7 < a.nsplit));
+  float bias8[8];
+#pragma unroll
+  for (int e = 0; e < 8; ++e) bias8[e] = (a.bias && n + e < a.N) ? a.bias[n + e] : 0.f;
+  const int res_dt = a.res_dtype;
+  const float descale = a.descale, alpha = a.alpha;
+  float local_amax = 0.f;
+
+  // Raw residual bits, 16 bytes per step and set. 16-bit residuals use the two sets as a double
+  // buffer over strips; an fp32 residual (8 values = 32 bytes) uses both sets for the current
+  // strip (low and high half), i.e. it is fetched at the start of its own strip.
+  const bool res32 = res_dt == DT_F32;
+  uint4 rraw[2][ITERS];
+  auto load_res = [&](int tm, int set, int half) {
+#pragma unroll
+    for (int it = 0; it < ITERS; ++it) {
+      const int m = mw0 + tm * 32 + er + it * RSTEP;
+      uint4 val = make_uint4(0, 0, 0, 0);
+      if (m < a.M && n_ok) {
+        const long ro = (long)(a.res_rows > 0 ? m % a.res_rows : m) * a.ldr + n;
+        if (res32) {
+          const float* rp = reinterpret_cast<const float*>(a.res) + ro + 4 * half;
+          if (full) val = *reinterpret_cast<const uint4*>(rp);
+          else {
+            uint32_t w[4];
+#pragma unroll
+            for (int e = 0; e < 4; ++e) w[e] = (n + 4 * half + e < a.N) ? __float_as_uint(rp[e]) : 0u;
+            val = make_uint4(w[0], w[1], w[2], w[3]);
+          }
+        } else {
+          const uint16_t* rp = reinterpret_cast<const uint16_t*>(a.res) + ro;
+          if (full) val = *reinterpret_cast<const uint4*>(rp);
+          else {
+            uint32_t h[8];
+#pragma unroll
+            for (int e = 0; e < 8; ++e) h[e] = (n + e < a.N) ? (uint32_t)rp[e] : 0u;
+            val = make_uint4(h[0] | (h[1] << 16), h[2] | (h[3] << 16), h[4] | (h[5] << 16), h[6] | (h[7] << 16));
+          }
+        }
+      }
+      rraw[set][it] = val;
+    }
+  };
+  auto res_value = [&](int tm, int it, int e) -> float {
+    if (res32) {
+      const uint4 q = rraw[e >> 2][it];
+      const uint32_t w[4] = {q.x, q.y, q.z, q.w};
+      return __uint_as_float(w[e & 3]);
+    }
+    const uint4 q = rraw[tm & 1][it];
+    const uint32_t w[4] = {q.x, q.y, q.z, q.w};
+    const uint16_t h = (uint16_t)((e & 1) ? (w[e >> 1] >> 16) : (w[e >> 1] & 0xffff));
+    return res_dt == DT_F16 ? f16_bits_to_f32(h) : bf16_bits_to_f32(h);
+  };
+
+  if (a.res && !res32) load_res(0, 0, 0);
+  static_for<0, TM>([&](auto tmc) {
+    constexpr int tm = decltype(tmc)::value;
+    if (a.res) {
+      if (res32) { load_res(tm, 0, 0); load_res(tm, 1, 1); }
+      else if constexpr (tm + 1 < TM) load_res(tm + 1, (tm + 1) & 1, 0);
+    }
+#pragma unroll
+    for (int tn = 0; tn < TN; ++tn)
+#pragma unroll
+      for (int rq = 0; rq < 4; ++rq) {
+        const int chunk = tn * 8 + 2 * rq + g;
+        f32x4_t v4 = {acc[tn][tm][4 * rq], acc[tn][tm][4 * rq + 1], acc[tn][tm][4 * rq + 2], acc[tn][tm][4 * rq + 3]};
+        *reinterpret_cast<f32x4_t*>(sC + lr * WN + ((chunk ^ (lr & (CH4 - 1))) << 2)) = v4;
+      }
+    wave_lds_fence();
+    float v[ITERS][8];
+#pragma unroll
+    for (int it = 0; it < ITERS; ++it) {
+      const int r = er + it * RSTEP;
+      const int sw = r & (CH4 - 1);
+      const f32x4_t lo = *reinterpret_cast<const f32x4_t*>(sC + r * WN + (((2 * ec) ^ sw) << 2));
+      const f32x4_t hi = *reinterpret_cast<const f32x4_t*>(sC + r * WN + (((2 * ec + 1) ^ sw) << 2));
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        v[it][e] = fmaf(lo[e], descale, bias8[e]);
+        v[it][4 + e] = fmaf(hi[e], descale, bias8[4 + e]);
+      }
+    }
+    switch (a.act) {  // uniform
+      case ACT_GELU:
+#pragma unroll
+        for (int it = 0; it < ITERS; ++it)
+#pragma unroll
+          for (int e = 0; e < 8; ++e) v[it][e] = act_gelu(v[it][e]);
+        break;
+      case ACT_MISH:
+#pragma unroll
+        for (int it = 0; it < ITERS; ++it)
+#pragma unroll
+          for (int e = 0; e < 8; ++e) v[it][e] = act_mish(v[it][e]);
+        break;
+      case ACT_SWISH:
+#pragma unroll
+        for (int it = 0; it < ITERS; ++it)
+#pragma unroll
+          for (int e = 0; e < 8; ++e) v[it][e] = act_swish(v[it][e]);
+        break;
+      default: break;
+    }
+    if (a.res) {
+#pragma unroll
+      for (int it = 0; it < ITERS; ++it)
+#pragma unroll
+        for (int e = 0; e < 8; ++e) v[it][e] = fmaf(v[it][e], alpha, res_value(tm, it, e));
+    } else {
+#pragma unroll
+      for (int it = 0; it < ITERS; ++it)
+#pragma unroll
+        for (int e = 0; e < 8; ++e) v[it][e] *= alpha;
+    }
+    if (a.amax) {
+#pragma unroll
+      for (int it = 0; it < ITERS; ++it)
+#pragma unroll
+        for (int e = 0; e < 8; ++e)
+          if (mw0 + tm * 32 + er + it * RSTEP < a.M && n + e < a.N) local_amax = fmaxf(local_amax, fabsf(v[it][e]));
+    }
+    if constexpr (OUT_DT == DT_FP8) {
+      const float os = a.out_scale;
+#pragma unroll
+      for (int it = 0; it < ITERS; ++it)
+#pragma unroll
+        for (int e = 0; e < 8; ++e) v[it][e] *= os;
+    }
+#pragma unroll
+    for (int it = 0; it < ITERS; ++it) {
+      const int m = mw0 + tm * 32 + er + it * RSTEP;
+      if (m >= a.M || !n_ok) continue;
+      if (full) {
+        if (n < a.nsplit) store8<OUT_DT>(a.C, (long)m * a.ldc + n, v[it]);
+        else store8<OUT_DT>(a.C2, (long)m * a.ldc2 + (n - a.nsplit), v[it]);
+      } else {
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+          if (n + e >= a.N) continue;
+          if (n + e < a.nsplit) store1<OUT_DT>(a.C, (long)m * a.ldc + n + e, v[it][e]);
+          else store1<OUT_DT>(a.C2, (long)m * a.ldc2 + (n + e - a.nsplit), v[it][e]);
+        }
+      }
+    }
+    wave_lds_fence();
+  });
+  if (a.amax) {
+    local_amax = wave_max(local_amax);
+    if (lane == 0) atomic_amax(a.amax, local_amax);
+  }
 }
 
 template <typename Cfg, int IN_DT, int OUT_DT>
@@ -283,157 +458,165 @@ __global__ void __launch_bounds__(Cfg::NT, Cfg::MIN_WAVES) gemm_kernel(const Gem
     }
   }
 
-  // Epilogue. acc[tn][tm][r] is output row m = m0 + wm*WM + tm*32 + lr, column
-  // n = n0 + wn*WN + tn*32 + 8*(r/4) + 4*g + (r%4). Each wave passes its 32 x WN strip
-  // through a private LDS patch (16-byte chunks XOR-swizzled by row) so that every store
-  // instruction writes whole contiguous row segments. A lane keeps the same four columns
-  // for every row of the strip (64 lanes cover 64/CH rows x CH chunks per step), so its
-  // bias values are loaded once; IU steps are processed together so their LDS reads and
-  // residual loads overlap, and the activation is selected once per group, not per element.
-  constexpr int WN = Cfg::WN, CH = WN / 4, ITERS = (32 * CH) / 64, RSTEP = 64 / CH;
-  constexpr int IU = ITERS < 4 ? ITERS : 4;
-  float* sC = reinterpret_cast<float*>(smem) + wave * (32 * WN);
-  const int ec = lane % CH, er = lane / CH;
-  const int n = n0 + wn * WN + ec * 4;
-  const bool n_ok = n < a.N;
-  const bool full = a.vec_ok && (n + 3 < a.N) && !(n < a.nsplit && n + 3 >= a.nsplit);
-  float bias4[4] = {0.f, 0.f, 0.f, 0.f};
-  if (a.bias && n_ok) {
-#pragma unroll
-    for (int e = 0; e < 4; ++e) if (n + e < a.N) bias4[e] = a.bias[n + e];
-  }
-  const bool res_f32 = a.res_dtype == DT_F32, res_f16 = a.res_dtype == DT_F16;
-  const float descale = a.descale, alpha = a.alpha;
-  float local_amax = 0.f;
+  gemm_epilogue<Cfg::WM, Cfg::WN, OUT_DT>(a, acc, reinterpret_cast<float*>(smem) + wave * (32 * Cfg::WN),
+                                         m0 + wm * Cfg::WM, n0 + wn * Cfg::WN, lane);
+}
 
-  static_for<0, TM>([&](auto tmc) {
-    constexpr int tm = decltype(tmc)::value;
-#pragma unroll
-    for (int tn = 0; tn < TN; ++tn)
-#pragma unroll
-      for (int rq = 0; rq < 4; ++rq) {
-        const int chunk = tn * 8 + 2 * rq + g;
-        f32x4_t v4 = {acc[tn][tm][4 * rq], acc[tn][tm][4 * rq + 1], acc[tn][tm][4 * rq + 2], acc[tn][tm][4 * rq + 3]};
-        *reinterpret_cast<f32x4_t*>(sC + lr * WN + ((chunk ^ (lr & (CH - 1))) << 2)) = v4;
-      }
-    wave_lds_fence();
-#pragma unroll 1
-    for (int ito = 0; ito < ITERS; ito += IU) {
-      const int rbase = er + ito * RSTEP;
-      const int mbase = m0 + wm * Cfg::WM + tm * 32 + rbase;
-      float v[IU][4];
-      f32x4_t lv[IU];
-#pragma unroll
-      for (int it = 0; it < IU; ++it) {
-        const int r = rbase + it * RSTEP;
-        lv[it] = *reinterpret_cast<const f32x4_t*>(sC + r * WN + ((ec ^ (r & (CH - 1))) << 2));
-      }
-      float rv[IU][4];
-      if (a.res) {
-#pragma unroll
-        for (int it = 0; it < IU; ++it) {
-          const int m = mbase + it * RSTEP;
-#pragma unroll
-          for (int e = 0; e < 4; ++e) rv[it][e] = 0.f;
-          if (m < a.M && n_ok) {
-            const long ro = (long)(a.res_rows > 0 ? m % a.res_rows : m) * a.ldr + n;
-            if (res_f32) {
-              const float* rp = reinterpret_cast<const float*>(a.res) + ro;
-              if (full) { const float4 r4 = *reinterpret_cast<const float4*>(rp); rv[it][0] = r4.x; rv[it][1] = r4.y; rv[it][2] = r4.z; rv[it][3] = r4.w; }
-              else {
-#pragma unroll
-                for (int e = 0; e < 4; ++e) if (n + e < a.N) rv[it][e] = rp[e];
-              }
-            } else {
-              const uint16_t* rp = reinterpret_cast<const uint16_t*>(a.res) + ro;
-              uint16_t rb[4] = {0, 0, 0, 0};
-              if (full) {
-                const uint2 r2 = *reinterpret_cast<const uint2*>(rp);
-                rb[0] = (uint16_t)(r2.x & 0xffff); rb[1] = (uint16_t)(r2.x >> 16);
-                rb[2] = (uint16_t)(r2.y & 0xffff); rb[3] = (uint16_t)(r2.y >> 16);
-              } else {
-#pragma unroll
-                for (int e = 0; e < 4; ++e) if (n + e < a.N) rb[e] = rp[e];
-              }
-#pragma unroll
-              for (int e = 0; e < 4; ++e) rv[it][e] = res_f16 ? f16_bits_to_f32(rb[e]) : bf16_bits_to_f32(rb[e]);
-            }
-          }
-        }
-      }
-#pragma unroll
-      for (int it = 0; it < IU; ++it)
-#pragma unroll
-        for (int e = 0; e < 4; ++e) v[it][e] = fmaf(lv[it][e], descale, bias4[e]);
-      switch (a.act) {  // uniform
-        case ACT_GELU:
-#pragma unroll
-          for (int it = 0; it < IU; ++it)
-#pragma unroll
-            for (int e = 0; e < 4; ++e) v[it][e] = act_gelu(v[it][e]);
-          break;
-        case ACT_MISH:
-#pragma unroll
-          for (int it = 0; it < IU; ++it)
-#pragma unroll
-            for (int e = 0; e < 4; ++e) v[it][e] = act_mish(v[it][e]);
-          break;
-        case ACT_SWISH:
-#pragma unroll
-          for (int it = 0; it < IU; ++it)
-#pragma unroll
-            for (int e = 0; e < 4; ++e) v[it][e] = act_swish(v[it][e]);
-          break;
-        default: break;
-      }
-      if (a.res) {
-#pragma unroll
-        for (int it = 0; it < IU; ++it)
-#pragma unroll
-          for (int e = 0; e < 4; ++e) v[it][e] = fmaf(v[it][e], alpha, rv[it][e]);
-      } else {
-#pragma unroll
-        for (int it = 0; it < IU; ++it)
-#pragma unroll
-          for (int e = 0; e < 4; ++e) v[it][e] *= alpha;
-      }
-      if (a.amax) {
-#pragma unroll
-        for (int it = 0; it < IU; ++it)
-#pragma unroll
-          for (int e = 0; e < 4; ++e)
-            if (mbase + it * RSTEP < a.M && n + e < a.N) local_amax = fmaxf(local_amax, fabsf(v[it][e]));
-      }
-      if constexpr (OUT_DT == DT_FP8) {
-        const float os = a.out_scale;
-#pragma unroll
-        for (int it = 0; it < IU; ++it)
-#pragma unroll
-          for (int e = 0; e < 4; ++e) v[it][e] *= os;
-      }
-#pragma unroll
-      for (int it = 0; it < IU; ++it) {
-        const int m = mbase + it * RSTEP;
-        if (m >= a.M || !n_ok) continue;
-        if (full) {
-          if (n < a.nsplit) store4<OUT_DT>(a.C, (long)m * a.ldc + n, v[it]);
-          else store4<OUT_DT>(a.C2, (long)m * a.ldc2 + (n - a.nsplit), v[it]);
-        } else {
-#pragma unroll
-          for (int e = 0; e < 4; ++e) {
-            if (n + e >= a.N) continue;
-            if (n + e < a.nsplit) store1<OUT_DT>(a.C, (long)m * a.ldc + n + e, v[it][e]);
-            else store1<OUT_DT>(a.C2, (long)m * a.ldc2 + (n + e - a.nsplit), v[it][e]);
-          }
-        }
-      }
-    }
-    wave_lds_fence();
-  });
-  if (a.amax) {
-    local_amax = wave_max(local_amax);
-    if (lane == 0) atomic_amax(a.amax, local_amax);
+// ---- 256x256 tile fed by direct global->LDS loads through a 4-stage ring ------------------
+// The register-staged kernel above can only keep one K-slab in flight (the staging registers),
+// so a slab's loads must land within one slab of MFMA time. Here the loads bypass the
+// register file (global_load_lds_dwordx4: lane l of a wave-instruction writes LDS bytes
+// [base + 16l, base + 16l + 16)), stages are 64 bytes per row, and three stages are in
+// flight while the fourth is consumed. One barrier per stage.
+//  * A stage holds 256 weight rows then 256 activation rows of 64 bytes = 4 chunks; chunk c of
+//    row r sits at chunk c ^ dma_swizzle(r), which spreads any 16 consecutive rows read at one
+//    logical chunk over all 64 banks.
+//  * Wave w issues the loads for rows [64(w&3), +64) of the weight block (w < 4) or of the
+//    activation block (w >= 4): four wave-instructions of 16 rows x 64 bytes per stage; the
+//    swizzle is applied on the global side (which chunk a lane fetches).
+struct DmaCfg {
+  static constexpr int BM = 256, BN = 256, WGM = 2, WGN = 4, NW = 8, NT = 512;
+  static constexpr int WM = 128, WN = 64, TM = 4, TN = 2;
+  static constexpr int ROWB = 64, NSTAGE = 4;
+  static constexpr int STAGE_BYTES = (BM + BN) * ROWB;
+  static constexpr int EPI_BYTES = NW * 32 * WN * 4;
+  static constexpr int LDS_BYTES = NSTAGE * STAGE_BYTES > EPI_BYTES ? NSTAGE * STAGE_BYTES : EPI_BYTES;
+};
+
+__device__ __forceinline__ int dma_swizzle(int r) { return (((r >> 2) & 1) << 1) | (((r >> 1) ^ (r >> 3)) & 1); }
+
+// s_waitcnt with only vmcnt constrained (gfx9 encoding: vmcnt[3:0] | expcnt[6:4] | lgkmcnt[11:8] | vmcnt_hi[15:14]).
+template <int N>
+__device__ __forceinline__ void wait_vmcnt() {
+  __builtin_amdgcn_s_waitcnt((N & 0xF) | ((N >> 4) << 14) | (0x7 << 4) | (0xF << 8));
+}
+
+template <int IN_DT, int OUT_DT>
+__global__ void __launch_bounds__(DmaCfg::NT, 2) gemm_dma_kernel(const GemmArgs a, const uint8_t* zeros) {
+  using Cfg = DmaCfg;
+  constexpr int BM = Cfg::BM, BN = Cfg::BN, TM = Cfg::TM, TN = Cfg::TN, NSTAGE = Cfg::NSTAGE;
+  constexpr int ESZ = (IN_DT == DT_FP8) ? 1 : 2;
+  constexpr int KSTEPS = (IN_DT == DT_FP8) ? 1 : 2;  // MFMA k-steps per 64-byte stage
+  extern __shared__ __align__(16) uint8_t smem[];
+
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int wm = wave % Cfg::WGM, wn = wave / Cfg::WGM;
+  const int lr = lane & 31, g = lane >> 5;
+
+  const int tiles_n = (a.N + BN - 1) / BN;
+  const int nblk = gridDim.x;
+  int pid = blockIdx.x;
+  {
+    const int per = nblk >> 3;
+    if (pid < (per << 3)) pid = (pid & 7) * per + (pid >> 3);
   }
+  const int tile_m = pid / tiles_n, tile_n = pid - tile_m * tiles_n;
+  const int m0 = tile_m * BM, n0 = tile_n * BN;
+
+  const long kbytes = (long)a.K * ESZ;
+  const int nslab = (int)((kbytes + Cfg::ROWB - 1) / Cfg::ROWB);
+  const long kmax = kbytes - 16;
+
+  // Loader role of this wave.
+  const bool loads_a = wave >= 4;
+  const int rbase = (wave & 3) * 64;
+  const uint8_t* gptr[4];
+  int kchunk[4];
+#pragma unroll
+  for (int j = 0; j < 4; ++j) {
+    const int r = rbase + 16 * j + (lane >> 2);
+    const int c = (lane & 3) ^ dma_swizzle(r);
+    kchunk[j] = c << 4;
+    if (loads_a) {
+      int gm = m0 + r;
+      gm = gm < a.M ? gm : a.M - 1;
+      gptr[j] = reinterpret_cast<const uint8_t*>(a.A) + (long)gm * a.lda * ESZ + kchunk[j];
+    } else {
+      int gn = n0 + r;
+      gn = gn < a.N ? gn : a.N - 1;
+      gptr[j] = reinterpret_cast<const uint8_t*>(a.W) + (long)gn * a.ldw * ESZ + kchunk[j];
+    }
+  }
+  const int lds_row0 = (loads_a ? BN : 0) + rbase;  // first stage row this wave fills
+  auto issue = [&](int slab) {
+    uint8_t* st = smem + (slab % NSTAGE) * Cfg::STAGE_BYTES + lds_row0 * Cfg::ROWB;
+    const long kb = (long)slab * Cfg::ROWB;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const uint8_t* src = (kb + kchunk[j] <= kmax) ? gptr[j] + kb : zeros;
+      __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)src,
+                                       (__attribute__((address_space(3))) void*)(st + j * 16 * Cfg::ROWB), 16, 0, 0);
+    }
+  };
+
+  f32x16_t acc[TN][TM];
+#pragma unroll
+  for (int i = 0; i < TN; ++i)
+#pragma unroll
+    for (int j = 0; j < TM; ++j)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
+
+  int wrow_off[TN], wrow_sw[TN], arow_off[TM], arow_sw[TM];
+#pragma unroll
+  for (int tn = 0; tn < TN; ++tn) {
+    const int wr = wn * Cfg::WN + tn * 32 + lr;
+    wrow_off[tn] = wr * Cfg::ROWB;
+    wrow_sw[tn] = dma_swizzle(wr);
+  }
+#pragma unroll
+  for (int tm = 0; tm < TM; ++tm) {
+    const int ar = wm * Cfg::WM + tm * 32 + lr;
+    arow_off[tm] = (BN + ar) * Cfg::ROWB;
+    arow_sw[tm] = dma_swizzle(ar);
+  }
+
+#pragma unroll
+  for (int s0 = 0; s0 < NSTAGE - 1; ++s0)
+    if (s0 < nslab) issue(s0);
+
+  for (int slab = 0; slab < nslab; ++slab) {
+    // Loads still allowed in flight behind this slab's: 4 per later slab already issued.
+    const int ahead = nslab - 1 - slab;
+    if (ahead >= 2) wait_vmcnt<8>();
+    else if (ahead == 1) wait_vmcnt<4>();
+    else wait_vmcnt<0>();
+    __syncthreads();
+    if (slab + NSTAGE - 1 < nslab) issue(slab + NSTAGE - 1);
+    const uint8_t* st = smem + (slab % NSTAGE) * Cfg::STAGE_BYTES;
+#pragma unroll
+    for (int ks = 0; ks < KSTEPS; ++ks) {
+      Frag<IN_DT> wf[TN], xf[TM];
+#pragma unroll
+      for (int tn = 0; tn < TN; ++tn) {
+        const uint8_t* row = st + wrow_off[tn];
+        if constexpr (IN_DT == DT_FP8) {
+          wf[tn].lo = *reinterpret_cast<const i32x4_t*>(row + (((2 * g) ^ wrow_sw[tn]) << 4));
+          wf[tn].hi = *reinterpret_cast<const i32x4_t*>(row + (((2 * g + 1) ^ wrow_sw[tn]) << 4));
+        } else {
+          wf[tn].lo = *reinterpret_cast<const i32x4_t*>(row + (((2 * ks + g) ^ wrow_sw[tn]) << 4));
+        }
+      }
+#pragma unroll
+      for (int tm = 0; tm < TM; ++tm) {
+        const uint8_t* row = st + arow_off[tm];
+        if constexpr (IN_DT == DT_FP8) {
+          xf[tm].lo = *reinterpret_cast<const i32x4_t*>(row + (((2 * g) ^ arow_sw[tm]) << 4));
+          xf[tm].hi = *reinterpret_cast<const i32x4_t*>(row + (((2 * g + 1) ^ arow_sw[tm]) << 4));
+        } else {
+          xf[tm].lo = *reinterpret_cast<const i32x4_t*>(row + (((2 * ks + g) ^ arow_sw[tm]) << 4));
+        }
+      }
+#pragma unroll
+      for (int tn = 0; tn < TN; ++tn)
+#pragma unroll
+        for (int tm = 0; tm < TM; ++tm) acc[tn][tm] = mfma_frag<IN_DT>(wf[tn], xf[tm], acc[tn][tm]);
+    }
+  }
+  __syncthreads();  // every wave is done with the ring before it becomes epilogue scratch
+
+  gemm_epilogue<Cfg::WM, Cfg::WN, OUT_DT>(a, acc, reinterpret_cast<float*>(smem) + wave * (32 * Cfg::WN),
+                                         m0 + wm * Cfg::WM, n0 + wn * Cfg::WN, lane);
 }
 
 // ---- host-side dispatch -------------------------------------------------------------
@@ -462,6 +645,42 @@ static hipError_t launch_cfg(const GemmArgs& a, hipStream_t st) {
   return hipGetLastError();
 }
 
+// One 256-byte block of zeros per device: the source of K-tail chunks for the direct-to-LDS loads.
+static const uint8_t* device_zeros(hipError_t* err) {
+  static uint8_t* z[16] = {};
+  int dev = 0;
+  *err = hipGetDevice(&dev);
+  if (*err != hipSuccess || dev < 0 || dev >= 16) { if (*err == hipSuccess) *err = hipErrorInvalidDevice; return nullptr; }
+  if (!z[dev]) {
+    uint8_t* p = nullptr;
+    *err = hipMalloc((void**)&p, 256);
+    if (*err != hipSuccess) return nullptr;
+    *err = hipMemset(p, 0, 256);
+    if (*err != hipSuccess) { (void)hipFree(p); return nullptr; }
+    z[dev] = p;
+  }
+  return z[dev];
+}
+
+template <int IN_DT, int OUT_DT>
+static hipError_t launch_dma(const GemmArgs& a, hipStream_t st) {
+  static bool attr_set[16] = {};
+  hipError_t e = hipSuccess;
+  const uint8_t* zeros = device_zeros(&e);
+  if (!zeros) return e;
+  int dev = 0;
+  (void)hipGetDevice(&dev);
+  auto kern = gemm_dma_kernel<IN_DT, OUT_DT>;
+  if (!attr_set[dev]) {
+    e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, DmaCfg::LDS_BYTES);
+    if (e != hipSuccess) return e;
+    attr_set[dev] = true;
+  }
+  const int tiles = ((a.M + DmaCfg::BM - 1) / DmaCfg::BM) * ((a.N + DmaCfg::BN - 1) / DmaCfg::BN);
+  hipLaunchKernelGGL(kern, dim3(tiles), dim3(DmaCfg::NT), DmaCfg::LDS_BYTES, st, a, zeros);
+  return hipGetLastError();
+}
+
 template <int IN_DT, int OUT_DT>
 static hipError_t launch_in_out(const GemmArgs& a, int tile, hipStream_t st) {
   if (tile == 0) {
@@ -470,6 +689,7 @@ static hipError_t launch_in_out(const GemmArgs& a, int tile, hipStream_t st) {
     const long mid = (long)((a.M + 127) / 128) * ((a.N + 127) / 128);
     tile = big >= 256 ? 3 : mid >= 256 ? 2 : 1;
   }
+  if (tile == 4) return launch_dma<IN_DT, OUT_DT>(a, st);
   if (tile == 3) return launch_cfg<CfgBig, IN_DT, OUT_DT>(a, st);
   if (tile == 2) return launch_cfg<CfgMid, IN_DT, OUT_DT>(a, st);
   return launch_cfg<CfgSmall, IN_DT, OUT_DT>(a, st);
@@ -497,14 +717,13 @@ hipError_t launch_gemm(GemmArgs a, int in_dt, int out_dt, int tile, hipStream_t 
       (reinterpret_cast<uintptr_t>(a.A) & 15) || (reinterpret_cast<uintptr_t>(a.W) & 15))
     return hipErrorInvalidValue;
   if (a.nsplit <= 0 || a.nsplit > a.N || !a.C2) { a.nsplit = a.N; a.C2 = a.C; a.ldc2 = a.ldc; }
-  const int osz = dtype_size(out_dt);
-  const int w = 4;  // elements per vector access
-  bool ok = (a.ldc % w == 0) && (reinterpret_cast<uintptr_t>(a.C) % (osz * w) == 0) &&
-            (a.ldc2 % w == 0) && (reinterpret_cast<uintptr_t>(a.C2) % (osz * w) == 0) && (a.nsplit % w == 0 || a.nsplit == a.N);
-  if (a.res) {
-    const int rsz = dtype_size(a.res_dtype);
-    ok = ok && (a.ldr % w == 0) && (reinterpret_cast<uintptr_t>(a.res) % (rsz * w) == 0);
-  }
+  // 8-element vector accesses along N: row strides in multiples of 8 elements, bases aligned to
+  // 16 bytes (the fp32 paths use two 16-byte accesses).
+  const int w = 8;
+  auto al16 = [](const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; };
+  bool ok = (a.ldc % w == 0) && al16(a.C) && (a.ldc2 % w == 0) && al16(a.C2) && (a.nsplit % w == 0 || a.nsplit == a.N);
+  if (out_dt == DT_FP8) ok = ok && (reinterpret_cast<uintptr_t>(a.C) & 7) == 0;
+  if (a.res) ok = ok && (a.ldr % w == 0) && al16(a.res);
   a.vec_ok = ok ? 1 : 0;
   switch (in_dt) {
     case DT_BF16: return launch_in<DT_BF16>(a, out_dt, tile, st);

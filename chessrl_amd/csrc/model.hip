@@ -43,7 +43,7 @@ Model::Model(const crl_model_config& c) : cfg(c) {
   if (cfg.smolgen_hidden == 0) cfg.smolgen_hidden = 256;
   if (cfg.smolgen_gen == 0) cfg.smolgen_gen = 256;
   if (cfg.head_dtype != DT_F16) cfg.head_dtype = DT_BF16;
-  if (cfg.micro_batch <= 0) cfg.micro_batch = 1024;
+  if (cfg.micro_batch <= 0) cfg.micro_batch = 4096;
   vocab = cfg.arch == CRL_ARCH_BT4CLASS ? VOCAB_LEELA : VOCAB_RL;
   const long C = cfg.d_model, F = cfg.d_ff, L = cfg.n_layer, H = cfg.n_head;
   auto add = [&](const std::string& k, long n) { expected.push_back({k, n}); };

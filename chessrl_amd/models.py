@@ -314,11 +314,58 @@ class _ModelBase:
             pol, _ = masked_softmax(pol, legal_mask, T)
         return pol, wdl
 
+    def graphed_evaluator(self, batch, T=1.0, device="cuda"):
+        """Leaf evaluation for a fixed batch size captured in a HIP graph (launch-bound small batches)."""
+        return GraphedEvaluator(self, batch, T, device)
+
     def _sample(self, logits_row, mask_row, T):
         probs, am = masked_softmax(logits_row, mask_row, T, want_probs=True)
         if T == 0:
             return int(am.item()), probs
         return int(torch.multinomial(probs, num_samples=1).item()), probs
+
+
+class GraphedEvaluator:
+    """forward + legal-masked softmax for one fixed batch size, recorded once into a HIP graph and
+    replayed per call. The ~200 kernel launches of a forward pass dominate the latency of small
+    batches (MCTS leaf evaluation); a replay issues them as one graph launch. The library calls
+    record no memset nodes (flags and scratch are cleared by kernels)."""
+
+    def __init__(self, model, batch, T=1.0, device="cuda"):
+        eng = model._engine
+        if not eng.ready:
+            eng.finalize()
+        self.batch, self.T = batch, float(T)
+        self.planes = torch.zeros((batch, 64, 19), dtype=torch.float32, device=device)
+        self.mask = torch.ones((batch, eng.vocab), dtype=torch.uint8, device=device)
+        self.policy = torch.empty((batch, eng.vocab), dtype=torch.float32, device=device)
+        self.probs = torch.empty_like(self.policy)
+        self.argmax = torch.empty((batch,), dtype=torch.int32, device=device)
+        self.wdl = torch.empty((batch, 3), dtype=torch.float32, device=device) if eng.cfg.arch != _lib.ARCH_GPT64 else None
+        self._eng = eng
+        self._run()                      # eager warm-up: allocates the workspace outside the capture
+        torch.cuda.synchronize()
+        self.graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(self.graph):
+            self._run()
+
+    def _run(self):
+        self._eng.forward(self.planes, out_policy=self.policy, out_wdl=self.wdl)
+        V = self._eng.vocab
+        check(lib().crl_masked_softmax(_ptr(self.policy), V, _ptr(self.mask), V, _ptr(self.probs), V, _ptr(self.argmax),
+                                       self.batch, V, self.T, _stream_ptr()), "crl_masked_softmax")
+
+    @torch.no_grad()
+    def __call__(self, planes, legal_mask=None):
+        """planes [batch,8,8,19] on the GPU -> (probs [batch,V], wdl logits [batch,3] or None, argmax [batch]).
+        The returned tensors are the evaluator's own buffers and are overwritten by the next call."""
+        self.planes.copy_(planes.reshape(self.batch, 64, 19))
+        if legal_mask is not None:
+            self.mask.copy_(legal_mask)
+        else:
+            self.mask.fill_(1)
+        self.graph.replay()
+        return self.probs, self.wdl, self.argmax
 
 
 @dataclass

@@ -155,3 +155,20 @@ def test_compact_input_equals_planes(cuda):
     p2, w2 = m._engine.forward_compact(torch.from_numpy(ids).to(cuda), torch.from_numpy(flags).to(cuda))
     assert torch.equal(w1, w2), (w1 - w2).abs().max()
     assert torch.equal(p1, p2), (p1 - p2).abs().max()
+
+
+def test_graphed_evaluator_replays_match_eager(cuda):
+    """A captured forward + masked softmax must reproduce the eager result on every replay, with
+    eager work and synchronisations in between."""
+    m = models.BT4Class(2, 256, 384, 8)
+    ge = m.graphed_evaluator(16, T=1.0)
+    for seed in (11, 12, 13, 14):
+        r = board.random_positions(seed, 16, masks_leela=True)
+        planes, mask = torch.from_numpy(r["planes"]).to(cuda), torch.from_numpy(r["masks_leela"]).to(cuda)
+        probs, wdl, am = ge(planes, mask)
+        probs, wdl, am = probs.clone(), wdl.clone(), am.clone()
+        torch.cuda.synchronize()
+        eprobs, ewdl = m.evaluate(planes, legal_mask=mask, T=1.0, want_probs=True)
+        torch.cuda.synchronize()
+        assert torch.equal(probs, eprobs) and torch.equal(wdl, ewdl)
+        assert torch.equal(am.long(), eprobs.argmax(-1))
