@@ -462,28 +462,35 @@ __global__ void __launch_bounds__(Cfg::NT, Cfg::MIN_WAVES) gemm_kernel(const Gem
                                          m0 + wm * Cfg::WM, n0 + wn * Cfg::WN, lane);
 }
 
-// ---- 256x256 tile fed by direct global->LDS loads through a 4-stage ring ------------------
-// The register-staged kernel above can only keep one K-slab in flight (the staging registers),
-// so a slab's loads must land within one slab of MFMA time. Here the loads bypass the
-// register file (global_load_lds_dwordx4: lane l of a wave-instruction writes LDS bytes
-// [base + 16l, base + 16l + 16)), stages are 64 bytes per row, and three stages are in
-// flight while the fourth is consumed. One barrier per stage.
-//  * A stage holds 256 weight rows then 256 activation rows of 64 bytes = 4 chunks; chunk c of
-//    row r sits at chunk c ^ dma_swizzle(r), which spreads any 16 consecutive rows read at one
-//    logical chunk over all 64 banks.
+// ---- 256x256 tile fed by direct global->LDS loads ------------------------------------------
+// The loads bypass the register file (global_load_lds_dwordx4: lane l of a wave-instruction
+// writes LDS bytes [base + 16l, base + 16l + 16)), which frees the 32 staging registers and the
+// LDS store instructions of the register-staged kernel. The kernel is written for a ring of
+// NSTAGE stages of ROWB bytes per row; the instantiated form uses 128-byte rows and two stages
+// (one barrier per 128 bytes of K): a 4-stage ring of 64-byte rows kept three stages in flight
+// but paid twice the barriers and measured slower.
+//  * A stage holds 256 weight rows then 256 activation rows; chunk c of row r sits at chunk
+//    c ^ swizzle(r) (the same XOR pattern as above for 8 chunks per row).
 //  * Wave w issues the loads for rows [64(w&3), +64) of the weight block (w < 4) or of the
-//    activation block (w >= 4): four wave-instructions of 16 rows x 64 bytes per stage; the
-//    swizzle is applied on the global side (which chunk a lane fetches).
-struct DmaCfg {
+//    activation block (w >= 4); the swizzle is applied on the global side (which chunk a lane
+//    fetches). A K tail is fetched from a block of zeros.
+template <int ROWB_, int NSTAGE_>
+struct DmaCfgT {
   static constexpr int BM = 256, BN = 256, WGM = 2, WGN = 4, NW = 8, NT = 512;
   static constexpr int WM = 128, WN = 64, TM = 4, TN = 2;
-  static constexpr int ROWB = 64, NSTAGE = 4;
+  static constexpr int ROWB = ROWB_, NSTAGE = NSTAGE_;
+  static constexpr int CHUNKS = ROWB / 16;            // 16-byte chunks per stage row
+  static constexpr int ROWS_PER_INSTR = 64 / CHUNKS;  // rows one wave-instruction fills
+  static constexpr int LOADS = 64 / ROWS_PER_INSTR;   // wave-instructions per wave and stage (64 rows each)
   static constexpr int STAGE_BYTES = (BM + BN) * ROWB;
   static constexpr int EPI_BYTES = NW * 32 * WN * 4;
   static constexpr int LDS_BYTES = NSTAGE * STAGE_BYTES > EPI_BYTES ? NSTAGE * STAGE_BYTES : EPI_BYTES;
 };
+typedef DmaCfgT<128, 2> DmaCfg2;     // 128-byte rows, 2 stages (one in flight), half as many barriers
 
 __device__ __forceinline__ int dma_swizzle(int r) { return (((r >> 2) & 1) << 1) | (((r >> 1) ^ (r >> 3)) & 1); }
+template <int CHUNKS>
+__device__ __forceinline__ int dma_sw(int r) { return CHUNKS == 4 ? dma_swizzle(r) : lds_swizzle(r); }
 
 // s_waitcnt with only vmcnt constrained (gfx9 encoding: vmcnt[3:0] | expcnt[6:4] | lgkmcnt[11:8] | vmcnt_hi[15:14]).
 template <int N>
@@ -491,12 +498,11 @@ __device__ __forceinline__ void wait_vmcnt() {
   __builtin_amdgcn_s_waitcnt((N & 0xF) | ((N >> 4) << 14) | (0x7 << 4) | (0xF << 8));
 }
 
-template <int IN_DT, int OUT_DT>
-__global__ void __launch_bounds__(DmaCfg::NT, 2) gemm_dma_kernel(const GemmArgs a, const uint8_t* zeros) {
-  using Cfg = DmaCfg;
-  constexpr int BM = Cfg::BM, BN = Cfg::BN, TM = Cfg::TM, TN = Cfg::TN, NSTAGE = Cfg::NSTAGE;
+template <typename Cfg, int IN_DT, int OUT_DT>
+__global__ void __launch_bounds__(Cfg::NT, 2) gemm_dma_kernel(const GemmArgs a, const uint8_t* zeros) {
+  constexpr int BM = Cfg::BM, BN = Cfg::BN, TM = Cfg::TM, TN = Cfg::TN, NSTAGE = Cfg::NSTAGE, LOADS = Cfg::LOADS;
   constexpr int ESZ = (IN_DT == DT_FP8) ? 1 : 2;
-  constexpr int KSTEPS = (IN_DT == DT_FP8) ? 1 : 2;  // MFMA k-steps per 64-byte stage
+  constexpr int KSTEPS = Cfg::ROWB / ((IN_DT == DT_FP8) ? 64 : 32);  // MFMA k-steps per stage
   extern __shared__ __align__(16) uint8_t smem[];
 
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
@@ -520,12 +526,12 @@ __global__ void __launch_bounds__(DmaCfg::NT, 2) gemm_dma_kernel(const GemmArgs 
   // Loader role of this wave.
   const bool loads_a = wave >= 4;
   const int rbase = (wave & 3) * 64;
-  const uint8_t* gptr[4];
-  int kchunk[4];
+  const uint8_t* gptr[LOADS];
+  int kchunk[LOADS];
 #pragma unroll
-  for (int j = 0; j < 4; ++j) {
-    const int r = rbase + 16 * j + (lane >> 2);
-    const int c = (lane & 3) ^ dma_swizzle(r);
+  for (int j = 0; j < LOADS; ++j) {
+    const int r = rbase + Cfg::ROWS_PER_INSTR * j + lane / Cfg::CHUNKS;
+    const int c = (lane % Cfg::CHUNKS) ^ dma_sw<Cfg::CHUNKS>(r);
     kchunk[j] = c << 4;
     if (loads_a) {
       int gm = m0 + r;
@@ -542,10 +548,10 @@ __global__ void __launch_bounds__(DmaCfg::NT, 2) gemm_dma_kernel(const GemmArgs 
     uint8_t* st = smem + (slab % NSTAGE) * Cfg::STAGE_BYTES + lds_row0 * Cfg::ROWB;
     const long kb = (long)slab * Cfg::ROWB;
 #pragma unroll
-    for (int j = 0; j < 4; ++j) {
+    for (int j = 0; j < LOADS; ++j) {
       const uint8_t* src = (kb + kchunk[j] <= kmax) ? gptr[j] + kb : zeros;
       __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)src,
-                                       (__attribute__((address_space(3))) void*)(st + j * 16 * Cfg::ROWB), 16, 0, 0);
+                                       (__attribute__((address_space(3))) void*)(st + j * 1024), 16, 0, 0);
     }
   };
 
@@ -562,24 +568,47 @@ __global__ void __launch_bounds__(DmaCfg::NT, 2) gemm_dma_kernel(const GemmArgs 
   for (int tn = 0; tn < TN; ++tn) {
     const int wr = wn * Cfg::WN + tn * 32 + lr;
     wrow_off[tn] = wr * Cfg::ROWB;
-    wrow_sw[tn] = dma_swizzle(wr);
+    wrow_sw[tn] = dma_sw<Cfg::CHUNKS>(wr);
   }
 #pragma unroll
   for (int tm = 0; tm < TM; ++tm) {
     const int ar = wm * Cfg::WM + tm * 32 + lr;
     arow_off[tm] = (BN + ar) * Cfg::ROWB;
-    arow_sw[tm] = dma_swizzle(ar);
+    arow_sw[tm] = dma_sw<Cfg::CHUNKS>(ar);
   }
+
+  auto read_frags = [&](Frag<IN_DT> (&wf)[TN], Frag<IN_DT> (&xf)[TM], const uint8_t* st, int ks) {
+#pragma unroll
+    for (int tn = 0; tn < TN; ++tn) {
+      const uint8_t* row = st + wrow_off[tn];
+      if constexpr (IN_DT == DT_FP8) {
+        wf[tn].lo = *reinterpret_cast<const i32x4_t*>(row + (((4 * ks + 2 * g) ^ wrow_sw[tn]) << 4));
+        wf[tn].hi = *reinterpret_cast<const i32x4_t*>(row + (((4 * ks + 2 * g + 1) ^ wrow_sw[tn]) << 4));
+      } else {
+        wf[tn].lo = *reinterpret_cast<const i32x4_t*>(row + (((2 * ks + g) ^ wrow_sw[tn]) << 4));
+      }
+    }
+#pragma unroll
+    for (int tm = 0; tm < TM; ++tm) {
+      const uint8_t* row = st + arow_off[tm];
+      if constexpr (IN_DT == DT_FP8) {
+        xf[tm].lo = *reinterpret_cast<const i32x4_t*>(row + (((4 * ks + 2 * g) ^ arow_sw[tm]) << 4));
+        xf[tm].hi = *reinterpret_cast<const i32x4_t*>(row + (((4 * ks + 2 * g + 1) ^ arow_sw[tm]) << 4));
+      } else {
+        xf[tm].lo = *reinterpret_cast<const i32x4_t*>(row + (((2 * ks + g) ^ arow_sw[tm]) << 4));
+      }
+    }
+  };
 
 #pragma unroll
   for (int s0 = 0; s0 < NSTAGE - 1; ++s0)
     if (s0 < nslab) issue(s0);
 
   for (int slab = 0; slab < nslab; ++slab) {
-    // Loads still allowed in flight behind this slab's: 4 per later slab already issued.
+    // Loads still allowed in flight behind this slab's: LOADS per later slab already issued.
     const int ahead = nslab - 1 - slab;
-    if (ahead >= 2) wait_vmcnt<8>();
-    else if (ahead == 1) wait_vmcnt<4>();
+    if (NSTAGE >= 4 && ahead >= 2) wait_vmcnt<2 * LOADS>();
+    else if (NSTAGE >= 3 && ahead == 1) wait_vmcnt<LOADS>();
     else wait_vmcnt<0>();
     __syncthreads();
     if (slab + NSTAGE - 1 < nslab) issue(slab + NSTAGE - 1);
@@ -587,32 +616,14 @@ __global__ void __launch_bounds__(DmaCfg::NT, 2) gemm_dma_kernel(const GemmArgs 
 #pragma unroll
     for (int ks = 0; ks < KSTEPS; ++ks) {
       Frag<IN_DT> wf[TN], xf[TM];
-#pragma unroll
-      for (int tn = 0; tn < TN; ++tn) {
-        const uint8_t* row = st + wrow_off[tn];
-        if constexpr (IN_DT == DT_FP8) {
-          wf[tn].lo = *reinterpret_cast<const i32x4_t*>(row + (((2 * g) ^ wrow_sw[tn]) << 4));
-          wf[tn].hi = *reinterpret_cast<const i32x4_t*>(row + (((2 * g + 1) ^ wrow_sw[tn]) << 4));
-        } else {
-          wf[tn].lo = *reinterpret_cast<const i32x4_t*>(row + (((2 * ks + g) ^ wrow_sw[tn]) << 4));
-        }
-      }
-#pragma unroll
-      for (int tm = 0; tm < TM; ++tm) {
-        const uint8_t* row = st + arow_off[tm];
-        if constexpr (IN_DT == DT_FP8) {
-          xf[tm].lo = *reinterpret_cast<const i32x4_t*>(row + (((2 * g) ^ arow_sw[tm]) << 4));
-          xf[tm].hi = *reinterpret_cast<const i32x4_t*>(row + (((2 * g + 1) ^ arow_sw[tm]) << 4));
-        } else {
-          xf[tm].lo = *reinterpret_cast<const i32x4_t*>(row + (((2 * ks + g) ^ arow_sw[tm]) << 4));
-        }
-      }
+      read_frags(wf, xf, st, ks);
 #pragma unroll
       for (int tn = 0; tn < TN; ++tn)
 #pragma unroll
         for (int tm = 0; tm < TM; ++tm) acc[tn][tm] = mfma_frag<IN_DT>(wf[tn], xf[tm], acc[tn][tm]);
     }
   }
+
   __syncthreads();  // every wave is done with the ring before it becomes epilogue scratch
 
   gemm_epilogue<Cfg::WM, Cfg::WN, OUT_DT>(a, acc, reinterpret_cast<float*>(smem) + wave * (32 * Cfg::WN),
@@ -621,11 +632,13 @@ __global__ void __launch_bounds__(DmaCfg::NT, 2) gemm_dma_kernel(const GemmArgs 
 
 // ---- host-side dispatch -------------------------------------------------------------
 //                 BM   BN  WGM WGN stages frag_db min_waves
-// Measured on MI355X (M=65536, K=1024..8192): the 8-wave 256x256 tile (two waves per SIMD
-// covering each other's LDS and barrier stalls) beats the 4-wave 256x256 tile with
-// double-buffered fragments, the single-stage 256x128 tile and the 128x128 tile for
-// every trunk shape in both fp8 and bf16.
-typedef GemmCfg<256, 256, 2, 4, 2, 0, 2> CfgBig;    // 8 waves, 128x64 per wave, two waves per SIMD
+// Measured on MI355X (M=65536, N=1024..3072, K=1024..8192, fp8 and bf16, same job): the 256x256
+// tile fed by direct-to-LDS loads with 128-byte rows and two stages (DmaCfg2) is 10-20 % faster
+// than the same 8-wave tile with register staging; the 4-wave 256x256 tile (one wave per SIMD,
+// with or without double-buffered fragments), a 256x128 single-stage tile at two workgroups per
+// CU, a 4-stage ring of 64-byte rows (twice the barriers) and a persistent
+// one-workgroup-per-CU loop (epilogue stores of tile t delay the first slab of tile t+1 because
+// loads and stores share vmcnt) were all slower. The register-staged kernel serves the small tiles.
 typedef GemmCfg<128, 128, 2, 2, 2, 0, 2> CfgMid;    // 4 waves, 64x64 per wave, two workgroups per CU
 typedef GemmCfg<64, 64, 2, 2, 2, 0, 2> CfgSmall;    // 4 waves, 32x32 per wave
 
@@ -662,7 +675,7 @@ static const uint8_t* device_zeros(hipError_t* err) {
   return z[dev];
 }
 
-template <int IN_DT, int OUT_DT>
+template <typename DCfg, int IN_DT, int OUT_DT>
 static hipError_t launch_dma(const GemmArgs& a, hipStream_t st) {
   static bool attr_set[16] = {};
   hipError_t e = hipSuccess;
@@ -670,14 +683,14 @@ static hipError_t launch_dma(const GemmArgs& a, hipStream_t st) {
   if (!zeros) return e;
   int dev = 0;
   (void)hipGetDevice(&dev);
-  auto kern = gemm_dma_kernel<IN_DT, OUT_DT>;
+  auto kern = gemm_dma_kernel<DCfg, IN_DT, OUT_DT>;
   if (!attr_set[dev]) {
-    e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, DmaCfg::LDS_BYTES);
+    e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, DCfg::LDS_BYTES);
     if (e != hipSuccess) return e;
     attr_set[dev] = true;
   }
-  const int tiles = ((a.M + DmaCfg::BM - 1) / DmaCfg::BM) * ((a.N + DmaCfg::BN - 1) / DmaCfg::BN);
-  hipLaunchKernelGGL(kern, dim3(tiles), dim3(DmaCfg::NT), DmaCfg::LDS_BYTES, st, a, zeros);
+  const int tiles = ((a.M + DCfg::BM - 1) / DCfg::BM) * ((a.N + DCfg::BN - 1) / DCfg::BN);
+  hipLaunchKernelGGL(kern, dim3(tiles), dim3(DCfg::NT), DCfg::LDS_BYTES, st, a, zeros);
   return hipGetLastError();
 }
 
@@ -689,8 +702,7 @@ static hipError_t launch_in_out(const GemmArgs& a, int tile, hipStream_t st) {
     const long mid = (long)((a.M + 127) / 128) * ((a.N + 127) / 128);
     tile = big >= 256 ? 3 : mid >= 256 ? 2 : 1;
   }
-  if (tile == 4) return launch_dma<IN_DT, OUT_DT>(a, st);
-  if (tile == 3) return launch_cfg<CfgBig, IN_DT, OUT_DT>(a, st);
+  if (tile == 3) return launch_dma<DmaCfg2, IN_DT, OUT_DT>(a, st);
   if (tile == 2) return launch_cfg<CfgMid, IN_DT, OUT_DT>(a, st);
   return launch_cfg<CfgSmall, IN_DT, OUT_DT>(a, st);
 }
@@ -707,7 +719,7 @@ static hipError_t launch_in(const GemmArgs& a, int out_dt, int tile, hipStream_t
 }
 
 // in_dt: element type of A and W; out_dt: element type of C/C2; tile: 0 auto, 1 = 64x64,
-// 2 = 128x128, 3 = 256x256 workgroup tile.
+// 2 = 128x128, 3 = 256x256 (direct-to-LDS loads).
 hipError_t launch_gemm(GemmArgs a, int in_dt, int out_dt, int tile, hipStream_t st) {
   if (a.M <= 0 || a.N <= 0) return hipSuccess;
   const int esz = in_dt == DT_FP8 ? 1 : 2;
