@@ -218,17 +218,17 @@ int crl_layernorm(const void* x, int64_t ldx, int in_dtype, const float* gamma, 
   return e == hipSuccess ? CRL_OK : hip_fail("crl_layernorm", e);
 }
 
-int crl_attention(const void* q, int64_t ldq, const void* k, int64_t ldk, const void* v, int64_t ldv, void* out, int64_t ldo,
+int crl_attention(const void* q, int64_t ldq, const void* k, int64_t ldk, const void* v, int64_t ldv, int in_dtype, void* out, int64_t ldo,
                   int out_dtype, float out_scale, int B, int H, int head_dim, int mode, float scale, const void* bias,
                   const void* pos, const float* u_bias, const float* v_bias, float* amax, void* stream) {
   if (!q || !k || !v || !out || B < 0 || H <= 0) return arg_fail("crl_attention: bad arguments");
   AttnArgs a;
   std::memset(&a, 0, sizeof(a));
-  a.q = q; a.k = k; a.v = v; a.ldq = ldq; a.ldk = ldk; a.ldv = ldv; a.out = out; a.ldo = ldo; a.out_dtype = out_dtype;
+  a.q = q; a.k = k; a.v = v; a.ldq = ldq; a.ldk = ldk; a.ldv = ldv; a.in_dtype = in_dtype; a.out = out; a.ldo = ldo; a.out_dtype = out_dtype;
   a.out_scale = out_scale; a.B = B; a.H = H; a.mode = mode; a.scale = scale; a.bias = bias; a.pos = pos;
   a.u_bias = u_bias; a.v_bias = v_bias; a.amax = amax;
   hipError_t e = launch_attention(a, head_dim, (hipStream_t)stream);
-  if (e == hipErrorInvalidValue) return arg_fail("crl_attention: head_dim must be 32 or 64, strides multiples of 8, mode inputs present");
+  if (e == hipErrorInvalidValue) return arg_fail("crl_attention: head_dim must be 32 or 64, in_dtype bf16/f16, out_dtype in_dtype or fp8, strides multiples of 8, mode inputs present");
   return e == hipSuccess ? CRL_OK : hip_fail("crl_attention", e);
 }
 

@@ -32,10 +32,31 @@ __host__ __device__ inline int attn_bias_slot(int i, int j) {
   return ((((it * 2 + jt) * 2 + rh) * 64 + lane) << 3) + e;
 }
 
-__device__ __forceinline__ bf16x8_t add_bias_bf16(bf16x8_t q, const float* bias8) {
-  bf16x8_t r;
+// The two 16-bit element types the kernel runs in.
+template <int DT>
+struct Half16;
+template <>
+struct Half16<DT_BF16> {
+  typedef bf16x8_t vec;
+  typedef __bf16 elem;
+  static __device__ __forceinline__ f32x16_t mfma(vec a, vec b, f32x16_t c) { return __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, 0, 0, 0); }
+  static __device__ __forceinline__ float to_f32(uint16_t h) { return bf16_bits_to_f32(h); }
+  static __device__ __forceinline__ uint32_t pack2(float lo, float hi) { return pack_bf16x2(lo, hi); }
+};
+template <>
+struct Half16<DT_F16> {
+  typedef f16x8_t vec;
+  typedef _Float16 elem;
+  static __device__ __forceinline__ f32x16_t mfma(vec a, vec b, f32x16_t c) { return __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, c, 0, 0, 0); }
+  static __device__ __forceinline__ float to_f32(uint16_t h) { return f16_bits_to_f32(h); }
+  static __device__ __forceinline__ uint32_t pack2(float lo, float hi) { return (uint32_t)f32_to_f16_bits(lo) | ((uint32_t)f32_to_f16_bits(hi) << 16); }
+};
+
+template <typename H>
+__device__ __forceinline__ typename H::vec add_bias_h(typename H::vec q, const float* bias8) {
+  typename H::vec r;
 #pragma unroll
-  for (int e = 0; e < 8; ++e) r[e] = (__bf16)((float)q[e] + bias8[e]);
+  for (int e = 0; e < 8; ++e) r[e] = (typename H::elem)((float)q[e] + bias8[e]);
   return r;
 }
 
@@ -44,8 +65,11 @@ __device__ __forceinline__ bf16x8_t add_bias_bf16(bf16x8_t q, const float* bias8
 template <int MODE>
 struct AttnWaves { static constexpr int N = MODE == ATTN_RELSHIFT ? 2 : 4; };
 
-template <int HS, int MODE, int OUT_DT>
+// OUT_FP8: write e4m3 (value*out_scale) instead of the input element type.
+template <int HS, int MODE, int OUT_FP8, int IN_DT>
 __global__ void __launch_bounds__(64 * AttnWaves<MODE>::N) attention_kernel(const AttnArgs a) {
+  typedef Half16<IN_DT> H16;
+  typedef typename H16::vec hvec;
   constexpr int KS = HS / 16;   // k-steps of the score product
   constexpr int DT_TILES = HS / 32;
   constexpr int NW = AttnWaves<MODE>::N;
@@ -90,13 +114,13 @@ __global__ void __launch_bounds__(64 * AttnWaves<MODE>::N) attention_kernel(cons
   }
 
   // ---- scores -----------------------------------------------------------------------
-  bf16x8_t qf[2][KS], kf[2][KS];
+  hvec qf[2][KS], kf[2][KS];
 #pragma unroll
   for (int t = 0; t < 2; ++t)
 #pragma unroll
     for (int ks = 0; ks < KS; ++ks) {
-      qf[t][ks] = *reinterpret_cast<const bf16x8_t*>(qp + (long)(32 * t + lr) * a.ldq + 16 * ks + 8 * g);
-      kf[t][ks] = *reinterpret_cast<const bf16x8_t*>(kp + (long)(32 * t + lr) * a.ldk + 16 * ks + 8 * g);
+      qf[t][ks] = *reinterpret_cast<const hvec*>(qp + (long)(32 * t + lr) * a.ldq + 16 * ks + 8 * g);
+      kf[t][ks] = *reinterpret_cast<const hvec*>(kp + (long)(32 * t + lr) * a.ldk + 16 * ks + 8 * g);
     }
 
   f32x16_t s[2][2];  // [jt][it]
@@ -126,17 +150,17 @@ __global__ void __launch_bounds__(64 * AttnWaves<MODE>::N) attention_kernel(cons
         ub[e] = a.u_bias[h * HS + 16 * ks + 8 * g + e];
         vb[e] = a.v_bias[h * HS + 16 * ks + 8 * g + e];
       }
-      bf16x8_t pf[2];
+      hvec pf[2];
 #pragma unroll
-      for (int t = 0; t < 2; ++t) pf[t] = *reinterpret_cast<const bf16x8_t*>(pp + (long)(32 * t + lr) * ldp + 16 * ks + 8 * g);
+      for (int t = 0; t < 2; ++t) pf[t] = *reinterpret_cast<const hvec*>(pp + (long)(32 * t + lr) * ldp + 16 * ks + 8 * g);
 #pragma unroll
       for (int it = 0; it < 2; ++it) {
-        const bf16x8_t qu = add_bias_bf16(qf[it][ks], ub);
-        const bf16x8_t qv = add_bias_bf16(qf[it][ks], vb);
+        const hvec qu = add_bias_h<H16>(qf[it][ks], ub);
+        const hvec qv = add_bias_h<H16>(qf[it][ks], vb);
 #pragma unroll
         for (int jt = 0; jt < 2; ++jt) {
-          s[jt][it] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf[jt][ks], qu, s[jt][it], 0, 0, 0);
-          sp[jt][it] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(pf[jt], qv, sp[jt][it], 0, 0, 0);
+          s[jt][it] = H16::mfma(kf[jt][ks], qu, s[jt][it]);
+          sp[jt][it] = H16::mfma(pf[jt], qv, sp[jt][it]);
         }
       }
     }
@@ -176,7 +200,7 @@ __global__ void __launch_bounds__(64 * AttnWaves<MODE>::N) attention_kernel(cons
       for (int jt = 0; jt < 2; ++jt)
 #pragma unroll
         for (int it = 0; it < 2; ++it)
-          s[jt][it] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf[jt][ks], qf[it][ks], s[jt][it], 0, 0, 0);
+          s[jt][it] = H16::mfma(kf[jt][ks], qf[it][ks], s[jt][it]);
 
     if constexpr (MODE == ATTN_BIAS) {
       const uint16_t* bp = reinterpret_cast<const uint16_t*>(a.bias) + (long)unit * 4096;
@@ -190,7 +214,7 @@ __global__ void __launch_bounds__(64 * AttnWaves<MODE>::N) attention_kernel(cons
             const uint32_t w[4] = {u.x, u.y, u.z, u.w};
 #pragma unroll
             for (int e = 0; e < 8; ++e) {
-              const float bv = bf16_bits_to_f32((uint16_t)((e & 1) ? (w[e >> 1] >> 16) : (w[e >> 1] & 0xffff)));
+              const float bv = H16::to_f32((uint16_t)((e & 1) ? (w[e >> 1] >> 16) : (w[e >> 1] & 0xffff)));
               s[jt][it][8 * rh + e] = s[jt][it][8 * rh + e] * a.scale + bv;
             }
           }
@@ -250,20 +274,20 @@ __global__ void __launch_bounds__(64 * AttnWaves<MODE>::N) attention_kernel(cons
 #pragma unroll
   for (int kb = 0; kb < 4; ++kb) {
     const int jt = kb >> 1, kh = kb & 1;
-    bf16x8_t pf[2];
+    hvec pf[2];
 #pragma unroll
     for (int it = 0; it < 2; ++it)
 #pragma unroll
-      for (int e = 0; e < 8; ++e) pf[it][e] = (__bf16)s[jt][it][8 * kh + e];
+      for (int e = 0; e < 8; ++e) pf[it][e] = (typename H16::elem)s[jt][it][8 * kh + e];
 #pragma unroll
     for (int dt = 0; dt < DT_TILES; ++dt) {
       const uint16_t* vrow = vt + (32 * dt + lr) * VT_STRIDE + 16 * kb + 4 * g;
       const uint2 lo = *reinterpret_cast<const uint2*>(vrow);
       const uint2 hi = *reinterpret_cast<const uint2*>(vrow + 8);
       const uint4 packed = make_uint4(lo.x, lo.y, hi.x, hi.y);
-      const bf16x8_t vf = __builtin_bit_cast(bf16x8_t, packed);
+      const hvec vf = __builtin_bit_cast(hvec, packed);
 #pragma unroll
-      for (int it = 0; it < 2; ++it) o[dt][it] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vf, pf[it], o[dt][it], 0, 0, 0);
+      for (int it = 0; it < 2; ++it) o[dt][it] = H16::mfma(vf, pf[it], o[dt][it]);
     }
   }
 
@@ -284,11 +308,11 @@ __global__ void __launch_bounds__(64 * AttnWaves<MODE>::N) attention_kernel(cons
           am = fmaxf(am, fabsf(v[e]));
         }
         const long off = row * a.ldo + h * HS + d;
-        if constexpr (OUT_DT == DT_FP8) {
+        if constexpr (OUT_FP8) {
           *reinterpret_cast<uint32_t*>(reinterpret_cast<uint8_t*>(a.out) + off) =
               pack_fp8x4(v[0] * a.out_scale, v[1] * a.out_scale, v[2] * a.out_scale, v[3] * a.out_scale);
         } else {
-          *reinterpret_cast<uint2*>(reinterpret_cast<uint16_t*>(a.out) + off) = make_uint2(pack_bf16x2(v[0], v[1]), pack_bf16x2(v[2], v[3]));
+          *reinterpret_cast<uint2*>(reinterpret_cast<uint16_t*>(a.out) + off) = make_uint2(H16::pack2(v[0], v[1]), H16::pack2(v[2], v[3]));
         }
       }
   }
@@ -298,14 +322,21 @@ __global__ void __launch_bounds__(64 * AttnWaves<MODE>::N) attention_kernel(cons
   }
 }
 
-template <int HS, int MODE>
-static hipError_t launch_attn_mode(const AttnArgs& a, hipStream_t st) {
+template <int HS, int MODE, int IN_DT>
+static hipError_t launch_attn_dt(const AttnArgs& a, hipStream_t st) {
   constexpr int NW = AttnWaves<MODE>::N;
   const dim3 grid((a.B * a.H + NW - 1) / NW), block(64 * NW);
-  if (a.out_dtype == DT_FP8) hipLaunchKernelGGL((attention_kernel<HS, MODE, DT_FP8>), grid, block, 0, st, a);
-  else if (a.out_dtype == DT_BF16) hipLaunchKernelGGL((attention_kernel<HS, MODE, DT_BF16>), grid, block, 0, st, a);
+  if (a.out_dtype == DT_FP8) hipLaunchKernelGGL((attention_kernel<HS, MODE, 1, IN_DT>), grid, block, 0, st, a);
+  else if (a.out_dtype == IN_DT) hipLaunchKernelGGL((attention_kernel<HS, MODE, 0, IN_DT>), grid, block, 0, st, a);
   else return hipErrorInvalidValue;
   return hipGetLastError();
+}
+
+template <int HS, int MODE>
+static hipError_t launch_attn_mode(const AttnArgs& a, hipStream_t st) {
+  if (a.in_dtype == DT_F16) return launch_attn_dt<HS, MODE, DT_F16>(a, st);
+  if (a.in_dtype == DT_BF16) return launch_attn_dt<HS, MODE, DT_BF16>(a, st);
+  return hipErrorInvalidValue;
 }
 
 template <int HS>

@@ -143,16 +143,17 @@ struct EmbedArgs {
 enum AttnMode : int { ATTN_PLAIN = 0, ATTN_CAUSAL = 1, ATTN_BIAS = 2, ATTN_RELSHIFT = 3 };
 
 struct AttnArgs {
-  const void* q; const void* k; const void* v;  // bf16, [B*64, ld*] with head h at column h*HS
+  const void* q; const void* k; const void* v;  // bf16 or f16, [B*64, ld*] with head h at column h*HS
   long ldq, ldk, ldv;
   const void* bias;     // ATTN_BIAS: bf16 [B,H,4096] in the kernel's register order
   const void* pos;      // ATTN_RELSHIFT: bf16 [64, H*HS] projected positional table
   const float* u_bias;  // ATTN_RELSHIFT: [H*HS]
   const float* v_bias;  // ATTN_RELSHIFT: [H*HS]
-  void* out;            // [B*64, ldo] bf16 or fp8
+  void* out;            // [B*64, ldo] in the input element type, or fp8
   long ldo;
   float* amax;
   int B, H, mode, out_dtype;
+  int in_dtype;         // DT_BF16 or DT_F16: element type of q, k, v, bias and pos
   float scale, out_scale;
 };
 

@@ -42,7 +42,8 @@ Model::Model(const crl_model_config& c) : cfg(c) {
   if (cfg.smolgen_compress == 0) cfg.smolgen_compress = 32;
   if (cfg.smolgen_hidden == 0) cfg.smolgen_hidden = 256;
   if (cfg.smolgen_gen == 0) cfg.smolgen_gen = 256;
-  if (cfg.head_dtype != DT_F16) cfg.head_dtype = DT_BF16;
+  if (cfg.act_dtype != DT_F16) cfg.act_dtype = DT_BF16;
+  if (cfg.head_dtype != DT_F16 && cfg.head_dtype != DT_BF16) cfg.head_dtype = cfg.act_dtype;
   if (cfg.micro_batch <= 0) cfg.micro_batch = 4096;
   vocab = cfg.arch == CRL_ARCH_BT4CLASS ? VOCAB_LEELA : VOCAB_RL;
   const long C = cfg.d_model, F = cfg.d_ff, L = cfg.n_layer, H = cfg.n_head;
@@ -171,7 +172,7 @@ int Model::finalize() {
   layers.assign(cfg.n_layer, Layer());
   const int C = cfg.d_model, F = cfg.d_ff, H = cfg.n_head;
   const bool f8 = cfg.fp8 != 0;
-  const int hd = cfg.head_dtype;
+  const int hd = cfg.head_dtype, ad = cfg.act_dtype;
   int rc;
 #define UP(vec, dt, out) do { rc = upload(vec, dt, 1.f, (void**)&(out)); if (rc) return rc; } while (0)
 #define LIN(L, W, B, N, K, dt, f) do { rc = make_lin(L, W, B, N, K, dt, f); if (rc) return rc; } while (0)
@@ -197,10 +198,10 @@ int Model::finalize() {
       const std::string p = lkey("transformer.h.%d.", i);
       UP(w(p + "ln_1.weight"), DT_F32, ly.ln1_g); UP(w(p + "ln_1.bias"), DT_F32, ly.ln1_b);
       UP(w(p + "ln_2.weight"), DT_F32, ly.ln2_g); UP(w(p + "ln_2.bias"), DT_F32, ly.ln2_b);
-      LIN(ly.qkv, w(p + "attn.c_attn.weight"), &w(p + "attn.c_attn.bias"), 3 * C, C, DT_BF16, f8);
-      LIN(ly.proj, w(p + "attn.c_proj.weight"), &w(p + "attn.c_proj.bias"), C, C, DT_BF16, f8);
-      LIN(ly.ff1, w(p + "mlp.c_fc.weight"), &w(p + "mlp.c_fc.bias"), F, C, DT_BF16, f8);
-      LIN(ly.ff2, w(p + "mlp.c_proj.weight"), &w(p + "mlp.c_proj.bias"), C, F, DT_BF16, f8);
+      LIN(ly.qkv, w(p + "attn.c_attn.weight"), &w(p + "attn.c_attn.bias"), 3 * C, C, ad, f8);
+      LIN(ly.proj, w(p + "attn.c_proj.weight"), &w(p + "attn.c_proj.bias"), C, C, ad, f8);
+      LIN(ly.ff1, w(p + "mlp.c_fc.weight"), &w(p + "mlp.c_fc.bias"), F, C, ad, f8);
+      LIN(ly.ff2, w(p + "mlp.c_proj.weight"), &w(p + "mlp.c_proj.bias"), C, F, ad, f8);
     }
     UP(w("transformer.ln_f.weight"), DT_F32, lnf_g); UP(w("transformer.ln_f.bias"), DT_F32, lnf_b);
     LIN(lm_head, w("lm_head.weight"), nullptr, VOCAB_RL, C, hd, false);
@@ -226,10 +227,10 @@ int Model::finalize() {
         bq.insert(bq.end(), (size_t)cfg.smolgen_compress, 0.f);
         nq += cfg.smolgen_compress;
       }
-      LIN(ly.qkv, wq, &bq, nq, C, DT_BF16, f8);
-      LIN(ly.proj, w(p + "attention.out_proj.weight"), &w(p + "attention.out_proj.bias"), C, C, DT_BF16, f8);
-      LIN(ly.ff1, w(p + "ff1.weight"), &w(p + "ff1.bias"), F, C, DT_BF16, f8);
-      LIN(ly.ff2, w(p + "ff2.weight"), &w(p + "ff2.bias"), C, F, DT_BF16, f8);
+      LIN(ly.qkv, wq, &bq, nq, C, ad, f8);
+      LIN(ly.proj, w(p + "attention.out_proj.weight"), &w(p + "attention.out_proj.bias"), C, C, ad, f8);
+      LIN(ly.ff1, w(p + "ff1.weight"), &w(p + "ff1.bias"), F, C, ad, f8);
+      LIN(ly.ff2, w(p + "ff2.weight"), &w(p + "ff2.bias"), C, F, ad, f8);
       UP(w(p + "norm1.weight"), DT_F32, ly.ln1_g); UP(w(p + "norm1.bias"), DT_F32, ly.ln1_b);
       UP(w(p + "norm2.weight"), DT_F32, ly.ln2_g); UP(w(p + "norm2.bias"), DT_F32, ly.ln2_b);
       if (cfg.arch == CRL_ARCH_BT4) {
@@ -242,13 +243,13 @@ int Model::finalize() {
             for (int c = 0; c < C; ++c) s += (double)pe[(size_t)t * C + c] * pw[(size_t)o * C + c];
             pt[(size_t)t * C + o] = (float)s;
           }
-        UP(pt, DT_BF16, ly.pos);
+        UP(pt, ad, ly.pos);
         UP(w(p + "attention.u_bias"), DT_F32, ly.u_bias);
         UP(w(p + "attention.v_bias"), DT_F32, ly.v_bias);
       } else {
         const int sc = cfg.smolgen_compress, sh = cfg.smolgen_hidden, sg = cfg.smolgen_gen;
-        LIN(ly.sm_hidden, w(p + "smolgen.hidden.weight"), &w(p + "smolgen.hidden.bias"), sh, 64 * sc, DT_BF16, false);
-        LIN(ly.sm_gen, w(p + "smolgen.gen_from.weight"), &w(p + "smolgen.gen_from.bias"), H * sg, sh, DT_BF16, false);
+        LIN(ly.sm_hidden, w(p + "smolgen.hidden.weight"), &w(p + "smolgen.hidden.bias"), sh, 64 * sc, ad, false);
+        LIN(ly.sm_gen, w(p + "smolgen.gen_from.weight"), &w(p + "smolgen.gen_from.bias"), H * sg, sh, ad, false);
         UP(w(p + "smolgen.hidden_ln.weight"), DT_F32, ly.sm_ln1_g); UP(w(p + "smolgen.hidden_ln.bias"), DT_F32, ly.sm_ln1_b);
         UP(w(p + "smolgen.gen_from_ln.weight"), DT_F32, ly.sm_ln2_g); UP(w(p + "smolgen.gen_from_ln.bias"), DT_F32, ly.sm_ln2_b);
       }
@@ -270,7 +271,7 @@ int Model::finalize() {
       for (int i = 0; i < 64; ++i)
         for (int j = 0; j < 64; ++j)
           std::memcpy(&perm[(size_t)attn_bias_slot_host(i, j) * sg], &gw[(size_t)(i * 64 + j) * sg], sizeof(float) * sg);
-      LIN(sm_weight_gen, perm, nullptr, 4096, sg, DT_BF16, false);
+      LIN(sm_weight_gen, perm, nullptr, 4096, sg, ad, false);
       UP(w("promotion_offsets.weight"), DT_F32, promo_w);
       // Gather tables: Leela move v -> (from_token*64+to_token) for black / white rows.
       std::vector<int16_t> gi((size_t)2 * VOCAB_LEELA);
@@ -446,10 +447,10 @@ int Model::forward_chunk(const float* planes, const uint8_t* ids, const uint8_t*
   const int C = cfg.d_model, F = cfg.d_ff, H = cfg.n_head, L = cfg.n_layer, hs = C / H;
   const int M = mb * 64;
   const bool f8 = cfg.fp8 && !calibrate;
-  const int hd = cfg.head_dtype;
+  const int hd = cfg.head_dtype, ad = cfg.act_dtype;
   const bool gpt = cfg.arch == CRL_ARCH_GPT64;
   const bool sf32 = gpt && cfg.stream_f32;
-  const int xdt = sf32 ? DT_F32 : DT_BF16;
+  const int xdt = sf32 ? DT_F32 : ad;
   auto am = [&](int l, int slot) -> float* { return calibrate ? amax_dev + (size_t)l * 4 + slot : nullptr; };
   int rc;
 #define RUN(call) do { rc = (call); if (rc) return rc; } while (0)
@@ -481,27 +482,27 @@ int Model::forward_chunk(const float* planes, const uint8_t* ids, const uint8_t*
     const void* a_in; int a_dt; float a_sc = 1.f;
     if (gpt) {
       // h = LN1(x)
-      RUN(lnorm(ws.x, C, xdt, ly.ln1_g, ly.ln1_b, f8 ? nullptr : ws.h, DT_BF16, f8 ? ws.h8 : nullptr, f8 ? act_scale(l, 0) : 1.f, C, M, C, am(l, 0), st));
-      a_in = f8 ? (const void*)ws.h8 : (const void*)ws.h; a_dt = f8 ? DT_FP8 : DT_BF16; a_sc = f8 ? act_scale(l, 0) : 1.f;
+      RUN(lnorm(ws.x, C, xdt, ly.ln1_g, ly.ln1_b, f8 ? nullptr : ws.h, ad, f8 ? ws.h8 : nullptr, f8 ? act_scale(l, 0) : 1.f, C, M, C, am(l, 0), st));
+      a_in = f8 ? (const void*)ws.h8 : (const void*)ws.h; a_dt = f8 ? DT_FP8 : ad; a_sc = f8 ? act_scale(l, 0) : 1.f;
     } else {
-      a_in = f8 ? (const void*)ws.x8 : (const void*)ws.x; a_dt = f8 ? DT_FP8 : DT_BF16; a_sc = f8 ? act_scale(l, 0) : 1.f;
+      a_in = f8 ? (const void*)ws.x8 : (const void*)ws.x; a_dt = f8 ? DT_FP8 : ad; a_sc = f8 ? act_scale(l, 0) : 1.f;
     }
     // q|k|v (and the smolgen compression for BT4-class) in one GEMM
     {
       GOpt o; o.a_scale = a_sc;
       if (cfg.arch == CRL_ARCH_BT4CLASS) { o.C2 = ws.comp; o.ldc2 = cfg.smolgen_compress; o.nsplit = 3 * C; }
-      RUN(gemm(ly.qkv, a_in, C, a_dt, ws.qkv, 3 * C, DT_BF16, M, o, st));
+      RUN(gemm(ly.qkv, a_in, C, a_dt, ws.qkv, 3 * C, ad, M, o, st));
     }
     const void* bias_tile = nullptr;
     if (cfg.arch == CRL_ARCH_BT4CLASS) {
       const int sc = cfg.smolgen_compress, sh = cfg.smolgen_hidden, sg = cfg.smolgen_gen;
       GOpt o; o.act = ACT_SWISH;
-      RUN(gemm(ly.sm_hidden, ws.comp, 64 * sc, DT_BF16, ws.sh1, sh, DT_BF16, mb, o, st));
-      RUN(lnorm(ws.sh1, sh, DT_BF16, ly.sm_ln1_g, ly.sm_ln1_b, ws.sh2, DT_BF16, nullptr, 1.f, sh, mb, sh, nullptr, st));
-      RUN(gemm(ly.sm_gen, ws.sh2, sh, DT_BF16, ws.sg1, H * sg, DT_BF16, mb, o, st));
-      RUN(lnorm(ws.sg1, H * sg, DT_BF16, ly.sm_ln2_g, ly.sm_ln2_b, ws.sg2, DT_BF16, nullptr, 1.f, H * sg, mb, H * sg, nullptr, st));
+      RUN(gemm(ly.sm_hidden, ws.comp, 64 * sc, ad, ws.sh1, sh, ad, mb, o, st));
+      RUN(lnorm(ws.sh1, sh, ad, ly.sm_ln1_g, ly.sm_ln1_b, ws.sh2, ad, nullptr, 1.f, sh, mb, sh, nullptr, st));
+      RUN(gemm(ly.sm_gen, ws.sh2, sh, ad, ws.sg1, H * sg, ad, mb, o, st));
+      RUN(lnorm(ws.sg1, H * sg, ad, ly.sm_ln2_g, ly.sm_ln2_b, ws.sg2, ad, nullptr, 1.f, H * sg, mb, H * sg, nullptr, st));
       GOpt o2;
-      RUN(gemm(sm_weight_gen, ws.sg2, sg, DT_BF16, ws.bias, 4096, DT_BF16, mb * H, o2, st));
+      RUN(gemm(sm_weight_gen, ws.sg2, sg, ad, ws.bias, 4096, ad, mb * H, o2, st));
       bias_tile = ws.bias;
     }
     // attention
@@ -511,9 +512,9 @@ int Model::forward_chunk(const float* planes, const uint8_t* ids, const uint8_t*
       const uint16_t* base = reinterpret_cast<const uint16_t*>(ws.qkv);
       a.q = base; a.k = base + C; a.v = base + 2 * C; a.ldq = a.ldk = a.ldv = 3 * C;
       a.bias = bias_tile; a.pos = ly.pos; a.u_bias = ly.u_bias; a.v_bias = ly.v_bias;
-      a.out = f8 ? (void*)ws.ao8 : (void*)ws.ao; a.ldo = C; a.out_dtype = f8 ? DT_FP8 : DT_BF16;
+      a.out = f8 ? (void*)ws.ao8 : (void*)ws.ao; a.ldo = C; a.out_dtype = f8 ? DT_FP8 : ad;
       a.out_scale = f8 ? act_scale(l, 1) : 1.f; a.amax = am(l, 1);
-      a.B = mb; a.H = H; a.scale = attn_scale;
+      a.B = mb; a.H = H; a.scale = attn_scale; a.in_dtype = ad;
       a.mode = gpt ? ATTN_CAUSAL : cfg.arch == CRL_ARCH_BT4 ? ATTN_RELSHIFT : ATTN_BIAS;
       prof_begin(1, st);
       hipError_t he = launch_attention(a, hs, st);
@@ -521,36 +522,36 @@ int Model::forward_chunk(const float* planes, const uint8_t* ids, const uint8_t*
       HIPCHK(he);
     }
     const void* ao_in = f8 ? (const void*)ws.ao8 : (const void*)ws.ao;
-    const int ao_dt = f8 ? DT_FP8 : DT_BF16;
+    const int ao_dt = f8 ? DT_FP8 : ad;
     if (gpt) {
       // x += proj(ao);  h = LN2(x);  x += proj2(gelu(fc(h)))
       { GOpt o; o.res = ws.x; o.ldr = C; o.res_dt = xdt; o.a_scale = f8 ? act_scale(l, 1) : 1.f;
         RUN(gemm(ly.proj, ao_in, C, ao_dt, ws.x, C, xdt, M, o, st)); }
-      RUN(lnorm(ws.x, C, xdt, ly.ln2_g, ly.ln2_b, f8 ? nullptr : ws.h, DT_BF16, f8 ? ws.h8 : nullptr, f8 ? act_scale(l, 2) : 1.f, C, M, C, am(l, 2), st));
+      RUN(lnorm(ws.x, C, xdt, ly.ln2_g, ly.ln2_b, f8 ? nullptr : ws.h, ad, f8 ? ws.h8 : nullptr, f8 ? act_scale(l, 2) : 1.f, C, M, C, am(l, 2), st));
       { GOpt o; o.act = ACT_GELU; o.a_scale = f8 ? act_scale(l, 2) : 1.f; o.out_scale = f8 ? act_scale(l, 3) : 1.f; o.amax = am(l, 3);
         RUN(gemm(ly.ff1, f8 ? (const void*)ws.h8 : (const void*)ws.h, C, ao_dt, f8 ? (void*)ws.f8 : (void*)ws.f, F, ao_dt, M, o, st)); }
       { GOpt o; o.res = ws.x; o.ldr = C; o.res_dt = xdt; o.a_scale = f8 ? act_scale(l, 3) : 1.f;
         RUN(gemm(ly.ff2, f8 ? (const void*)ws.f8 : (const void*)ws.f, F, ao_dt, ws.x, C, xdt, M, o, st)); }
     } else {
       // t = x + alpha*proj(ao);  h = LN1(t)
-      { GOpt o; o.res = ws.x; o.ldr = C; o.res_dt = DT_BF16; o.alpha = alpha; o.a_scale = f8 ? act_scale(l, 1) : 1.f;
-        RUN(gemm(ly.proj, ao_in, C, ao_dt, ws.t, C, DT_BF16, M, o, st)); }
-      RUN(lnorm(ws.t, C, DT_BF16, ly.ln1_g, ly.ln1_b, ws.h, DT_BF16, f8 ? ws.h8 : nullptr, f8 ? act_scale(l, 2) : 1.f, C, M, C, am(l, 2), st));
+      { GOpt o; o.res = ws.x; o.ldr = C; o.res_dt = ad; o.alpha = alpha; o.a_scale = f8 ? act_scale(l, 1) : 1.f;
+        RUN(gemm(ly.proj, ao_in, C, ao_dt, ws.t, C, ad, M, o, st)); }
+      RUN(lnorm(ws.t, C, ad, ly.ln1_g, ly.ln1_b, ws.h, ad, f8 ? ws.h8 : nullptr, f8 ? act_scale(l, 2) : 1.f, C, M, C, am(l, 2), st));
       const void* h_in = f8 ? (const void*)ws.h8 : (const void*)ws.h;
       if (cfg.arch == CRL_ARCH_BT4) {
         // y = ff2(ff1(h)) with no activation in between; t = gelu(y) + h (new_paradigm/value.py:65-70)
         { GOpt o; o.a_scale = f8 ? act_scale(l, 2) : 1.f; o.out_scale = f8 ? act_scale(l, 3) : 1.f; o.amax = am(l, 3);
           RUN(gemm(ly.ff1, h_in, C, ao_dt, f8 ? (void*)ws.f8 : (void*)ws.f, F, ao_dt, M, o, st)); }
-        { GOpt o; o.act = ACT_GELU; o.res = ws.h; o.ldr = C; o.res_dt = DT_BF16; o.a_scale = f8 ? act_scale(l, 3) : 1.f;
-          RUN(gemm(ly.ff2, f8 ? (const void*)ws.f8 : (const void*)ws.f, F, ao_dt, ws.t, C, DT_BF16, M, o, st)); }
+        { GOpt o; o.act = ACT_GELU; o.res = ws.h; o.ldr = C; o.res_dt = ad; o.a_scale = f8 ? act_scale(l, 3) : 1.f;
+          RUN(gemm(ly.ff2, f8 ? (const void*)ws.f8 : (const void*)ws.f, F, ao_dt, ws.t, C, ad, M, o, st)); }
       } else {
         { GOpt o; o.act = ACT_MISH; o.a_scale = f8 ? act_scale(l, 2) : 1.f; o.out_scale = f8 ? act_scale(l, 3) : 1.f; o.amax = am(l, 3);
           RUN(gemm(ly.ff1, h_in, C, ao_dt, f8 ? (void*)ws.f8 : (void*)ws.f, F, ao_dt, M, o, st)); }
-        { GOpt o; o.res = ws.h; o.ldr = C; o.res_dt = DT_BF16; o.alpha = alpha; o.a_scale = f8 ? act_scale(l, 3) : 1.f;
-          RUN(gemm(ly.ff2, f8 ? (const void*)ws.f8 : (const void*)ws.f, F, ao_dt, ws.t, C, DT_BF16, M, o, st)); }
+        { GOpt o; o.res = ws.h; o.ldr = C; o.res_dt = ad; o.alpha = alpha; o.a_scale = f8 ? act_scale(l, 3) : 1.f;
+          RUN(gemm(ly.ff2, f8 ? (const void*)ws.f8 : (const void*)ws.f, F, ao_dt, ws.t, C, ad, M, o, st)); }
       }
       // x = LN2(t); the last layer's output feeds only the heads.
-      RUN(lnorm(ws.t, C, DT_BF16, ly.ln2_g, ly.ln2_b, ws.x, last ? hd : DT_BF16, (f8 && !last) ? ws.x8 : nullptr,
+      RUN(lnorm(ws.t, C, ad, ly.ln2_g, ly.ln2_b, ws.x, last ? hd : ad, (f8 && !last) ? ws.x8 : nullptr,
                 (f8 && !last) ? act_scale(l + 1, 0) : 1.f, C, M, C, last ? nullptr : am(l + 1, 0), st));
     }
   }

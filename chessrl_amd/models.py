@@ -135,13 +135,14 @@ class _Engine:
     """Owns one crl_model handle."""
 
     def __init__(self, arch, n_layer, d_model, n_head, d_ff, fp8=False, micro_batch=0, stream_f32=True,
-                 head_dtype="bf16", compress=32, hidden=256, gen=256):
+                 head_dtype=None, act_dtype="bf16", compress=32, hidden=256, gen=256):
         cfg = _lib.ModelConfig()
         cfg.arch, cfg.n_layer, cfg.d_model, cfg.n_head, cfg.d_ff = arch, n_layer, d_model, n_head, d_ff
         cfg.fp8 = 1 if fp8 else 0
         cfg.micro_batch = micro_batch
         cfg.stream_f32 = 1 if stream_f32 else 0
-        cfg.head_dtype = _lib.F16 if head_dtype in ("f16", "fp16") else _lib.BF16
+        cfg.act_dtype = _lib.F16 if act_dtype in ("f16", "fp16") else _lib.BF16
+        cfg.head_dtype = cfg.act_dtype if head_dtype is None else _lib.F16 if head_dtype in ("f16", "fp16") else _lib.BF16
         cfg.smolgen_compress, cfg.smolgen_hidden, cfg.smolgen_gen = compress, hidden, gen
         self.cfg = cfg
         self.n_layer = n_layer
@@ -382,7 +383,7 @@ class GPTConfig:
 class GPT(_ModelBase):
     """model_bis.GPT for the 64 board tokens (model_bis.py:125-199, 358-398)."""
 
-    def __init__(self, config, fp8=False, micro_batch=0, stream_f32=True, head_dtype="bf16", seed=0):
+    def __init__(self, config, fp8=False, micro_batch=0, stream_f32=True, head_dtype=None, act_dtype="bf16", seed=0):
         if config.vocab_size != VOCAB_RL:
             raise ValueError("vocab_size must be %d (utils/vocab.py)" % VOCAB_RL)
         if not config.bias:
@@ -398,7 +399,7 @@ class GPT(_ModelBase):
         from_pe[:, 1::2] = torch.cos(pos * div)
         self._sd["pe"] = from_pe
         self._engine = _Engine(_lib.ARCH_GPT64, config.n_layer, config.n_embd, config.n_head, 4 * config.n_embd,
-                               fp8=fp8, micro_batch=micro_batch, stream_f32=stream_f32, head_dtype=head_dtype)
+                               fp8=fp8, micro_batch=micro_batch, stream_f32=stream_f32, head_dtype=head_dtype, act_dtype=act_dtype)
         self._engine.load(self._sd)
 
     def get_num_params(self, non_embedding=True):
@@ -430,11 +431,11 @@ class GPT(_ModelBase):
 class BT4(_ModelBase):
     """new_paradigm/value.py BT4 (value.py:121-400)."""
 
-    def __init__(self, num_layers=10, d_model=512, d_ff=736, num_heads=8, fp8=False, micro_batch=0, head_dtype="bf16", seed=0):
+    def __init__(self, num_layers=10, d_model=512, d_ff=736, num_heads=8, fp8=False, micro_batch=0, head_dtype=None, act_dtype="bf16", seed=0):
         self.num_layers, self.d_model = num_layers, d_model
         self._shapes = bt4_shapes(num_layers, d_model, d_ff, num_heads)
         self._sd = _default_init(self._shapes, seed)
-        self._engine = _Engine(_lib.ARCH_BT4, num_layers, d_model, num_heads, d_ff, fp8=fp8, micro_batch=micro_batch, head_dtype=head_dtype)
+        self._engine = _Engine(_lib.ARCH_BT4, num_layers, d_model, num_heads, d_ff, fp8=fp8, micro_batch=micro_batch, head_dtype=head_dtype, act_dtype=act_dtype)
         self._engine.load(self._sd)
 
     @torch.no_grad()
@@ -498,12 +499,12 @@ class BT4Class(_ModelBase):
     attention policy gathered to the 1858 side-to-move-frame moves, WDL head."""
 
     def __init__(self, num_layers=15, d_model=1024, d_ff=1536, num_heads=32, fp8=False, micro_batch=0,
-                 head_dtype="bf16", compress=32, hidden=256, gen=256, seed=0):
+                 head_dtype=None, act_dtype="bf16", compress=32, hidden=256, gen=256, seed=0):
         self.num_layers, self.d_model = num_layers, d_model
         self._shapes = bt4_shapes(num_layers, d_model, d_ff, num_heads, True, compress, hidden, gen)
         self._sd = _default_init(self._shapes, seed)
         self._engine = _Engine(_lib.ARCH_BT4CLASS, num_layers, d_model, num_heads, d_ff, fp8=fp8, micro_batch=micro_batch,
-                               head_dtype=head_dtype, compress=compress, hidden=hidden, gen=gen)
+                               head_dtype=head_dtype, act_dtype=act_dtype, compress=compress, hidden=hidden, gen=gen)
         self._engine.load(self._sd)
 
     @torch.no_grad()

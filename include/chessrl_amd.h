@@ -108,11 +108,11 @@ int crl_gemm(const void* A, int64_t lda, const void* W, int64_t ldw, void* C, in
 int crl_layernorm(const void* x, int64_t ldx, int in_dtype, const float* gamma, const float* beta,
                   void* out, int out_dtype, uint8_t* out_fp8, float fp8_scale, int64_t ldo,
                   int rows, int C, float eps, float* amax, void* stream);
-/* Attention over 64 tokens per position, bf16 q/k/v with head h at columns [h*head_dim, ...).
+/* Attention over 64 tokens per position, q/k/v of in_dtype (bf16 or f16) with head h at columns [h*head_dim, ...).
  * mode CAUSAL: model_bis.py:71; RELSHIFT: new_paradigm/attn.py:507-521 with pos = pos_proj(PE)
- * (bf16 [64,H*head_dim]) and u_bias/v_bias fp32[H*head_dim]; BIAS: bias bf16 [B,H,64,64] in the
- * order crl_attn_bias_slot defines. out is bf16 or fp8 (value*out_scale) [B*64, ldo]. */
-int crl_attention(const void* q, int64_t ldq, const void* k, int64_t ldk, const void* v, int64_t ldv,
+ * (in_dtype [64,H*head_dim]) and u_bias/v_bias fp32[H*head_dim]; BIAS: bias of in_dtype [B,H,64,64] in the
+ * order crl_attn_bias_slot defines. out is of in_dtype or fp8 (value*out_scale) [B*64, ldo]. */
+int crl_attention(const void* q, int64_t ldq, const void* k, int64_t ldk, const void* v, int64_t ldv, int in_dtype,
                   void* out, int64_t ldo, int out_dtype, float out_scale,
                   int B, int H, int head_dim, int mode, float scale,
                   const void* bias, const void* pos, const float* u_bias, const float* v_bias,
@@ -138,10 +138,11 @@ typedef struct crl_model_config {
   int32_t fp8;            /* 1: trunk linears (qkv, out-proj, ffn) run in e4m3 with static per-tensor scales */
   int32_t micro_batch;    /* positions per pass through the trunk; 0 = default */
   int32_t stream_f32;     /* GPT64 only: keep the residual stream in fp32 (default 1) */
-  int32_t head_dtype;     /* CRL_BF16 or CRL_F16: element type of the policy/value head GEMM inputs */
+  int32_t head_dtype;     /* CRL_BF16 or CRL_F16: element type of the policy/value head GEMM inputs; 0 = act_dtype */
   int32_t smolgen_compress, smolgen_hidden, smolgen_gen;  /* BT4-class; 0 = 32/256/256 */
   float eps;              /* LayerNorm epsilon; 0 = 1e-5 */
-  int32_t reserved[4];
+  int32_t act_dtype;      /* CRL_BF16 (default) or CRL_F16: 16-bit element type of activations and weights */
+  int32_t reserved[3];
 } crl_model_config;
 
 /* GPT(config) / BT4(...) constructors (model_bis.py:127-157, new_paradigm/value.py:122-152). */

@@ -131,10 +131,10 @@ def test_layernorm(cuda, C_, in_dt):
     assert abs(amax.item() - ref.abs().max().item()) < 1e-3 * ref.abs().max().item()
 
 
-def make_qkv(B, H, hs, device, seed):
+def make_qkv(B, H, hs, device, seed, dtype=torch.bfloat16):
     torch.manual_seed(seed)
     Cm = H * hs
-    qkv = (torch.randn(B * 64, 3 * Cm, device=device)).bfloat16()
+    qkv = (torch.randn(B * 64, 3 * Cm, device=device)).to(dtype)
     return qkv, Cm
 
 
@@ -144,11 +144,13 @@ def split_heads(qkv, B, H, hs):
     return [t.view(B, 64, H, hs).transpose(1, 2) for t in (q, k, v)]
 
 
-def run_attn(qkv, B, H, hs, mode, scale, bias=None, pos=None, u=None, v=None, out_dt=_lib.BF16, out_scale=1.0):
+def run_attn(qkv, B, H, hs, mode, scale, bias=None, pos=None, u=None, v=None, out_dt=None, out_scale=1.0):
     Cm = H * hs
-    out = torch.zeros(B * 64, Cm, dtype=torch.bfloat16 if out_dt == _lib.BF16 else torch.uint8, device=qkv.device)
+    in_dt = _lib.F16 if qkv.dtype == torch.float16 else _lib.BF16
+    out_dt = in_dt if out_dt is None else out_dt
+    out = torch.zeros(B * 64, Cm, dtype=qkv.dtype if out_dt != _lib.FP8 else torch.uint8, device=qkv.device)
     base = qkv.data_ptr()
-    check(lib().crl_attention(C.c_void_p(base), 3 * Cm, C.c_void_p(base + 2 * Cm), 3 * Cm, C.c_void_p(base + 4 * Cm), 3 * Cm,
+    check(lib().crl_attention(C.c_void_p(base), 3 * Cm, C.c_void_p(base + 2 * Cm), 3 * Cm, C.c_void_p(base + 4 * Cm), 3 * Cm, in_dt,
                               p(out), Cm, out_dt, out_scale, B, H, hs, mode, scale, p(bias), p(pos), p(u), p(v), None, stream()), "attn")
     torch.cuda.synchronize()
     return out
@@ -156,15 +158,17 @@ def run_attn(qkv, B, H, hs, mode, scale, bias=None, pos=None, u=None, v=None, ou
 
 @pytest.mark.parametrize("H,hs", [(8, 32), (12, 64), (32, 32)])
 @pytest.mark.parametrize("mode", [_lib.ATTN_PLAIN, _lib.ATTN_CAUSAL])
-def test_attention_plain_causal(cuda, H, hs, mode):
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+def test_attention_plain_causal(cuda, H, hs, mode, dtype):
     B = 5
-    qkv, Cm = make_qkv(B, H, hs, cuda, H + mode)
+    qkv, Cm = make_qkv(B, H, hs, cuda, H + mode, dtype)
     out = run_attn(qkv, B, H, hs, mode, 1 / math.sqrt(hs))
     q, k, v = split_heads(qkv, B, H, hs)
     ref = F.scaled_dot_product_attention(q, k, v, is_causal=(mode == _lib.ATTN_CAUSAL))
     ref = ref.transpose(1, 2).reshape(B * 64, Cm)
-    # probabilities are rounded to bf16 before P·V and the output to bf16: 2^-8 relative each
-    assert torch.allclose(out.float(), ref, rtol=2 ** -6, atol=2 ** -6), (out.float() - ref).abs().max()
+    # probabilities are rounded to the 16-bit type before P·V, and so is the output: 2^-8 (bf16) or 2^-11 (f16) relative each
+    tol = 2 ** -6 if dtype == torch.bfloat16 else 2 ** -9
+    assert torch.allclose(out.float(), ref, rtol=tol, atol=tol), (out.float() - ref).abs().max()
 
 
 def test_attention_bias(cuda):
