@@ -33,6 +33,9 @@ def parse():
     ap.add_argument("--layers", type=int, default=15, help=argparse.SUPPRESS)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-latency", action="store_true", help="skip the batch-64 latency leg")
+    ap.add_argument("--act-dtype", default="bf16", choices=["bf16", "f16"], help="16-bit element type of activations and weights")
+    ap.add_argument("--calibrate-copy", action="store_true",
+                    help="also run three 1 GiB device copies, a kernel of known traffic to scale profiler byte counters with")
     return ap.parse_args()
 
 
@@ -54,7 +57,7 @@ def main():
     late = 0.3 if B >= 8192 else 0.0
     L, C, F, H = a.layers, 1024, 1536, 32
 
-    model = models.BT4Class(L, C, F, H, fp8=fp8, micro_batch=a.micro_batch, seed=0)
+    model = models.BT4Class(L, C, F, H, fp8=fp8, micro_batch=a.micro_batch, act_dtype=a.act_dtype, seed=0)
     planes = torch.from_numpy(board.random_positions(1, B, late_fraction=late)["planes"]).to(dev)
     if fp8:
         calib = torch.from_numpy(board.random_positions(2, 512)["planes"]).to(dev)
@@ -89,7 +92,7 @@ def main():
     peak = PEAK_TFLOPS["fp8" if fp8 else "bf16"]
     achieved = g["flops"] / (g["ms"] * 1e-3) / 1e12 if g["ms"] > 0 else 0.0
     roofline = {
-        "bound": "mfma", "kernel": "gemm_kernel<%s>" % ("fp8" if fp8 else "bf16"),
+        "bound": "mfma", "kernel": "gemm_dma_kernel<256x256, %s>" % ("fp8" if fp8 else a.act_dtype),
         "achieved": round(achieved, 1), "peak": peak, "unit": "TFLOP/s", "frac": round(achieved / peak, 4),
         "traffic": None,
         "avg_launch_us": round(g["ms"] * 1e3 / max(g["launches"], 1), 2), "launches": g["launches"],
@@ -99,9 +102,17 @@ def main():
         "family_ms_per_step": {k: round(v["ms"] / a.steps, 3) for k, v in prof.items()},
     }
 
+    if a.calibrate_copy:
+        src = torch.empty(1 << 30, dtype=torch.uint8, device=dev).fill_(1)
+        dst = torch.empty_like(src)
+        for _ in range(3):
+            dst.copy_(src)
+        torch.cuda.synchronize()
+        del src, dst
+
     latency = None
     if not a.no_latency:
-        lat_model = models.BT4Class(L, C, F, H, fp8=False, seed=0)
+        lat_model = models.BT4Class(L, C, F, H, fp8=False, act_dtype=a.act_dtype, seed=0)
         r = board.random_positions(3, 64, masks_leela=True)
         lp = torch.from_numpy(r["planes"]).to(dev)
         lm = torch.from_numpy(r["masks_leela"]).to(dev)
@@ -152,9 +163,9 @@ def main():
         "metric": "positions/sec, BT4-class encoder %s b%d" % ("fp8" if fp8 else "bf16", B),
         "value": round(pos_per_s, 1), "unit": "positions/s", "n_gpus": 1, "steps": a.steps, "warmup": a.warmup,
         "ms_per_step": round(ms_per_step, 3), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
-        "dtype": "fp8" if fp8 else "bf16", "data": "synthetic",
+        "dtype": "fp8" if fp8 else a.act_dtype, "data": "synthetic",
         "config": {"workload": a.workload, "layers": L, "d_model": C, "heads": H, "ffn": F, "batch": B,
-                   "micro_batch": eng.cfg.micro_batch or 4096, "positions": "seeded random playouts 0-80 plies",
+                   "micro_batch": eng.cfg.micro_batch or 4096, "act_dtype": a.act_dtype, "positions": "seeded random playouts 0-80 plies",
                    "weights": "normal(0,0.02) seed 0", "fp8_calibration_positions": 512 if fp8 else 0},
         "roofline": roofline, "cpu_baseline": cpu, "latency_b64": latency,
     }

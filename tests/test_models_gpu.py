@@ -126,6 +126,40 @@ def test_bt4class_16bit(cuda, cfg, act):
     assert top1_agreement(pol, rpol, mask) >= 0.98
 
 
+@pytest.mark.parametrize("act", ["bf16", "f16"])
+def test_bt4class_full_size(cuda, act):
+    """The benchmark model at its real size (15 layers, d=1024, 32 heads, FFN 1536) and its benchmark
+    initialisation (normal(0, 0.02), zero biases), 256 positions.
+
+    WDL meets the 1e-2 bar in both element types. The top-1 bar (99.5 %) cannot be met by any 16-bit
+    pipeline on THIS initialisation: the reference's top-1/top-2 logit gap has a median near 1e-3 while
+    the logits' standard deviation is 0.07, so rounding noise of 8 (bf16) or 11 (f16) significant bits
+    per stored activation is larger than most gaps. What the test pins instead: the logit error itself,
+    and that every position whose reference gap exceeds twice the largest logit error picks the same move."""
+    L, Cm, Fm, H = 15, 1024, 1536, 32
+    oracle = om.spec_init_(om.BT4ClassOracle(policy_leela, L, Cm, Fm, H), seed=0)
+    planes, mask = positions(256, seed=1, leela=True)
+    rpol, rwdl = oracle.forward_pv(planes)
+    m = models.BT4Class(L, Cm, Fm, H, act_dtype=act)
+    m.load_state_dict(oracle.state_dict())
+    pol, wdl = m(planes.to(cuda))
+    pol, wdl = pol.cpu(), wdl.cpu()
+    report("bt4class full size %s" % act, pol, rpol, mask, wdl, rwdl)
+    neg = (1.0 - mask.float()) * -999.0
+    top2 = (rpol + neg).topk(2, -1).values
+    gap = top2[:, 0] - top2[:, 1]
+    err = (pol - rpol).abs().max().item()
+    same = (pol + neg).argmax(-1) == (rpol + neg).argmax(-1)
+    decisive = gap > 2 * err
+    print("   logit std %.3e, median gap %.3e, max logit error %.3e, decisive positions %d of %d, agreement on them %.4f, overall %.4f"
+          % (rpol.std().item(), gap.median().item(), err, int(decisive.sum()), len(gap),
+             same[decisive].float().mean().item() if decisive.any() else 1.0, same.float().mean().item()))
+    assert rel_rms(pol, rpol) < (4e-2 if act == "bf16" else 6e-3)
+    assert (wdl - rwdl).abs().max() <= (1e-2 if act == "bf16" else 2e-3)
+    assert bool(same[decisive].all())
+    assert same.float().mean() >= (0.6 if act == "bf16" else 0.9)
+
+
 def test_bt4class_fp8_vs_emulation(cuda):
     """fp8 path against the quantise->dequantise oracle using the SAME static scales."""
     L, Cm, Fm, H = 3, 512, 768, 16
