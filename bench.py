@@ -45,8 +45,9 @@ def main():
         print("bench.py measures one GPU: positions are independent, so N GPUs run N copies of this "
               "workload with no exchange; run it with --gpus 1", file=sys.stderr)
         sys.exit(2)
+    import ctypes as ct
     import torch
-    from chessrl_amd import board, models
+    from chessrl_amd import _lib, board, models
 
     if not torch.cuda.is_available():
         print("bench.py needs an MI355X (no CPU fallback for the measured path)", file=sys.stderr)
@@ -109,6 +110,17 @@ def main():
             dst.copy_(src)
         torch.cuda.synchronize()
         del src, dst
+
+    # What the matrix cores sustain with nothing else running: all-zero operands give the clock-limited
+    # peak, random operand bits the rate under the board's power limit (the shader clock drops).
+    probe = {}
+    st = ct.c_void_p(torch.cuda.current_stream().cuda_stream)
+    for name, dt in (("fp8", _lib.FP8), ("bf16", _lib.BF16)):
+        for mode, rnd in (("zero_operands", 0), ("random_operands", 1)):
+            tf, ghz = ct.c_double(), ct.c_double()
+            _lib.check(_lib.lib().crl_probe_mfma(dt, rnd, 50000, ct.byref(tf), ct.byref(ghz), st))
+            probe["%s_%s" % (name, mode)] = {"tflops": round(tf.value, 1), "ghz": round(ghz.value, 3)}
+    roofline["mfma_probe"] = probe
 
     latency = None
     if not a.no_latency:

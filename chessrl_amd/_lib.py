@@ -70,6 +70,7 @@ SIGNATURES = {
     "crl_model_flops_per_position": (C.c_double, [_vp]),
     "crl_model_set_profiling": (_i, [_vp, _i]),
     "crl_model_get_profile": (_i, [_vp, _vp, _vp, _vp]),
+    "crl_probe_mfma": (_i, [_i, _i, _i, _vp, _vp, _vp]),
 }
 
 _lib = None

@@ -19,6 +19,7 @@ SOURCES = [
     "kernels/norm_embed.hip",
     "kernels/attention.hip",
     "kernels/heads.hip",
+    "kernels/probe.hip",
     "model.hip",
     "api.hip",
 ]

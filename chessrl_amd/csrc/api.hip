@@ -353,4 +353,11 @@ int crl_model_get_profile(crl_model* m, double* ms6, int64_t* launches6, double*
   return CRL_OK;
 }
 
+int crl_probe_mfma(int dtype, int random_bits, int iters, double* tflops, double* ghz, void* stream) {
+  if ((dtype != DT_BF16 && dtype != DT_F16 && dtype != DT_FP8) || iters <= 0 || !tflops || !ghz) return arg_fail("crl_probe_mfma: bad arguments");
+  hipError_t e = run_mfma_probe(dtype, random_bits, iters, tflops, ghz, (hipStream_t)stream);
+  if (e != hipSuccess) return hip_fail("crl_probe_mfma", e);
+  return CRL_OK;
+}
+
 }  // extern "C"

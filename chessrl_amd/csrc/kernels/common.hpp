@@ -205,6 +205,8 @@ hipError_t launch_leela_to_rl(const ScatterArgs& a, hipStream_t st);
 hipError_t launch_extract_stm(const float* planes, const uint8_t* flags, uint8_t* white_to_move, int B, hipStream_t st);
 hipError_t launch_fill_f32(float* p, float v, long n, hipStream_t st);
 hipError_t launch_convert(const float* src, void* dst, long n, int dt, float scale, hipStream_t st);
+// Back-to-back MFMAs from registers on every CU: sustained TFLOP/s and the clock it ran at.
+hipError_t run_mfma_probe(int dtype, int random_bits, int iters, double* tflops, double* ghz, hipStream_t st);
 // Slot of (query i, key j) inside a 4096-element attention bias tile.
 int attn_bias_slot_host(int i, int j);
 

@@ -180,6 +180,13 @@ double crl_model_flops_per_position(const crl_model* m);
 int crl_model_set_profiling(crl_model* m, int on);
 int crl_model_get_profile(crl_model* m, double* ms6, int64_t* launches6, double* flops6);
 
+/* Measurement probe with no counterpart in the reference: every CU runs 8 waves that issue
+ * 32x32 MFMAs back to back from registers (dtype CRL_BF16, CRL_F16 or CRL_FP8; iters rounds of 8
+ * MFMAs per wave). random_bits = 0 uses all-zero operands (clock-limited peak), 1 uses random
+ * operand bits (the rate the part sustains under its power limit). Returns the sustained
+ * TFLOP/s and the shader clock in GHz the kernel ran at. Synchronises the stream. */
+int crl_probe_mfma(int dtype, int random_bits, int iters, double* tflops, double* ghz, void* stream);
+
 #ifdef __cplusplus
 }
 #endif
