@@ -36,6 +36,7 @@ def parse():
     ap.add_argument("--layers", type=int, default=15, help=argparse.SUPPRESS)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-latency", action="store_true", help="skip the batch-64 latency leg")
+    ap.add_argument("--no-pipeline", action="store_true", help="skip the FEN-strings-to-host-results leg")
     ap.add_argument("--act-dtype", default="bf16", choices=["bf16", "f16"], help="16-bit element type of activations and weights")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run three 1 GiB device copies, a kernel of known traffic to scale profiler byte counters with")
@@ -155,6 +156,21 @@ def main():
         latency["graph_p99_ms"] = round(ts[min(len(ts) - 1, int(len(ts) * 0.99))], 3)
         del ge, lat_model
 
+    # End to end from FEN strings in host memory to probabilities, WDL and best move in host memory: host parsing,
+    # encoding and legal masks, upload, forward, masked softmax, download (chunks of the benchmark batch overlap).
+    pipeline = None
+    if not a.no_pipeline:
+        nf = 4 * B if B <= 4096 else B
+        fens = board.random_positions(5, nf, late_fraction=late, planes=False, fens=True)["fens"]
+        model.evaluate_fens(fens[:B], chunk=B)
+        res = {}
+        for name, kw in (("probs_wdl_best", dict(want_probs=True)), ("wdl_best", dict(want_probs=False))):
+            t1 = time.perf_counter()
+            model.evaluate_fens(fens, chunk=min(B, 4096), **kw)
+            res[name] = round(nf / (time.perf_counter() - t1), 1)
+        pipeline = {"positions": nf, "chunk": min(B, 4096), "unit": "positions/s", "positions_per_s": res,
+                    "includes": "FEN parse + encode + legal masks on host threads, PCIe both ways, forward, masked softmax"}
+
     cpu = None
     if not a.no_cpu:
         from chessrl_amd.vocab import policy_leela
@@ -182,7 +198,7 @@ def main():
         "config": {"workload": a.workload, "layers": L, "d_model": C, "heads": H, "ffn": F, "batch": B,
                    "micro_batch": eng.cfg.micro_batch or 4096, "act_dtype": a.act_dtype, "positions": "seeded random playouts 0-80 plies",
                    "weights": "normal(0,0.02) seed 0", "fp8_calibration_positions": 512 if fp8 else 0},
-        "roofline": roofline, "cpu_baseline": cpu, "latency_b64": latency,
+        "roofline": roofline, "cpu_baseline": cpu, "latency_b64": latency, "fen_pipeline": pipeline,
     }
     print(json.dumps(out))
 

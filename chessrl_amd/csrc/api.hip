@@ -279,7 +279,71 @@ int crl_leela_to_rl(const float* src, int64_t lds, float* dst, int64_t ldd, cons
 }
 
 // ---------------------------------------------------------------------------- models
-struct crl_model { Model impl; explicit crl_model(const crl_model_config& c) : impl(c) {} };
+// Double-buffered staging of the FEN front-end: pinned host and device buffers for two chunks,
+// one copy stream, one compute stream (both default priority), events per slot.
+struct FenPipeline {
+  int chunk = 0, vocab = 0;
+  hipStream_t copy_st = nullptr, comp_st = nullptr;
+  struct Slot {
+    uint8_t *h_ids = nullptr, *h_flags = nullptr, *h_mask = nullptr;  // pinned inputs
+    float *h_probs = nullptr, *h_wdl = nullptr; int32_t* h_best = nullptr;  // pinned outputs
+    uint8_t *d_ids = nullptr, *d_flags = nullptr, *d_mask = nullptr;
+    float *d_logits = nullptr, *d_probs = nullptr, *d_wdl = nullptr; int32_t* d_best = nullptr;
+    hipEvent_t uploaded = nullptr, done = nullptr;
+    int first = 0, count = 0;  // positions of the chunk in flight (count 0 = idle)
+  } slot[2];
+  void release() {
+    for (Slot& s : slot) {
+      (void)hipHostFree(s.h_ids); (void)hipHostFree(s.h_flags); (void)hipHostFree(s.h_mask);
+      (void)hipHostFree(s.h_probs); (void)hipHostFree(s.h_wdl); (void)hipHostFree(s.h_best);
+      (void)hipFree(s.d_ids); (void)hipFree(s.d_flags); (void)hipFree(s.d_mask);
+      (void)hipFree(s.d_logits); (void)hipFree(s.d_probs); (void)hipFree(s.d_wdl); (void)hipFree(s.d_best);
+      if (s.uploaded) (void)hipEventDestroy(s.uploaded);
+      if (s.done) (void)hipEventDestroy(s.done);
+      s = Slot();
+    }
+    if (copy_st) (void)hipStreamDestroy(copy_st);
+    if (comp_st) (void)hipStreamDestroy(comp_st);
+    copy_st = comp_st = nullptr;
+    chunk = 0;
+  }
+  hipError_t ensure(int want_chunk, int V) {
+    if (want_chunk <= chunk && V == vocab) return hipSuccess;
+    release();
+    hipError_t e;
+#define PIPE_TRY(call) do { e = (call); if (e != hipSuccess) { release(); return e; } } while (0)
+    PIPE_TRY(hipStreamCreateWithFlags(&copy_st, hipStreamNonBlocking));
+    PIPE_TRY(hipStreamCreateWithFlags(&comp_st, hipStreamNonBlocking));
+    const size_t c = (size_t)want_chunk;
+    for (Slot& s : slot) {
+      PIPE_TRY(hipHostMalloc((void**)&s.h_ids, c * 64, hipHostMallocDefault));
+      PIPE_TRY(hipHostMalloc((void**)&s.h_flags, c * 4, hipHostMallocDefault));
+      PIPE_TRY(hipHostMalloc((void**)&s.h_mask, c * V, hipHostMallocDefault));
+      PIPE_TRY(hipHostMalloc((void**)&s.h_probs, c * V * sizeof(float), hipHostMallocDefault));
+      PIPE_TRY(hipHostMalloc((void**)&s.h_wdl, c * 3 * sizeof(float), hipHostMallocDefault));
+      PIPE_TRY(hipHostMalloc((void**)&s.h_best, c * sizeof(int32_t), hipHostMallocDefault));
+      PIPE_TRY(hipMalloc((void**)&s.d_ids, c * 64));
+      PIPE_TRY(hipMalloc((void**)&s.d_flags, c * 4));
+      PIPE_TRY(hipMalloc((void**)&s.d_mask, c * V));
+      PIPE_TRY(hipMalloc((void**)&s.d_logits, c * V * sizeof(float)));
+      PIPE_TRY(hipMalloc((void**)&s.d_probs, c * V * sizeof(float)));
+      PIPE_TRY(hipMalloc((void**)&s.d_wdl, c * 3 * sizeof(float)));
+      PIPE_TRY(hipMalloc((void**)&s.d_best, c * sizeof(int32_t)));
+      PIPE_TRY(hipEventCreateWithFlags(&s.uploaded, hipEventDisableTiming));
+      PIPE_TRY(hipEventCreateWithFlags(&s.done, hipEventDisableTiming));
+    }
+#undef PIPE_TRY
+    chunk = want_chunk; vocab = V;
+    return hipSuccess;
+  }
+};
+
+struct crl_model {
+  Model impl;
+  FenPipeline pipe;
+  explicit crl_model(const crl_model_config& c) : impl(c) {}
+  ~crl_model() { pipe.release(); }
+};
 
 int crl_model_create(const crl_model_config* cfg, crl_model** out) {
   if (!cfg || !out) return arg_fail("crl_model_create: null argument");
@@ -334,6 +398,85 @@ int crl_model_forward_compact(crl_model* m, const uint8_t* ids, const uint8_t* f
                               float* wdl_logits, void* stream) {
   if (!m || !ids || !flags) return arg_fail("crl_model_forward_compact: bad arguments");
   return m->impl.forward(nullptr, ids, flags, B, policy_logits, wdl_logits, false, (hipStream_t)stream);
+}
+int crl_model_evaluate_fens(crl_model* m, const char* const* fens, int n, int chunk, float temperature, float* probs,
+                            float* wdl, int32_t* best, int threads) {
+  if (!m || n < 0 || (n && !fens) || chunk <= 0) return arg_fail("crl_model_evaluate_fens: bad arguments");
+  if (!m->impl.finalized) { set_error("crl_model_evaluate_fens: call crl_model_finalize first"); return CRL_ERR_STATE; }
+  const int V = m->impl.vocab;
+  const bool leela = m->impl.cfg.arch == CRL_ARCH_BT4CLASS, has_wdl = m->impl.cfg.arch != CRL_ARCH_GPT64;
+  if (wdl && !has_wdl) return arg_fail("crl_model_evaluate_fens: this architecture has no value head");
+  if (n == 0) return CRL_OK;
+  if (chunk > n) chunk = n;
+  FenPipeline& P = m->pipe;
+  hipError_t e = P.ensure(chunk, V);
+  if (e != hipSuccess) return hip_fail("crl_model_evaluate_fens: staging buffers", e);
+  // Results of a finished slot go from pinned staging to the caller's arrays.
+  auto drain = [&](FenPipeline::Slot& s) -> hipError_t {
+    if (s.count == 0) return hipSuccess;
+    hipError_t de = hipEventSynchronize(s.done);
+    if (de != hipSuccess) return de;
+    if (probs) std::memcpy(probs + (size_t)s.first * V, s.h_probs, sizeof(float) * (size_t)s.count * V);
+    if (wdl) std::memcpy(wdl + (size_t)s.first * 3, s.h_wdl, sizeof(float) * (size_t)s.count * 3);
+    if (best) std::memcpy(best + s.first, s.h_best, sizeof(int32_t) * (size_t)s.count);
+    s.count = 0;
+    return hipSuccess;
+  };
+  int rc = CRL_OK;
+  int k = 0;
+  for (int first = 0; first < n && rc == CRL_OK; first += chunk, ++k) {
+    FenPipeline::Slot& s = P.slot[k & 1];
+    e = drain(s);  // the chunk that used this slot two steps ago
+    if (e != hipSuccess) { rc = hip_fail("crl_model_evaluate_fens: wait", e); break; }
+    const int cnt = std::min(chunk, n - first);
+    // Host work of this chunk overlaps the device work of the previous one.
+    rc = parallel_for(cnt, threads, [&](int i) {
+      Board b;
+      int prc = parse(fens[first + i], b);
+      if (prc) return prc;
+      b.compact(s.h_ids + (size_t)i * 64, s.h_flags + (size_t)i * 4);
+      if (leela) legal_mask_leela(b, s.h_mask + (size_t)i * V);
+      else legal_mask_rl(b, s.h_mask + (size_t)i * V);
+      return 0;
+    });
+    if (rc) break;
+#define PIPE_HIP(call) do { e = (call); if (e != hipSuccess) { rc = hip_fail("crl_model_evaluate_fens", e); } } while (0)
+    PIPE_HIP(hipMemcpyAsync(s.d_ids, s.h_ids, (size_t)cnt * 64, hipMemcpyHostToDevice, P.copy_st));
+    if (rc == CRL_OK) PIPE_HIP(hipMemcpyAsync(s.d_flags, s.h_flags, (size_t)cnt * 4, hipMemcpyHostToDevice, P.copy_st));
+    if (rc == CRL_OK) PIPE_HIP(hipMemcpyAsync(s.d_mask, s.h_mask, (size_t)cnt * V, hipMemcpyHostToDevice, P.copy_st));
+    if (rc == CRL_OK) PIPE_HIP(hipEventRecord(s.uploaded, P.copy_st));
+    if (rc == CRL_OK) PIPE_HIP(hipStreamWaitEvent(P.comp_st, s.uploaded, 0));
+    if (rc) break;
+    rc = m->impl.forward(nullptr, s.d_ids, s.d_flags, cnt, s.d_logits, has_wdl ? s.d_wdl : nullptr, false, P.comp_st);
+    if (rc) break;
+    SoftmaxArgs a;
+    std::memset(&a, 0, sizeof(a));
+    a.logits = s.d_logits; a.ldl = V; a.mask = s.d_mask; a.ldm = V; a.probs = probs ? s.d_probs : nullptr; a.ldp = V;
+    a.argmax = s.d_best; a.B = cnt; a.V = V; a.temperature = temperature;
+    PIPE_HIP(launch_masked_softmax(a, P.comp_st));
+    if (rc == CRL_OK && probs) PIPE_HIP(hipMemcpyAsync(s.h_probs, s.d_probs, sizeof(float) * (size_t)cnt * V, hipMemcpyDeviceToHost, P.comp_st));
+    if (rc == CRL_OK && wdl) PIPE_HIP(hipMemcpyAsync(s.h_wdl, s.d_wdl, sizeof(float) * (size_t)cnt * 3, hipMemcpyDeviceToHost, P.comp_st));
+    if (rc == CRL_OK && best) PIPE_HIP(hipMemcpyAsync(s.h_best, s.d_best, sizeof(int32_t) * (size_t)cnt, hipMemcpyDeviceToHost, P.comp_st));
+    if (rc == CRL_OK) PIPE_HIP(hipEventRecord(s.done, P.comp_st));
+#undef PIPE_HIP
+    if (rc == CRL_OK) { s.first = first; s.count = cnt; }
+  }
+  // Leave nothing in flight, also on an error path (the staging buffers are reused by the next call).
+  const std::string err = rc ? std::string(get_error()) : std::string();
+  for (FenPipeline::Slot& s : P.slot) {
+    if (rc == CRL_OK) {
+      e = drain(s);
+      if (e != hipSuccess) rc = hip_fail("crl_model_evaluate_fens: wait", e);
+    } else {
+      s.count = 0;
+    }
+  }
+  if (rc != CRL_OK) {
+    (void)hipStreamSynchronize(P.copy_st);
+    (void)hipStreamSynchronize(P.comp_st);
+    if (!err.empty()) set_error(err);
+  }
+  return rc;
 }
 int crl_model_vocab(const crl_model* m) { return m ? m->impl.vocab : 0; }
 double crl_model_flops_per_position(const crl_model* m) { return m ? m->impl.flops_per_position() : 0.0; }

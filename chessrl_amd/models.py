@@ -223,6 +223,21 @@ class _Engine:
               "crl_model_forward_compact")
         return pol, wdl
 
+    def evaluate_fens(self, fens, T=1.0, chunk=4096, want_probs=True, want_wdl=True, threads=0):
+        """FEN strings -> (probs [n,V] or None, wdl logits [n,3] or None, best move index [n]) as CPU tensors.
+        Host encoding, upload and device work of consecutive chunks overlap inside the library."""
+        if not self.ready:
+            self.finalize()
+        n = len(fens)
+        has_wdl = want_wdl and self.cfg.arch != _lib.ARCH_GPT64
+        probs = torch.empty((n, self.vocab), dtype=torch.float32) if want_probs else None
+        wdl = torch.empty((n, 3), dtype=torch.float32) if has_wdl else None
+        best = torch.empty((n,), dtype=torch.int32)
+        arr = _lib.str_array(fens)
+        check(lib().crl_model_evaluate_fens(self.handle, arr, n, int(chunk), float(T), _ptr(probs), _ptr(wdl), _ptr(best), int(threads)),
+              "crl_model_evaluate_fens")
+        return probs, wdl, best
+
     def flops_per_position(self):
         return lib().crl_model_flops_per_position(self.handle)
 
@@ -314,6 +329,13 @@ class _ModelBase:
         if want_probs:
             pol, _ = masked_softmax(pol, legal_mask, T)
         return pol, wdl
+
+    @torch.no_grad()
+    def evaluate_fens(self, fens, T=1.0, chunk=4096, want_probs=True, want_wdl=True):
+        """Leaf evaluation from FEN strings with everything host-side done in the library: parsing, encoding,
+        legal masks, upload (overlapped with the device work of the previous chunk), masked softmax, download.
+        Returns CPU tensors (probs [n,V] or None, wdl logits [n,3] or None, best legal move index [n])."""
+        return self._engine.evaluate_fens(list(fens), T, chunk, want_probs, want_wdl)
 
     def graphed_evaluator(self, batch, T=1.0, device="cuda"):
         """Leaf evaluation for a fixed batch size captured in a HIP graph (launch-bound small batches)."""

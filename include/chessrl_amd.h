@@ -170,6 +170,17 @@ int crl_model_forward(crl_model* m, const float* planes, int B, float* policy_lo
 /* Same from the compact board form (device uint8[B,64] ids + uint8[B,4] flags). */
 int crl_model_forward_compact(crl_model* m, const uint8_t* ids, const uint8_t* flags, int B,
                               float* policy_logits, float* wdl_logits, void* stream);
+/* Host front-end of leaf evaluation: n FEN strings in host memory -> results in host memory. Replaces the per-FEN
+ * Python of model_bis.py:358-398 and new_paradigm/value.py:214-243,275-317 (encode_fens, the legal-move loop with
+ * policy_index.index per move, mask, softmax/arg-max) for whole batches. The positions are walked in chunks of
+ * `chunk`: host threads parse, encode (64 piece ids + 4 flag bytes) and build the legal mask of chunk i+1 into
+ * pinned memory while the device runs chunk i; uploads go over a copy stream of their own. probs [n, V] receives
+ * softmax((logits + (1-mask)*-999)/temperature) (one-hot at the arg-max for temperature 0), wdl [n,3] the value
+ * logits, best [n] the index of the best legal move; each may be NULL. V and the move order are those of the model
+ * (1929 / crl_policy_index, or 1858 side-to-move-frame / crl_policy_leela for CRL_ARCH_BT4CLASS). One call at a time
+ * per model; the staging buffers (2 chunks, pinned + device) stay with the model until it is destroyed. */
+int crl_model_evaluate_fens(crl_model* m, const char* const* fens, int n, int chunk, float temperature, float* probs,
+                            float* wdl, int32_t* best, int threads);
 int crl_model_vocab(const crl_model* m);
 /* 2*MAC count of one position through this model (for roofline accounting). */
 double crl_model_flops_per_position(const crl_model* m);

@@ -213,3 +213,40 @@ def test_graphed_evaluator_replays_match_eager(cuda):
         torch.cuda.synchronize()
         assert torch.equal(probs, eprobs) and torch.equal(wdl, ewdl)
         assert torch.equal(am.long(), eprobs.argmax(-1))
+
+
+@pytest.mark.parametrize("arch", ["bt4class", "bt4", "gpt"])
+def test_evaluate_fens_pipeline_equals_direct(cuda, arch):
+    """The chunked FEN front-end (host encode + upload overlapped with device work) returns exactly what the
+    direct path returns for planes and masks built one call at a time."""
+    n = 300
+    leela = arch == "bt4class"
+    r = board.random_positions(11, n, masks_rl=not leela, masks_leela=leela, fens=True)
+    fens = r["fens"]
+    planes = torch.from_numpy(r["planes"]).to(cuda)
+    mask = torch.from_numpy(r["masks_leela" if leela else "masks_rl"]).to(cuda)
+    if arch == "bt4class":
+        m = models.BT4Class(2, 256, 384, 8)
+    elif arch == "bt4":
+        m = models.BT4(2, 256, 368, 4)
+    else:
+        m = models.GPT(models.GPTConfig(block_size=256, vocab_size=1929, n_layer=2, n_head=8, n_embd=256))
+    pol, wdl = m._engine.forward(planes)
+    ref_probs, ref_best = models.masked_softmax(pol, mask, 1.0, want_probs=True)
+    for chunk in (64, 128, 1000):     # ragged last chunk, several chunks in flight, one chunk
+        probs, w, best = m.evaluate_fens(fens, T=1.0, chunk=chunk)
+        assert torch.equal(probs, ref_probs.cpu())
+        assert torch.equal(best, ref_best.cpu().to(torch.int32))
+        if arch == "gpt":
+            assert w is None
+        else:
+            assert torch.equal(w, wdl.cpu())
+    # arg-max only, temperature 0, and the error path leaves the model usable
+    _, _, best0 = m.evaluate_fens(fens[:10], T=0.0, chunk=4, want_probs=False, want_wdl=False)
+    assert torch.equal(best0, ref_best.cpu().to(torch.int32)[:10])
+    from chessrl_amd._lib import CrlError
+    with pytest.raises(CrlError):
+        m.evaluate_fens(fens[:5] + ["not a fen"] + fens[5:9], chunk=4)
+    probs, _, _ = m.evaluate_fens(fens[:7], chunk=4)
+    assert torch.equal(probs, ref_probs.cpu()[:7])
+    assert m.evaluate_fens([], chunk=4)[2].numel() == 0
