@@ -278,6 +278,37 @@ int crl_leela_to_rl(const float* src, int64_t lds, float* dst, int64_t ldd, cons
   return e == hipSuccess ? CRL_OK : hip_fail("crl_leela_to_rl", e);
 }
 
+int crl_attention_causal(const void* q, int64_t ldq, const void* k, int64_t ldk, const void* v, int64_t ldv, int in_dtype, void* out,
+                         int64_t ldo, int out_dtype, float out_scale, int B, int H, int head_dim, int T, float scale, float* amax, void* stream) {
+  if (!q || !k || !v || !out || B < 0 || H <= 0 || T < 1) return arg_fail("crl_attention_causal: bad arguments");
+  AttnArgs a;
+  std::memset(&a, 0, sizeof(a));
+  a.q = q; a.k = k; a.v = v; a.ldq = ldq; a.ldk = ldk; a.ldv = ldv; a.in_dtype = in_dtype; a.out = out; a.ldo = ldo;
+  a.out_dtype = out_dtype; a.out_scale = out_scale; a.B = B; a.H = H; a.mode = ATTN_CAUSAL; a.scale = scale; a.amax = amax;
+  a.T = T == 64 ? 0 : T;
+  hipError_t e = launch_attention(a, head_dim, (hipStream_t)stream);
+  if (e == hipErrorInvalidValue) return arg_fail("crl_attention_causal: head_dim must be 32 or 64, in_dtype bf16/f16, out_dtype in_dtype or fp8, strides multiples of 8, T <= 4096");
+  return e == hipSuccess ? CRL_OK : hip_fail("crl_attention_causal", e);
+}
+int crl_token_scores(const float* logits, int64_t ldl, const float* ref_logits, int64_t ldr, const int64_t* target, int rows, int V,
+                     int64_t ignore_index, float* logp, float* ref_logp, float* kl, void* stream) {
+  if (!logits || rows < 0 || V <= 0) return arg_fail("crl_token_scores: bad arguments");
+  if (V > 2048) return arg_fail("crl_token_scores: at most 2048 classes");
+  if ((kl || ref_logp) && !ref_logits) return arg_fail("crl_token_scores: reference logits missing");
+  if ((logp || ref_logp) && !target) return arg_fail("crl_token_scores: targets missing");
+  TokenScoreArgs a;
+  std::memset(&a, 0, sizeof(a));
+  a.logits = logits; a.ldl = ldl; a.ref = ref_logits; a.ldr = ldr; a.target = target; a.rows = rows; a.V = V;
+  a.ignore_index = ignore_index; a.logp = logp; a.ref_logp = ref_logp; a.kl = kl;
+  hipError_t e = launch_token_scores(a, (hipStream_t)stream);
+  return e == hipSuccess ? CRL_OK : hip_fail("crl_token_scores", e);
+}
+int crl_masked_nll_mean(const float* logp, const int64_t* target, int64_t ignore_index, int rows, float* out, void* stream) {
+  if (!logp || !target || !out || rows < 0) return arg_fail("crl_masked_nll_mean: bad arguments");
+  hipError_t e = launch_masked_nll_mean(logp, target, ignore_index, rows, out, (hipStream_t)stream);
+  return e == hipSuccess ? CRL_OK : hip_fail("crl_masked_nll_mean", e);
+}
+
 // ---------------------------------------------------------------------------- models
 // Double-buffered staging of the FEN front-end: pinned host and device buffers for two chunks,
 // one copy stream, one compute stream (both default priority), events per slot.
@@ -398,6 +429,11 @@ int crl_model_forward_compact(crl_model* m, const uint8_t* ids, const uint8_t* f
                               float* wdl_logits, void* stream) {
   if (!m || !ids || !flags) return arg_fail("crl_model_forward_compact: bad arguments");
   return m->impl.forward(nullptr, ids, flags, B, policy_logits, wdl_logits, false, (hipStream_t)stream);
+}
+int crl_model_forward_tokens(crl_model* m, const float* planes, const int64_t* idx, int B, int t, float* last_logits,
+                             float* all_logits, void* stream) {
+  if (!m || !planes) return arg_fail("crl_model_forward_tokens: bad arguments");
+  return m->impl.forward_tokens(planes, nullptr, nullptr, idx, t, B, last_logits, all_logits, nullptr, false, (hipStream_t)stream);
 }
 int crl_model_evaluate_fens(crl_model* m, const char* const* fens, int n, int chunk, float temperature, float* probs,
                             float* wdl, int32_t* best, int threads) {

@@ -322,6 +322,207 @@ __global__ void __launch_bounds__(64 * AttnWaves<MODE>::N) attention_kernel(cons
   }
 }
 
+// Causal attention over T > 64 tokens per position (the board tokens followed by move tokens,
+// model_bis.py:171-199 with F.scaled_dot_product_attention(is_causal=True) at :71). One wave per
+// (position, head, block of 64 queries) walks the key blocks 0..own block with the running
+// maximum and sum of a streaming softmax. In the transposed layout a lane owns one query in the
+// score tile and in the output tile alike, so the rescale of the running output is one
+// multiply per register with the lane's own factor.
+template <int HS, int OUT_FP8, int IN_DT>
+__global__ void __launch_bounds__(256) causal_long_kernel(const AttnArgs a) {
+  typedef Half16<IN_DT> H16;
+  typedef typename H16::vec hvec;
+  constexpr int KS = HS / 16;
+  constexpr int DT_TILES = HS / 32;
+  __shared__ __align__(16) uint16_t s_vt[4][HS * VT_STRIDE];
+
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  const int lr = lane & 31, g = lane >> 5;
+  const int T = a.T, nqb = (T + 63) >> 6;
+  const int unit = blockIdx.x * 4 + wave;
+  if (unit >= a.B * a.H * nqb) return;
+  // Longest units (last query block) first: they walk the most key blocks.
+  const int qb = nqb - 1 - unit / (a.B * a.H);
+  const int bh = unit % (a.B * a.H);
+  const int b = bh / a.H, h = bh - b * a.H;
+  const long row0 = (long)b * T;
+
+  const uint16_t* qp = reinterpret_cast<const uint16_t*>(a.q) + row0 * a.ldq + h * HS;
+  const uint16_t* kp = reinterpret_cast<const uint16_t*>(a.k) + row0 * a.ldk + h * HS;
+  const uint16_t* vp = reinterpret_cast<const uint16_t*>(a.v) + row0 * a.ldv + h * HS;
+  uint16_t* vt = s_vt[wave];
+  auto clampT = [&](int t) { return t < T ? t : T - 1; };   // rows past the end re-read the last token
+
+  hvec qf[2][KS];
+#pragma unroll
+  for (int t = 0; t < 2; ++t)
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks)
+      qf[t][ks] = *reinterpret_cast<const hvec*>(qp + (long)clampT(64 * qb + 32 * t + lr) * a.ldq + 16 * ks + 8 * g);
+
+  float run_m[2] = {-INFINITY, -INFINITY}, run_l[2] = {0.f, 0.f};
+  f32x16_t o[DT_TILES][2];
+#pragma unroll
+  for (int dt = 0; dt < DT_TILES; ++dt)
+#pragma unroll
+    for (int it = 0; it < 2; ++it)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) o[dt][it][r] = 0.f;
+
+  for (int kb = 0; kb <= qb; ++kb) {
+    // ---- V block -> V^T in LDS (the previous block's reads are complete: same wave, in order)
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+    {
+      constexpr int DC = HS / 8;
+      constexpr int PASSES = (16 * DC) / 64;
+#pragma unroll
+      for (int p = 0; p < PASSES; ++p) {
+        const int id = p * 64 + lane;
+        const int jq = id / DC, dc = id - jq * DC;
+        uint4 rows[4];
+#pragma unroll
+        for (int t = 0; t < 4; ++t) rows[t] = *reinterpret_cast<const uint4*>(vp + (long)clampT(64 * kb + 4 * jq + t) * a.ldv + 8 * dc);
+        const uint32_t* w0 = reinterpret_cast<const uint32_t*>(&rows[0]);
+        const uint32_t* w1 = reinterpret_cast<const uint32_t*>(&rows[1]);
+        const uint32_t* w2 = reinterpret_cast<const uint32_t*>(&rows[2]);
+        const uint32_t* w3 = reinterpret_cast<const uint32_t*>(&rows[3]);
+#pragma unroll
+        for (int e2 = 0; e2 < 4; ++e2) {
+          uint2 lo = make_uint2((w0[e2] & 0xffffu) | (w1[e2] << 16), (w2[e2] & 0xffffu) | (w3[e2] << 16));
+          uint2 hi = make_uint2((w0[e2] >> 16) | (w1[e2] & 0xffff0000u), (w2[e2] >> 16) | (w3[e2] & 0xffff0000u));
+          *reinterpret_cast<uint2*>(vt + (8 * dc + 2 * e2) * VT_STRIDE + 4 * jq) = lo;
+          *reinterpret_cast<uint2*>(vt + (8 * dc + 2 * e2 + 1) * VT_STRIDE + 4 * jq) = hi;
+        }
+      }
+    }
+    // ---- scores of this key block
+    hvec kf[2][KS];
+#pragma unroll
+    for (int t = 0; t < 2; ++t)
+#pragma unroll
+      for (int ks = 0; ks < KS; ++ks)
+        kf[t][ks] = *reinterpret_cast<const hvec*>(kp + (long)clampT(64 * kb + 32 * t + lr) * a.ldk + 16 * ks + 8 * g);
+    f32x16_t s[2][2];
+#pragma unroll
+    for (int jt = 0; jt < 2; ++jt)
+#pragma unroll
+      for (int it = 0; it < 2; ++it) {
+#pragma unroll
+        for (int r = 0; r < 16; ++r) s[jt][it][r] = 0.f;
+#pragma unroll
+        for (int ks = 0; ks < KS; ++ks) s[jt][it] = H16::mfma(kf[jt][ks], qf[it][ks], s[jt][it]);
+      }
+    const bool edge = kb == qb;   // only the diagonal block needs the causal test; keys past T sit in it too
+#pragma unroll
+    for (int it = 0; it < 2; ++it) {
+      const int i = 64 * qb + 32 * it + lr;
+      float mx = run_m[it];
+#pragma unroll
+      for (int jt = 0; jt < 2; ++jt)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+          const int j = 64 * kb + 32 * jt + 8 * (r >> 2) + 4 * g + (r & 3);
+          float x = s[jt][it][r] * a.scale;
+          if (edge && (j > i || j >= T)) x = -INFINITY;
+          s[jt][it][r] = x;
+          mx = fmaxf(mx, x);
+        }
+      mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+      // Key 0 is visible to every query, so mx is finite from the first block on.
+      const float alpha = __expf(run_m[it] - mx);
+      float sum = 0.f;
+#pragma unroll
+      for (int jt = 0; jt < 2; ++jt)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+          const float p = __expf(s[jt][it][r] - mx);
+          s[jt][it][r] = p;
+          sum += p;
+        }
+      sum += __shfl_xor(sum, 32, 64);
+      run_l[it] = run_l[it] * alpha + sum;
+      run_m[it] = mx;
+#pragma unroll
+      for (int dt = 0; dt < DT_TILES; ++dt)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) o[dt][it][r] *= alpha;
+    }
+    // ---- O^T += V^T · P^T
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+#pragma unroll
+    for (int k4 = 0; k4 < 4; ++k4) {
+      const int jt = k4 >> 1, kh = k4 & 1;
+      hvec pf[2];
+#pragma unroll
+      for (int it = 0; it < 2; ++it)
+#pragma unroll
+        for (int e = 0; e < 8; ++e) pf[it][e] = (typename H16::elem)s[jt][it][8 * kh + e];
+#pragma unroll
+      for (int dt = 0; dt < DT_TILES; ++dt) {
+        const uint16_t* vrow = vt + (32 * dt + lr) * VT_STRIDE + 16 * k4 + 4 * g;
+        const uint2 lo = *reinterpret_cast<const uint2*>(vrow);
+        const uint2 hi = *reinterpret_cast<const uint2*>(vrow + 8);
+        const uint4 packed = make_uint4(lo.x, lo.y, hi.x, hi.y);
+        const hvec vf = __builtin_bit_cast(hvec, packed);
+#pragma unroll
+        for (int it = 0; it < 2; ++it) o[dt][it] = H16::mfma(vf, pf[it], o[dt][it]);
+      }
+    }
+  }
+
+  float am = 0.f;
+#pragma unroll
+  for (int it = 0; it < 2; ++it) {
+    const int i = 64 * qb + 32 * it + lr;
+    if (i >= T) continue;
+    const float inv_l = 1.0f / run_l[it];
+    const long row = row0 + i;
+#pragma unroll
+    for (int dt = 0; dt < DT_TILES; ++dt)
+#pragma unroll
+      for (int rq = 0; rq < 4; ++rq) {
+        const int d = 32 * dt + 8 * rq + 4 * g;
+        float v[4];
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          v[e] = o[dt][it][4 * rq + e] * inv_l;
+          am = fmaxf(am, fabsf(v[e]));
+        }
+        const long off = row * a.ldo + h * HS + d;
+        if constexpr (OUT_FP8) {
+          *reinterpret_cast<uint32_t*>(reinterpret_cast<uint8_t*>(a.out) + off) =
+              pack_fp8x4(v[0] * a.out_scale, v[1] * a.out_scale, v[2] * a.out_scale, v[3] * a.out_scale);
+        } else {
+          *reinterpret_cast<uint2*>(reinterpret_cast<uint16_t*>(a.out) + off) = make_uint2(H16::pack2(v[0], v[1]), H16::pack2(v[2], v[3]));
+        }
+      }
+  }
+  if (a.amax) {
+    am = wave_max(am);
+    if (lane == 0) atomic_amax(a.amax, am);
+  }
+}
+
+template <int HS, int IN_DT>
+static hipError_t launch_causal_long_dt(const AttnArgs& a, hipStream_t st) {
+  const long units = (long)a.B * a.H * ((a.T + 63) / 64);
+  const dim3 grid((unsigned)((units + 3) / 4)), block(256);
+  if (a.out_dtype == DT_FP8) hipLaunchKernelGGL((causal_long_kernel<HS, 1, IN_DT>), grid, block, 0, st, a);
+  else if (a.out_dtype == IN_DT) hipLaunchKernelGGL((causal_long_kernel<HS, 0, IN_DT>), grid, block, 0, st, a);
+  else return hipErrorInvalidValue;
+  return hipGetLastError();
+}
+template <int HS>
+static hipError_t launch_causal_long(const AttnArgs& a, hipStream_t st) {
+  if (a.in_dtype == DT_F16) return launch_causal_long_dt<HS, DT_F16>(a, st);
+  if (a.in_dtype == DT_BF16) return launch_causal_long_dt<HS, DT_BF16>(a, st);
+  return hipErrorInvalidValue;
+}
+
 template <int HS, int MODE, int IN_DT>
 static hipError_t launch_attn_dt(const AttnArgs& a, hipStream_t st) {
   constexpr int NW = AttnWaves<MODE>::N;
@@ -358,6 +559,12 @@ hipError_t launch_attention(const AttnArgs& a, int head_dim, hipStream_t st) {
     return hipErrorInvalidValue;
   if (a.mode == ATTN_BIAS && !a.bias) return hipErrorInvalidValue;
   if (a.mode == ATTN_RELSHIFT && (!a.pos || !a.u_bias || !a.v_bias)) return hipErrorInvalidValue;
+  if (a.T != 0 && a.T != 64) {
+    if (a.mode != ATTN_CAUSAL || a.T < 1 || a.T > 4096) return hipErrorInvalidValue;
+    if (head_dim == 32) return launch_causal_long<32>(a, st);
+    if (head_dim == 64) return launch_causal_long<64>(a, st);
+    return hipErrorInvalidValue;
+  }
   if (head_dim == 32) return launch_attn_hs<32>(a, st);
   if (head_dim == 64) return launch_attn_hs<64>(a, st);
   return hipErrorInvalidValue;

@@ -138,6 +138,16 @@ struct EmbedArgs {
   float* amax;
   int tokens, C, out_dtype, act;
   float eps, fp8_scale;
+  int out_T;            // rows per position in `out` (0 or 64: dense); token s of position b is written at row b*out_T + s
+};
+
+// Rows 64.. of a position that also carries move tokens: out[b*T + 64 + j] = wte[idx[b][j]] + pe[64 + j].
+struct TokenEmbedArgs {
+  const int64_t* idx;   // [B, t]
+  const float* wte;     // [V, C]
+  const float* pe;      // [>= T, C]
+  void* out;            // [B*T, C] in out_dtype
+  int B, t, T, C, V, out_dtype;
 };
 
 enum AttnMode : int { ATTN_PLAIN = 0, ATTN_CAUSAL = 1, ATTN_BIAS = 2, ATTN_RELSHIFT = 3 };
@@ -153,6 +163,7 @@ struct AttnArgs {
   long ldo;
   float* amax;
   int B, H, mode, out_dtype;
+  int T;                // tokens per position; 0 or 64 for the single-tile kernel, more only with ATTN_CAUSAL
   int in_dtype;         // DT_BF16 or DT_F16: element type of q, k, v, bias and pos
   float scale, out_scale;
 };
@@ -183,6 +194,18 @@ struct SoftmaxArgs {
   float temperature;               // 0 -> one-hot at the arg-max
 };
 
+// Per-row log-softmax statistics of a logits matrix.
+struct TokenScoreArgs {
+  const float* logits; long ldl;    // [rows, V]
+  const float* ref; long ldr;       // optional second logits matrix [rows, V]
+  const int64_t* target;            // optional [rows]
+  float* logp;                      // optional [rows]: log_softmax(logits)[target] (0 where target is ignore_index or out of range)
+  float* ref_logp;                  // optional [rows]: log_softmax(ref)[target]
+  float* kl;                        // optional [rows]: sum_v softmax(logits)*(log_softmax(logits)-log_softmax(ref))
+  int rows, V;
+  long ignore_index;
+};
+
 struct ScatterArgs {
   const float* src; long lds;       // [B, 1858]
   float* dst; long ldd;             // [B, 1929], fully written (zeros where no source)
@@ -198,6 +221,10 @@ struct ScatterArgs {
 hipError_t launch_gemm(GemmArgs a, int in_dt, int out_dt, int tile, hipStream_t st);
 hipError_t launch_layernorm(const LayerNormArgs& a, hipStream_t st);
 hipError_t launch_embed(const EmbedArgs& a, hipStream_t st);
+hipError_t launch_token_embed(const TokenEmbedArgs& a, hipStream_t st);
+hipError_t launch_token_scores(const TokenScoreArgs& a, hipStream_t st);
+// mean of -logp over rows whose target is not ignore_index, in a fixed summation order; *out = 0 if there is none.
+hipError_t launch_masked_nll_mean(const float* logp, const int64_t* target, long ignore_index, int rows, float* out, hipStream_t st);
 hipError_t launch_attention(const AttnArgs& a, int head_dim, hipStream_t st);
 hipError_t launch_policy_qk(const PolicyQKArgs& a, hipStream_t st);
 hipError_t launch_masked_softmax(const SoftmaxArgs& a, hipStream_t st);

@@ -210,6 +210,105 @@ __global__ void extract_stm_kernel(const float* planes, const uint8_t* flags, ui
   if (b >= B) return;
   out[b] = planes ? (planes[(long)b * 64 * 19 + 12] > 0.5f ? 1 : 0) : (flags[(long)b * 4] ? 1 : 0);
 }
+// ---- per-row log-softmax statistics ---------------------------------------------------------
+// Serves the cross-entropy of GPT.forward(compute_loss=True) (model_bis.py:192-193) and the
+// scoring terms of GRPO (grpo_refactored.py:337-342: log_softmax of the policy and the frozen
+// reference model, the per-token KL and the log-probabilities of the tokens taken).
+// One wave per row; the row (and the reference row) stays in registers, so each logit is read
+// from memory once. V <= 64 * TS_VPL.
+constexpr int TS_VPL = 32;
+
+template <int WITH_REF>
+__global__ void __launch_bounds__(256) token_score_kernel(const TokenScoreArgs a) {
+  const int lane = threadIdx.x & 63;
+  const int row = blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (row >= a.rows) return;
+  const float* x = a.logits + (long)row * a.ldl;
+  const float* y = WITH_REF ? a.ref + (long)row * a.ldr : nullptr;
+  float xv[TS_VPL], yv[WITH_REF ? TS_VPL : 1];
+  float mx = -INFINITY, my = -INFINITY;
+#pragma unroll
+  for (int i = 0; i < TS_VPL; ++i) {
+    const int c = i * 64 + lane;
+    xv[i] = c < a.V ? x[c] : -INFINITY;
+    mx = fmaxf(mx, xv[i]);
+    if constexpr (WITH_REF) {
+      yv[i] = c < a.V ? y[c] : -INFINITY;
+      my = fmaxf(my, yv[i]);
+    }
+  }
+  mx = wave_max(mx);
+  if constexpr (WITH_REF) my = wave_max(my);
+  float sx = 0.f, sy = 0.f;
+#pragma unroll
+  for (int i = 0; i < TS_VPL; ++i) {
+    sx += __expf(xv[i] - mx);
+    if constexpr (WITH_REF) sy += __expf(yv[i] - my);
+  }
+  sx = wave_sum(sx);
+  const float lse_x = mx + __logf(sx);
+  float lse_y = 0.f;
+  if constexpr (WITH_REF) {
+    sy = wave_sum(sy);
+    lse_y = my + __logf(sy);
+    if (a.kl) {
+      float k = 0.f;
+#pragma unroll
+      for (int i = 0; i < TS_VPL; ++i) {
+        const int c = i * 64 + lane;
+        if (c < a.V) {
+          const float lp = xv[i] - lse_x;
+          k += __expf(lp) * (lp - (yv[i] - lse_y));
+        }
+      }
+      k = wave_sum(k);
+      if (lane == 0) a.kl[row] = k;
+    }
+  }
+  if (a.target && (a.logp || a.ref_logp)) {
+    const long t = a.target[row];
+    const bool ok = t != a.ignore_index && t >= 0 && t < a.V;
+    if (lane == 0) {
+      if (a.logp) a.logp[row] = ok ? x[t] - lse_x : 0.f;
+      if (WITH_REF && a.ref_logp) a.ref_logp[row] = ok ? y[t] - lse_y : 0.f;
+    }
+  }
+}
+
+hipError_t launch_token_scores(const TokenScoreArgs& a, hipStream_t st) {
+  if (a.rows <= 0) return hipSuccess;
+  if (!a.logits || a.V <= 0 || a.V > 64 * TS_VPL) return hipErrorInvalidValue;
+  if ((a.kl || a.ref_logp) && !a.ref) return hipErrorInvalidValue;
+  const dim3 grid((a.rows + 3) / 4), block(256);
+  if (a.ref) hipLaunchKernelGGL((token_score_kernel<1>), grid, block, 0, st, a);
+  else hipLaunchKernelGGL((token_score_kernel<0>), grid, block, 0, st, a);
+  return hipGetLastError();
+}
+
+// One workgroup, fixed order: every thread sums a strided slice, then a tree over the workgroup.
+__global__ void __launch_bounds__(256) masked_nll_mean_kernel(const float* logp, const int64_t* target, long ignore_index, int rows, float* out) {
+  __shared__ float s_sum[256];
+  __shared__ int s_cnt[256];
+  float sum = 0.f;
+  int cnt = 0;
+  for (int r = threadIdx.x; r < rows; r += 256)
+    if (target[r] != ignore_index) { sum -= logp[r]; ++cnt; }
+  s_sum[threadIdx.x] = sum;
+  s_cnt[threadIdx.x] = cnt;
+  __syncthreads();
+  for (int o = 128; o > 0; o >>= 1) {
+    if ((int)threadIdx.x < o) { s_sum[threadIdx.x] += s_sum[threadIdx.x + o]; s_cnt[threadIdx.x] += s_cnt[threadIdx.x + o]; }
+    __syncthreads();
+  }
+  if (threadIdx.x == 0) out[0] = s_cnt[0] > 0 ? s_sum[0] / (float)s_cnt[0] : 0.f;
+}
+
+hipError_t launch_masked_nll_mean(const float* logp, const int64_t* target, long ignore_index, int rows, float* out, hipStream_t st) {
+  if (!logp || !target || !out || rows < 0) return hipErrorInvalidValue;
+  hipLaunchKernelGGL(masked_nll_mean_kernel, dim3(1), dim3(256), 0, st, logp, target, ignore_index, rows, out);
+  return hipGetLastError();
+}
+
 hipError_t launch_extract_stm(const float* planes, const uint8_t* flags, uint8_t* white_to_move, int B, hipStream_t st) {
   if (B <= 0) return hipSuccess;
   hipLaunchKernelGGL(extract_stm_kernel, dim3((B + 255) / 256), dim3(256), 0, st, planes, flags, white_to_move, B);

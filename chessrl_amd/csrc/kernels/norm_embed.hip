@@ -198,6 +198,7 @@ __global__ void __launch_bounds__(256) embed_kernel(const EmbedArgs a) {
     }
   }
   ln_finish<VPL>(x, lane, a.C, a.ln_g, a.ln_b, a.eps, y);
+  const long orow = a.out_T > 64 ? (long)(tok >> 6) * a.out_T + sqr : (long)tok;
   float am = 0.f;
 #pragma unroll
   for (int i = 0; i < VPL; ++i) {
@@ -214,8 +215,8 @@ __global__ void __launch_bounds__(256) embed_kernel(const EmbedArgs a) {
 #pragma unroll
         for (int e = 0; e < 8; ++e) y[i][e] += pe[e];
       }
-      store8(a.out, (long)tok * a.C + col, y[i], a.out_dtype);
-      if (a.out_fp8) store8_fp8(a.out_fp8, (long)tok * a.C + col, y[i], a.fp8_scale);
+      store8(a.out, orow * a.C + col, y[i], a.out_dtype);
+      if (a.out_fp8) store8_fp8(a.out_fp8, orow * a.C + col, y[i], a.fp8_scale);
       if (a.amax) {
 #pragma unroll
         for (int e = 0; e < 8; ++e) am = fmaxf(am, fabsf(y[i][e]));
@@ -226,6 +227,29 @@ __global__ void __launch_bounds__(256) embed_kernel(const EmbedArgs a) {
     am = wave_max(am);
     if (lane == 0) atomic_amax(a.amax, am);
   }
+}
+
+// One workgroup per (position, move token).
+__global__ void __launch_bounds__(256) token_embed_kernel(const TokenEmbedArgs a) {
+  const int b = blockIdx.x / a.t, j = blockIdx.x - b * a.t;
+  long id = a.idx[(long)b * a.t + j];
+  id = id < 0 ? 0 : id >= a.V ? a.V - 1 : id;
+  const float* w = a.wte + id * a.C;
+  const float* pe = a.pe + (long)(64 + j) * a.C;
+  const long row = (long)b * a.T + 64 + j;
+  for (int c = threadIdx.x; c < a.C; c += 256) {
+    const float v = w[c] + pe[c];
+    if (a.out_dtype == DT_F32) reinterpret_cast<float*>(a.out)[row * a.C + c] = v;
+    else if (a.out_dtype == DT_BF16) reinterpret_cast<uint16_t*>(a.out)[row * a.C + c] = f32_to_bf16_bits(v);
+    else reinterpret_cast<uint16_t*>(a.out)[row * a.C + c] = f32_to_f16_bits(v);
+  }
+}
+
+hipError_t launch_token_embed(const TokenEmbedArgs& a, hipStream_t st) {
+  if (a.B <= 0 || a.t <= 0) return hipSuccess;
+  if (!a.idx || !a.wte || !a.pe || !a.out || a.T != 64 + a.t || a.out_dtype == DT_FP8) return hipErrorInvalidValue;
+  hipLaunchKernelGGL(token_embed_kernel, dim3(a.B * a.t), dim3(256), 0, st, a);
+  return hipGetLastError();
 }
 
 hipError_t launch_embed(const EmbedArgs& a, hipStream_t st) {

@@ -14,6 +14,7 @@
 
 #include <cmath>
 #include <cstdio>
+#include <algorithm>
 #include <cstring>
 
 namespace crl {
@@ -108,7 +109,9 @@ int Model::set_weight(const char* key, const float* data, long numel) {
     if (e.first != k) continue;
     const bool ok = (k == "pe") ? numel >= e.second : numel == e.second;
     if (!ok) { set_error("set_weight: " + k + " has " + std::to_string(numel) + " elements, expected " + std::to_string(e.second)); return CRL_ERR_ARG; }
-    host[k].assign(data, data + e.second);
+    // The positional table may carry more rows than the 64 board tokens (block_size rows, model_bis.py:141-146).
+    const long keep = (k == "pe") ? numel - numel % cfg.d_model : e.second;
+    host[k].assign(data, data + keep);
     finalized = false;
     return CRL_OK;
   }
@@ -193,6 +196,8 @@ int Model::finalize() {
   }
   if (cfg.arch == CRL_ARCH_GPT64) {
     UP(w("pe"), DT_F32, pe_f32);
+    pe_rows = (int)(w("pe").size() / (size_t)C);
+    UP(w("lm_head.weight"), DT_F32, wte_f32);   // token embedding, tied to the output head (model_bis.py:148)
     for (int i = 0; i < cfg.n_layer; ++i) {
       Layer& ly = layers[i];
       const std::string p = lkey("transformer.h.%d.", i);
@@ -426,26 +431,40 @@ float Model::act_scale(int layer, int slot) const {
 
 int Model::forward(const float* planes, const uint8_t* ids, const uint8_t* flags, int B, float* policy, float* wdl,
                    bool calibrate, hipStream_t st) {
+  if (!policy) { set_error("forward: bad arguments"); return CRL_ERR_ARG; }
+  return forward_tokens(planes, ids, flags, nullptr, 0, B, policy, nullptr, wdl, calibrate, st);
+}
+
+int Model::forward_tokens(const float* planes, const uint8_t* ids, const uint8_t* flags, const int64_t* idx, int t, int B,
+                          float* policy, float* all_logits, float* wdl, bool calibrate, hipStream_t st) {
   if (!finalized) { set_error("forward: call crl_model_finalize first"); return CRL_ERR_STATE; }
-  if (B < 0 || (!planes && !(ids && flags)) || !policy) { set_error("forward: bad arguments"); return CRL_ERR_ARG; }
-  const int mbmax = cfg.micro_batch;
-  int rc = ensure_ws(B < mbmax ? B : mbmax);
+  if (B < 0 || t < 0 || (!planes && !(ids && flags)) || (!policy && !all_logits)) { set_error("forward: bad arguments"); return CRL_ERR_ARG; }
+  if ((t > 0 || all_logits) && cfg.arch != CRL_ARCH_GPT64) { set_error("forward: move tokens and per-token logits exist only for CRL_ARCH_GPT64"); return CRL_ERR_ARG; }
+  if (t > 0 && !idx) { set_error("forward: move tokens missing"); return CRL_ERR_ARG; }
+  const int T = 64 + t;
+  if (t > 0 && T > pe_rows) { set_error("forward: " + std::to_string(T) + " tokens exceed the " + std::to_string(pe_rows) + " rows of the positional table"); return CRL_ERR_ARG; }
+  // The workspace is counted in 64-token units; longer positions take proportionally fewer per micro-batch.
+  const int mbmax = std::max(1, (int)((long)cfg.micro_batch * 64 / T));
+  const int mb0 = B < mbmax ? B : mbmax;
+  int rc = ensure_ws((int)(((long)mb0 * T + 63) / 64));
   if (rc) return rc;
   for (int b0 = 0; b0 < B; b0 += mbmax) {
     const int mb = (B - b0) < mbmax ? (B - b0) : mbmax;
     rc = forward_chunk(planes ? planes + (size_t)b0 * 64 * 19 : nullptr, ids ? ids + (size_t)b0 * 64 : nullptr,
-                       flags ? flags + (size_t)b0 * 4 : nullptr, mb, policy + (size_t)b0 * vocab, wdl ? wdl + (size_t)b0 * 3 : nullptr,
-                       calibrate, st);
+                       flags ? flags + (size_t)b0 * 4 : nullptr, idx ? idx + (size_t)b0 * t : nullptr, t, mb,
+                       policy ? policy + (size_t)b0 * vocab : nullptr, all_logits ? all_logits + (size_t)b0 * T * vocab : nullptr,
+                       wdl ? wdl + (size_t)b0 * 3 : nullptr, calibrate, st);
     if (rc) return rc;
   }
   prof_collect(st);
   return CRL_OK;
 }
 
-int Model::forward_chunk(const float* planes, const uint8_t* ids, const uint8_t* flags, int mb, float* policy, float* wdl,
-                         bool calibrate, hipStream_t st) {
+int Model::forward_chunk(const float* planes, const uint8_t* ids, const uint8_t* flags, const int64_t* idx, int t, int mb,
+                         float* policy, float* all_logits, float* wdl, bool calibrate, hipStream_t st) {
   const int C = cfg.d_model, F = cfg.d_ff, H = cfg.n_head, L = cfg.n_layer, hs = C / H;
-  const int M = mb * 64;
+  const int T = 64 + t;          // tokens per position: the board, then t move tokens (CRL_ARCH_GPT64 only)
+  const int M = mb * T;
   const bool f8 = cfg.fp8 && !calibrate;
   const int hd = cfg.head_dtype, ad = cfg.act_dtype;
   const bool gpt = cfg.arch == CRL_ARCH_GPT64;
@@ -462,12 +481,22 @@ int Model::forward_chunk(const float* planes, const uint8_t* ids, const uint8_t*
     e.planes = planes; e.ids = ids; e.flags = flags;
     e.w1t = emb_w1t; e.b1 = emb_b1; e.ln_g = emb_g; e.ln_b = emb_b; e.gate_a_exp = gate_a_exp; e.gate_b = gate_b;
     e.pe = gpt ? pe_f32 : nullptr;
-    e.out = ws.x; e.out_dtype = (L == 0 && !gpt) ? hd : xdt; e.tokens = M; e.C = C; e.act = ACT_GELU; e.eps = cfg.eps;
+    e.out = ws.x; e.out_dtype = (L == 0 && !gpt) ? hd : xdt; e.tokens = mb * 64; e.C = C; e.act = ACT_GELU; e.eps = cfg.eps;
+    e.out_T = T;
     if (!gpt && L > 0) { e.out_fp8 = f8 ? ws.x8 : nullptr; e.fp8_scale = f8 ? act_scale(0, 0) : 1.f; e.amax = am(0, 0); }
     prof_begin(3, st);
     hipError_t he = launch_embed(e, st);
     prof_end(st);
     HIPCHK(he);
+    if (t > 0) {
+      TokenEmbedArgs te;
+      std::memset(&te, 0, sizeof(te));
+      te.idx = idx; te.wte = wte_f32; te.pe = pe_f32; te.out = ws.x; te.B = mb; te.t = t; te.T = T; te.C = C; te.V = VOCAB_RL; te.out_dtype = xdt;
+      prof_begin(3, st);
+      he = launch_token_embed(te, st);
+      prof_end(st);
+      HIPCHK(he);
+    }
   }
   if (cfg.arch == CRL_ARCH_BT4CLASS) {
     HIPCHK(launch_extract_stm(planes, flags, ws.stm, mb, st));
@@ -514,7 +543,7 @@ int Model::forward_chunk(const float* planes, const uint8_t* ids, const uint8_t*
       a.bias = bias_tile; a.pos = ly.pos; a.u_bias = ly.u_bias; a.v_bias = ly.v_bias;
       a.out = f8 ? (void*)ws.ao8 : (void*)ws.ao; a.ldo = C; a.out_dtype = f8 ? DT_FP8 : ad;
       a.out_scale = f8 ? act_scale(l, 1) : 1.f; a.amax = am(l, 1);
-      a.B = mb; a.H = H; a.scale = attn_scale; a.in_dtype = ad;
+      a.B = mb; a.H = H; a.scale = attn_scale; a.in_dtype = ad; a.T = T;
       a.mode = gpt ? ATTN_CAUSAL : cfg.arch == CRL_ARCH_BT4 ? ATTN_RELSHIFT : ATTN_BIAS;
       prof_begin(1, st);
       hipError_t he = launch_attention(a, hs, st);
@@ -558,11 +587,19 @@ int Model::forward_chunk(const float* planes, const uint8_t* ids, const uint8_t*
 
   // ---- heads
   if (gpt) {
-    // ln_f and lm_head on token 63 only (model_bis.py:369-370).
-    const char* last_tok = reinterpret_cast<const char*>(ws.x) + (size_t)63 * C * dtype_size(xdt);
-    RUN(lnorm(last_tok, 64L * C, xdt, lnf_g, lnf_b, ws.hl, hd, nullptr, 1.f, C, mb, C, nullptr, st));
-    GOpt o;
-    RUN(gemm(lm_head, ws.hl, C, hd, policy, VOCAB_RL, DT_F32, mb, o, st));
+    if (all_logits) {
+      // ln_f and lm_head on every token (model_bis.py:189-192, compute_loss=True).
+      RUN(lnorm(ws.x, C, xdt, lnf_g, lnf_b, ws.h, hd, nullptr, 1.f, C, M, C, nullptr, st));
+      GOpt o;
+      RUN(gemm(lm_head, ws.h, C, hd, all_logits, VOCAB_RL, DT_F32, M, o, st));
+    }
+    if (policy) {
+      // ln_f and lm_head on the last token only (model_bis.py:195-196, 369-370).
+      const char* last_tok = reinterpret_cast<const char*>(ws.x) + (size_t)(T - 1) * C * dtype_size(xdt);
+      RUN(lnorm(last_tok, (long)T * C, xdt, lnf_g, lnf_b, ws.hl, hd, nullptr, 1.f, C, mb, C, nullptr, st));
+      GOpt o;
+      RUN(gemm(lm_head, ws.hl, C, hd, policy, VOCAB_RL, DT_F32, mb, o, st));
+    }
     return CRL_OK;
   }
   const int hact = cfg.arch == CRL_ARCH_BT4 ? ACT_GELU : ACT_MISH;

@@ -51,7 +51,8 @@ struct Model {
   std::vector<void*> allocs, ws_allocs;
   std::vector<Layer> layers;
   float *emb_w1t = nullptr, *emb_b1 = nullptr, *emb_g = nullptr, *emb_b = nullptr, *gate_a_exp = nullptr, *gate_b = nullptr;
-  float *pe_f32 = nullptr, *lnf_g = nullptr, *lnf_b = nullptr, *promo_w = nullptr;
+  float *pe_f32 = nullptr, *wte_f32 = nullptr, *lnf_g = nullptr, *lnf_b = nullptr, *promo_w = nullptr;
+  int pe_rows = 0;
   void* pe_head = nullptr;
   Lin lm_head, pol_tok, pol_qk, pol_head, val1, val2, val3, sm_weight_gen;
   int16_t* gidx = nullptr;
@@ -74,6 +75,10 @@ struct Model {
   int set_weight(const char* key, const float* data, long numel);
   int finalize();
   int forward(const float* planes, const uint8_t* ids, const uint8_t* flags, int B, float* policy, float* wdl, bool calibrate, hipStream_t st);
+  // CRL_ARCH_GPT64 with t move tokens after the 64 board tokens; policy = logits of the last token [B,V],
+  // all_logits = logits of every token [B, 64+t, V]; either may be null.
+  int forward_tokens(const float* planes, const uint8_t* ids, const uint8_t* flags, const int64_t* idx, int t, int B, float* policy,
+                     float* all_logits, float* wdl, bool calibrate, hipStream_t st);
   int calibrate(const float* planes, int B, hipStream_t st);
   double flops_per_position() const;
 
@@ -83,7 +88,8 @@ struct Model {
   int upload(const std::vector<float>& v, int dt, float scale, void** out);
   int make_lin(Lin& L, const std::vector<float>& W, const std::vector<float>* bias, int N, int K, int dt16, bool fp8);
   int ensure_ws(int mb);
-  int forward_chunk(const float* planes, const uint8_t* ids, const uint8_t* flags, int mb, float* policy, float* wdl, bool calibrate, hipStream_t st);
+  int forward_chunk(const float* planes, const uint8_t* ids, const uint8_t* flags, const int64_t* idx, int t, int mb, float* policy,
+                    float* all_logits, float* wdl, bool calibrate, hipStream_t st);
   int gemm(const Lin& L, const void* A, long lda, int in_dt, void* C, long ldc, int out_dt, int M, const GOpt& o, hipStream_t st);
   int lnorm(const void* x, long ldx, int in_dt, const float* g, const float* b, void* out, int out_dt, uint8_t* out8, float scale8,
             long ldo, int rows, int C, float* amax, hipStream_t st);

@@ -131,6 +131,30 @@ def _default_init(shapes, seed, n_layer=None):
     return sd
 
 
+def token_scores(logits, target=None, ref_logits=None, ignore_index=-100, want_kl=False):
+    """Row-wise log-softmax statistics of cuda float32 logits [rows, V] through the library's kernel:
+    returns (logp [rows] of `target` or None, ref_logp or None, kl(softmax(logits) || softmax(ref_logits)) or None)."""
+    rows, V = logits.shape
+    assert logits.stride(1) == 1 and (ref_logits is None or ref_logits.stride(1) == 1)
+    dev = logits.device
+    logp = torch.empty(rows, dtype=torch.float32, device=dev) if target is not None else None
+    rlogp = torch.empty(rows, dtype=torch.float32, device=dev) if (target is not None and ref_logits is not None) else None
+    kl = torch.empty(rows, dtype=torch.float32, device=dev) if (want_kl and ref_logits is not None) else None
+    tgt = target.to(torch.int64).contiguous() if target is not None else None
+    check(lib().crl_token_scores(_ptr(logits), logits.stride(0), _ptr(ref_logits), ref_logits.stride(0) if ref_logits is not None else 0,
+                                 _ptr(tgt), rows, V, int(ignore_index), _ptr(logp), _ptr(rlogp), _ptr(kl), _stream_ptr()), "crl_token_scores")
+    return logp, rlogp, kl
+
+
+def cross_entropy(logits, targets, ignore_index=-100):
+    """F.cross_entropy(logits, targets, ignore_index=...) (mean over the rows that count) on the device."""
+    tgt = targets.to(torch.int64).contiguous()
+    logp, _, _ = token_scores(logits, tgt, ignore_index=ignore_index)
+    out = torch.empty(1, dtype=torch.float32, device=logits.device)
+    check(lib().crl_masked_nll_mean(_ptr(logp), _ptr(tgt), int(ignore_index), logits.shape[0], _ptr(out), _stream_ptr()), "crl_masked_nll_mean")
+    return out[0]
+
+
 class _Engine:
     """Owns one crl_model handle."""
 
@@ -222,6 +246,19 @@ class _Engine:
         check(lib().crl_model_forward_compact(self.handle, _ptr(ids.contiguous()), _ptr(flags.contiguous()), B, _ptr(pol), _ptr(wdl), _stream_ptr()),
               "crl_model_forward_compact")
         return pol, wdl
+
+    def forward_tokens(self, planes, idx, last=True, every=False):
+        """CRL_ARCH_GPT64 with move tokens idx [B,t] (cuda int64): (logits of the last token [B,V] or None,
+        logits of every token [B,64+t,V] or None)."""
+        if not self.ready:
+            self.finalize()
+        planes = _as_planes(planes)
+        B, t = planes.shape[0], idx.shape[1]
+        lastl = torch.empty((B, self.vocab), dtype=torch.float32, device=planes.device) if last else None
+        alll = torch.empty((B, 64 + t, self.vocab), dtype=torch.float32, device=planes.device) if every else None
+        check(lib().crl_model_forward_tokens(self.handle, _ptr(planes), _ptr(idx) if t else None, B, t, _ptr(lastl), _ptr(alll), _stream_ptr()),
+              "crl_model_forward_tokens")
+        return lastl, alll
 
     def evaluate_fens(self, fens, T=1.0, chunk=4096, want_probs=True, want_wdl=True, threads=0):
         """FEN strings -> (probs [n,V] or None, wdl logits [n,3] or None, best move index [n]) as CPU tensors.
@@ -429,14 +466,24 @@ class GPT(_ModelBase):
 
     @torch.no_grad()
     def forward(self, batch, compute_loss=False):
-        """batch = (planes [B,8,8,19], idx [B,t]); only t == 0 (the 64-token forward) runs here.
-        Returns (logits [B,1,1929], None, targets) like model_bis.py:196-199."""
+        """batch = (planes [B,8,8,19], idx [B,t] int64 move tokens, t >= 0). Like model_bis.py:171-199 returns
+        (logits, loss, targets): logits [B,1,1929] of the last token and loss None, or with compute_loss the logits
+        of every token [B,64+t,1929] and the cross-entropy against the shifted targets (ignore_index 1928)."""
         planes, idx = batch[0], batch[1]
-        if compute_loss or (idx is not None and idx.numel() > 0):
-            raise NotImplementedError("only the 64-token forward (no move tokens, no loss) is implemented")
-        pol, _ = self._engine.forward(planes)
-        targets = torch.full((pol.shape[0], 64), 1928, device=pol.device, dtype=torch.int64)
-        return pol.unsqueeze(1), None, targets
+        B = _as_planes(planes).shape[0]
+        dev = planes.device
+        if idx is None:
+            idx = torch.zeros((B, 0), dtype=torch.int64, device=dev)
+        idx = idx.to(device=dev, dtype=torch.int64).contiguous()
+        t = idx.shape[1]
+        if 64 + t > self.config.block_size:
+            raise ValueError("Cannot forward sequence of length %d, block size is %d" % (64 + t, self.config.block_size))
+        targets = torch.cat((torch.full((B, 64), 1928, device=dev, dtype=torch.int64), idx), dim=1).roll(-1, dims=1)
+        if not compute_loss:
+            return self._engine.forward_tokens(planes, idx, last=True)[0].unsqueeze(1), None, targets
+        logits = self._engine.forward_tokens(planes, idx, last=False, every=True)[1]
+        loss = cross_entropy(logits.view(-1, logits.shape[-1]), targets.reshape(-1), ignore_index=1928)
+        return logits, loss, targets
 
     __call__ = forward
 

@@ -170,6 +170,13 @@ int crl_model_forward(crl_model* m, const float* planes, int B, float* policy_lo
 /* Same from the compact board form (device uint8[B,64] ids + uint8[B,4] flags). */
 int crl_model_forward_compact(crl_model* m, const uint8_t* ids, const uint8_t* flags, int B,
                               float* policy_logits, float* wdl_logits, void* stream);
+/* CRL_ARCH_GPT64 with move tokens: GPT.forward((planes, idx), compute_loss) of model_bis.py:171-199. idx [B,t] int64 are
+ * the t move tokens that follow the 64 board tokens (embedded with the tied lm_head weight plus rows 64.. of `pe`,
+ * 64+t <= rows of `pe` given to crl_model_set_weight). last_logits [B,1929] receives the logits of the last token
+ * (compute_loss=False, :195-196), all_logits [B,64+t,1929] those of every token (compute_loss=True, :191); either
+ * may be NULL. Attention is causal over all 64+t tokens. */
+int crl_model_forward_tokens(crl_model* m, const float* planes, const int64_t* idx, int B, int t, float* last_logits,
+                             float* all_logits, void* stream);
 /* Host front-end of leaf evaluation: n FEN strings in host memory -> results in host memory. Replaces the per-FEN
  * Python of model_bis.py:358-398 and new_paradigm/value.py:214-243,275-317 (encode_fens, the legal-move loop with
  * policy_index.index per move, mask, softmax/arg-max) for whole batches. The positions are walked in chunks of
@@ -190,6 +197,23 @@ double crl_model_flops_per_position(const crl_model* m);
  * 2 LayerNorm, 3 embedding, 4 policy QK^T, 5 16-bit GEMM. flops6 may be NULL. */
 int crl_model_set_profiling(crl_model* m, int on);
 int crl_model_get_profile(crl_model* m, double* ms6, int64_t* launches6, double* flops6);
+
+/* Causal attention over T tokens per position (any T in 1..4096): F.scaled_dot_product_attention(q,k,v,is_causal=True)
+ * of model_bis.py:71 for the 64+t token sequences of model_bis.py:171-199. Layout and types as crl_attention; rows of
+ * position b are b*T .. b*T+T-1. */
+int crl_attention_causal(const void* q, int64_t ldq, const void* k, int64_t ldk, const void* v, int64_t ldv, int in_dtype, void* out,
+                         int64_t ldo, int out_dtype, float out_scale, int B, int H, int head_dim, int T, float scale, float* amax, void* stream);
+/* Per-row log-softmax statistics of logits [rows, V] (V <= 2048), each output optional:
+ *   logp[r]     = log_softmax(logits[r])[target[r]]      (0 where target[r] == ignore_index or outside 0..V-1)
+ *   ref_logp[r] = log_softmax(ref_logits[r])[target[r]]
+ *   kl[r]       = sum_v softmax(logits[r])[v] * (log_softmax(logits[r])[v] - log_softmax(ref_logits[r])[v])
+ * i.e. the terms of F.cross_entropy in model_bis.py:192-193 and of the GRPO scoring of grpo_refactored.py:337-342
+ * (new_log_probs, ref_log_probs, per_token_kl and their gather at the sampled tokens). */
+int crl_token_scores(const float* logits, int64_t ldl, const float* ref_logits, int64_t ldr, const int64_t* target, int rows, int V,
+                     int64_t ignore_index, float* logp, float* ref_logp, float* kl, void* stream);
+/* out[0] = mean of -logp[r] over rows with target[r] != ignore_index (F.cross_entropy(..., ignore_index), model_bis.py:193);
+ * summed in a fixed order; 0 when no row counts. */
+int crl_masked_nll_mean(const float* logp, const int64_t* target, int64_t ignore_index, int rows, float* out, void* stream);
 
 /* Measurement probe with no counterpart in the reference: every CU runs 8 waves that issue
  * 32x32 MFMAs back to back from registers (dtype CRL_BF16, CRL_F16 or CRL_FP8; iters rounds of 8

@@ -162,10 +162,7 @@ class GPTOracle(nn.Module):
         self.register_buffer("pe", sinusoid_gpt(block_size, n_embd))
         self.transformer.wte.weight = self.lm_head.weight
 
-    @torch.no_grad()
-    def forward_last(self, planes, plan=None):
-        """planes [B,8,8,19] -> logits [B,1929] of token 63 (model_bis.py:360-370)."""
-        x = self.FenEncoder(planes) + self.pe[:64]
+    def _trunk(self, x, plan=None):
         B, T, C = x.shape
         H = self.n_head
         for li, blk in enumerate(self.transformer.h):
@@ -178,8 +175,27 @@ class GPTOracle(nn.Module):
             h = blk.ln_2(x)
             f = F.gelu(_lin(plan, h, li, 2, blk.mlp.c_fc))
             x = x + _lin(plan, f, li, 3, blk.mlp.c_proj)
-        x = self.transformer.ln_f(x)
+        return self.transformer.ln_f(x)
+
+    @torch.no_grad()
+    def forward_last(self, planes, plan=None):
+        """planes [B,8,8,19] -> logits [B,1929] of token 63 (model_bis.py:360-370)."""
+        x = self._trunk(self.FenEncoder(planes) + self.pe[:64], plan)
         return self.lm_head(x[:, -1, :])
+
+    @torch.no_grad()
+    def forward_tokens(self, planes, idx, compute_loss=False):
+        """(planes [B,8,8,19], idx [B,t]) -> (logits, loss, targets) of model_bis.py:171-199."""
+        position = self.FenEncoder(planes)
+        B, t = idx.shape
+        targets = torch.cat((torch.full((B, 64), 1928, dtype=torch.int64), idx), dim=1).roll(-1, dims=1)
+        x = torch.cat((position, self.transformer.wte(idx)), dim=1) + self.pe[:64 + t]
+        x = self._trunk(x)
+        if compute_loss:
+            logits = self.lm_head(x)
+            loss = F.cross_entropy(logits.view(-1, logits.size(-1)), targets.view(-1), ignore_index=1928)
+            return logits, loss, targets
+        return self.lm_head(x[:, [-1], :]), None, targets
 
 
 # ------------------------------------------------------------------ Model B

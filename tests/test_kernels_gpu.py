@@ -262,3 +262,65 @@ def test_mfma_probe(cuda):
             res[(dt, rnd)] = tf.value
     assert res[(_lib.FP8, 1)] <= res[(_lib.FP8, 0)] * 1.02
     assert lib().crl_probe_mfma(_lib.F32, 0, 10, None, None, st) != 0
+
+
+@pytest.mark.parametrize("T", [1, 17, 63, 64, 65, 130, 256])
+@pytest.mark.parametrize("H,hs", [(8, 32), (4, 64)])
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+def test_attention_causal_long(cuda, T, H, hs, dtype):
+    """Causal attention over T tokens per position against F.scaled_dot_product_attention(is_causal=True)."""
+    B, Cm = 3, H * hs
+    torch.manual_seed(T + H)
+    qkv = torch.randn(B * T, 3 * Cm, device=cuda).to(dtype)
+    out = torch.zeros(B * T, Cm, dtype=dtype, device=cuda)
+    base = qkv.data_ptr()
+    dt = _lib.F16 if dtype == torch.float16 else _lib.BF16
+    st = C.c_void_p(torch.cuda.current_stream().cuda_stream)
+    check(lib().crl_attention_causal(C.c_void_p(base), 3 * Cm, C.c_void_p(base + 2 * Cm), 3 * Cm, C.c_void_p(base + 4 * Cm), 3 * Cm, dt,
+                                     p(out), Cm, dt, 1.0, B, H, hs, T, 1.0 / math.sqrt(hs), None, st))
+    q, k, v = (t.float().view(B, T, H, hs).transpose(1, 2) for t in qkv.split(Cm, dim=1))
+    ref = F.scaled_dot_product_attention(q, k, v, is_causal=True).transpose(1, 2).reshape(B * T, Cm)
+    tol = 2 ** -6 if dtype == torch.bfloat16 else 2 ** -9
+    assert torch.allclose(out.float(), ref, rtol=tol, atol=tol), (out.float() - ref).abs().max()
+
+
+def test_attention_causal_long_equals_single_tile_at_64(cuda):
+    """T=64 through the streaming kernel's entry point is the single-tile kernel: same bits."""
+    B, H, hs = 4, 8, 32
+    qkv, Cm = make_qkv(B, H, hs, cuda, 5)
+    a = run_attn(qkv, B, H, hs, _lib.ATTN_CAUSAL, 1.0 / math.sqrt(hs))
+    out = torch.zeros_like(a)
+    base = qkv.data_ptr()
+    st = C.c_void_p(torch.cuda.current_stream().cuda_stream)
+    check(lib().crl_attention_causal(C.c_void_p(base), 3 * Cm, C.c_void_p(base + 2 * Cm), 3 * Cm, C.c_void_p(base + 4 * Cm), 3 * Cm, _lib.BF16,
+                                     p(out), Cm, _lib.BF16, 1.0, B, H, hs, 64, 1.0 / math.sqrt(hs), None, st))
+    assert torch.equal(a, out)
+
+
+@pytest.mark.parametrize("V", [1929, 1858, 7, 2048])
+def test_token_scores_and_cross_entropy(cuda, V):
+    """log-softmax gather, per-row KL and the ignore_index mean against torch (grpo_refactored.py:337-342, model_bis.py:193)."""
+    from chessrl_amd import models
+    torch.manual_seed(V)
+    rows = 333
+    x = torch.randn(rows, V, device=cuda) * 3
+    y = torch.randn(rows, V, device=cuda) * 3
+    tgt = torch.randint(0, V, (rows,), device=cuda)
+    ign = V - 1
+    tgt[::7] = ign
+    logp, rlogp, kl = models.token_scores(x, tgt, y, ignore_index=ign, want_kl=True)
+    lx, ly = F.log_softmax(x, -1), F.log_softmax(y, -1)
+    keep = tgt != ign
+    want = lx.gather(1, tgt[:, None])[:, 0]
+    assert torch.allclose(logp[keep], want[keep], atol=2e-5) and bool((logp[~keep] == 0).all())
+    assert torch.allclose(rlogp[keep], ly.gather(1, tgt[:, None])[:, 0][keep], atol=2e-5)
+    assert torch.allclose(kl, (lx.exp() * (lx - ly)).sum(-1), atol=1e-4, rtol=1e-4)
+    loss = models.cross_entropy(x, tgt, ignore_index=ign)
+    assert abs(loss.item() - F.cross_entropy(x, tgt, ignore_index=ign).item()) < 1e-5
+    # a strided view (the GRPO slice new_logits[:, 63:-1]) and an all-ignored batch
+    big = torch.randn(10, 20, V, device=cuda)
+    sl = big[:, 3:-1].reshape(-1, V) if False else big[:, 3:-1]
+    lp2, _, _ = models.token_scores(sl.reshape(-1, V), torch.zeros(160, dtype=torch.int64, device=cuda))
+    assert torch.allclose(lp2, F.log_softmax(sl.reshape(-1, V), -1)[:, 0], atol=2e-5)
+    assert models.cross_entropy(x, torch.full((rows,), ign, device=cuda), ignore_index=ign).item() == 0.0
+    assert lib().crl_token_scores(p(x), V, None, 0, None, rows, 4096, 0, None, None, None, None) != 0

@@ -250,3 +250,33 @@ def test_evaluate_fens_pipeline_equals_direct(cuda, arch):
     probs, _, _ = m.evaluate_fens(fens[:7], chunk=4)
     assert torch.equal(probs, ref_probs.cpu()[:7])
     assert m.evaluate_fens([], chunk=4)[2].numel() == 0
+
+
+@pytest.mark.parametrize("t", [1, 37, 192])
+def test_gpt_forward_with_move_tokens(cuda, t):
+    """GPT.forward((planes, idx), compute_loss) of model_bis.py:171-199: 64 board tokens followed by t move tokens,
+    causal attention over all of them; last-token logits, per-token logits and the cross-entropy."""
+    B = 6
+    oracle = om.test_init_(om.GPTOracle(3, 8, 256), seed=5)
+    planes, _ = positions(B, seed=9)
+    gen = torch.Generator().manual_seed(t)
+    idx = torch.randint(0, 1929, (B, t), generator=gen)
+    idx[0, -1] = 1928            # an ignored target inside the sequence
+    rl, _, rt = oracle.forward_tokens(planes, idx, compute_loss=False)
+    ra, rloss, _ = oracle.forward_tokens(planes, idx, compute_loss=True)
+    m = models.GPT(models.GPTConfig(block_size=256, vocab_size=1929, n_layer=3, n_head=8, n_embd=256))
+    m.load_state_dict(oracle.state_dict())
+    logits, loss, targets = m.forward((planes.to(cuda), idx.to(cuda)))
+    assert logits.shape == (B, 1, 1929) and loss is None and torch.equal(targets.cpu(), rt)
+    assert rel_rms(logits.cpu(), rl) < 1e-2
+    alll, loss, _ = m.forward((planes.to(cuda), idx.to(cuda)), compute_loss=True)
+    assert alll.shape == (B, 64 + t, 1929)
+    print("gpt T=%d: last rel-rms %.2e, all rel-rms %.2e, loss %.5f vs %.5f" % (64 + t, rel_rms(logits.cpu(), rl), rel_rms(alll.cpu(), ra), loss.item(), rloss.item()))
+    assert rel_rms(alll.cpu(), ra) < 1e-2
+    assert abs(loss.item() - rloss.item()) < 2e-3
+    # the last row of the per-token logits is the last-token call; the first 64 rows do not depend on the move tokens
+    assert torch.equal(alll[:, -1], logits[:, 0])
+    base, _, _ = m.forward((planes.to(cuda), idx[:, :0].to(cuda)), compute_loss=True)
+    assert torch.allclose(alll[:, :64], base, atol=1e-6, rtol=0)
+    with pytest.raises(ValueError):
+        m.forward((planes.to(cuda), torch.zeros(B, 193, dtype=torch.int64, device=cuda)))
