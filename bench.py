@@ -31,7 +31,8 @@ def parse():
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--workload", default="bt4class_fp8_b4096",
-                    choices=["bt4class_fp8_b4096", "bt4class_bf16_b1024", "bt4class_fp8_b16384", "bt4class_bf16_b8192"])
+                    choices=["bt4class_fp8_b4096", "bt4class_bf16_b1024", "bt4class_fp8_b16384", "bt4class_bf16_b8192",
+                             "grpo_scoring_gpt6x768_g8_b16_t256"])
     ap.add_argument("--micro-batch", type=int, default=0)
     ap.add_argument("--layers", type=int, default=15, help=argparse.SUPPRESS)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
@@ -41,6 +42,39 @@ def parse():
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run three 1 GiB device copies, a kernel of known traffic to scale profiler byte counters with")
     return ap.parse_args()
+
+
+def grpo_scoring(a, torch, models, board, dev):
+    """The scoring half of a GRPO step (grpo_refactored.py:395-404 and 337-342) at the reference's own sizes: policy and
+    frozen reference model (GPTConfig defaults 6x768, 12 heads, block 256) each run G*B = 8*16 sequences of 64 board + 192
+    move tokens to per-token logits; then log-softmax, per-token KL and the log-probabilities of the sampled tokens."""
+    G, Bp, t = 8, 16, 192
+    n = G * Bp
+    cfg = models.GPTConfig(block_size=256, vocab_size=1929, n_layer=6, n_head=12, n_embd=768)
+    policy, ref = models.GPT(cfg, seed=0), models.GPT(cfg, seed=1)
+    planes = torch.from_numpy(board.random_positions(1, Bp)["planes"]).to(dev).reshape(Bp, 64, 19).repeat(G, 1, 1)
+    seq = torch.randint(0, 1924, (n, t), generator=torch.Generator().manual_seed(0)).to(dev)
+
+    def step():
+        new_logits = policy._engine.forward_tokens(planes, seq, last=False, every=True)[1]
+        ref_logits = ref._engine.forward_tokens(planes, seq, last=False, every=True)[1]
+        a_, b_ = new_logits[:, 63:-1].reshape(-1, 1929), ref_logits[:, 63:-1].reshape(-1, 1929)
+        return models.token_scores(a_, seq.reshape(-1), b_, want_kl=True)
+
+    for _ in range(a.warmup):
+        step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(a.steps):
+        step()
+    torch.cuda.synchronize()
+    dt = (time.perf_counter() - t0) / a.steps
+    print(json.dumps({"metric": "scored sequences/sec, GRPO scoring (policy + reference forward over 256 tokens, KL and log-probs)",
+                      "value": round(n / dt, 1), "unit": "sequences/s", "n_gpus": 1, "steps": a.steps, "warmup": a.warmup,
+                      "ms_per_step": round(dt * 1e3, 3), "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "bf16",
+                      "data": "synthetic", "config": {"workload": a.workload, "layers": 6, "d_model": 768, "heads": 12, "G": G, "batch": Bp,
+                                                      "tokens_per_sequence": 256, "tokens_per_s": round(2 * n * 256 / dt, 1)},
+                      "roofline": None, "cpu_baseline": None}))
 
 
 def main():
@@ -57,6 +91,8 @@ def main():
         print("bench.py needs an MI355X (no CPU fallback for the measured path)", file=sys.stderr)
         sys.exit(2)
     dev = torch.device("cuda:0")
+    if a.workload.startswith("grpo_scoring"):
+        return grpo_scoring(a, torch, models, board, dev)
     fp8 = "fp8" in a.workload
     B = int(a.workload.rsplit("_b", 1)[1])
     late = 0.3 if B >= 8192 else 0.0
