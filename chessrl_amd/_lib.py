@@ -75,6 +75,8 @@ SIGNATURES = {
     "crl_attention_causal": (_i, [_vp, _i64, _vp, _i64, _vp, _i64, _i, _vp, _i64, _i, _f, _i, _i, _i, _i, _f, _vp, _vp]),
     "crl_token_scores": (_i, [_vp, _i64, _vp, _i64, _vp, _i, _i, _i64, _vp, _vp, _vp, _vp]),
     "crl_masked_nll_mean": (_i, [_vp, _vp, _i64, _i, _vp, _vp]),
+    "crl_model_generate": (_i, [_vp, _vp, _i, _i, _f, C.c_uint64, _i, _vp, _vp, _i, _vp]),
+    "crl_sample": (_i, [_vp, _i64, _i, _i, _f, C.c_uint64, _i, _vp, _vp, _vp]),
     "crl_probe_mfma": (_i, [_i, _i, _i, _vp, _vp, _vp]),
 }
 

@@ -20,6 +20,7 @@ SOURCES = [
     "kernels/attention.hip",
     "kernels/heads.hip",
     "kernels/probe.hip",
+    "kernels/decode.hip",
     "model.hip",
     "api.hip",
 ]

@@ -290,6 +290,16 @@ int crl_attention_causal(const void* q, int64_t ldq, const void* k, int64_t ldk,
   if (e == hipErrorInvalidValue) return arg_fail("crl_attention_causal: head_dim must be 32 or 64, in_dtype bf16/f16, out_dtype in_dtype or fp8, strides multiples of 8, T <= 4096");
   return e == hipSuccess ? CRL_OK : hip_fail("crl_attention_causal", e);
 }
+int crl_sample(const float* logits, int64_t ldl, int B, int V, float temperature, uint64_t seed, int step, int64_t* tokens, float* probs,
+               void* stream) {
+  if (!logits || !tokens || B < 0 || V <= 0 || V > 2048 || temperature < 0.f) return arg_fail("crl_sample: bad arguments (V <= 2048)");
+  SampleArgs a;
+  std::memset(&a, 0, sizeof(a));
+  a.logits = logits; a.ldl = ldl; a.seq = tokens; a.ld_seq = 1; a.tok_out = tokens; a.step_out = probs; a.ld_out = V;
+  a.B = B; a.V = V; a.k = 0; a.step = step; a.temperature = temperature; a.seed = seed;
+  hipError_t e = launch_sample(a, (hipStream_t)stream);
+  return e == hipSuccess ? CRL_OK : hip_fail("crl_sample", e);
+}
 int crl_token_scores(const float* logits, int64_t ldl, const float* ref_logits, int64_t ldr, const int64_t* target, int rows, int V,
                      int64_t ignore_index, float* logp, float* ref_logp, float* kl, void* stream) {
   if (!logits || rows < 0 || V <= 0) return arg_fail("crl_token_scores: bad arguments");
@@ -434,6 +444,11 @@ int crl_model_forward_tokens(crl_model* m, const float* planes, const int64_t* i
                              float* all_logits, void* stream) {
   if (!m || !planes) return arg_fail("crl_model_forward_tokens: bad arguments");
   return m->impl.forward_tokens(planes, nullptr, nullptr, idx, t, B, last_logits, all_logits, nullptr, false, (hipStream_t)stream);
+}
+int crl_model_generate(crl_model* m, const float* planes, int B, int steps, float temperature, uint64_t seed, int rules,
+                       int64_t* sequences, float* step_out, int out_logits, void* stream) {
+  if (!m) return arg_fail("crl_model_generate: null model");
+  return m->impl.generate(planes, B, steps, temperature, seed, rules, sequences, step_out, out_logits, (hipStream_t)stream);
 }
 int crl_model_evaluate_fens(crl_model* m, const char* const* fens, int n, int chunk, float temperature, float* probs,
                             float* wdl, int32_t* best, int threads) {

@@ -3,6 +3,7 @@
 #pragma once
 #include <hip/hip_runtime.h>
 #include <stdint.h>
+#include <algorithm>
 
 namespace crl {
 
@@ -206,6 +207,19 @@ struct TokenScoreArgs {
   long ignore_index;
 };
 
+// One sampling step of sequence generation.
+struct SampleArgs {
+  const float* logits; long ldl;     // [B, V]
+  int64_t* seq; long ld_seq;         // [B, >= k+1]: token k is written, token k-2 is read by the rules
+  int64_t* tok_out;                  // [B]: the same token, dense, for the next embedding
+  int32_t* num_zeros;                // [B] end_variation counters (rules only)
+  float* step_out; long ld_out;      // optional [B, V]: probabilities, or the raw logits when out_logits
+  int B, V, k, step, rules, out_logits;
+  long end_think, end_tok, end_variation;
+  float temperature;
+  uint64_t seed;
+};
+
 struct ScatterArgs {
   const float* src; long lds;       // [B, 1858]
   float* dst; long ldd;             // [B, 1929], fully written (zeros where no source)
@@ -232,6 +246,11 @@ hipError_t launch_leela_to_rl(const ScatterArgs& a, hipStream_t st);
 hipError_t launch_extract_stm(const float* planes, const uint8_t* flags, uint8_t* white_to_move, int B, hipStream_t st);
 hipError_t launch_fill_f32(float* p, float v, long n, hipStream_t st);
 hipError_t launch_convert(const float* src, void* dst, long n, int dt, float scale, hipStream_t st);
+hipError_t launch_kv_store(const void* qkv, void* cache, int B, int T, int Tmax, int C, hipStream_t st);
+hipError_t launch_decode_embed(const int64_t* tok, const float* wte, const float* pe_row, void* out, int B, int C, int V, int out_dtype, hipStream_t st);
+hipError_t launch_decode_attention(const void* q, long ldq, const void* cache, int Tmax, int C, int n, void* out, long ldo, int B, int H,
+                                   int head_dim, int in_dtype, float scale, hipStream_t st);
+hipError_t launch_sample(const SampleArgs& a, hipStream_t st);
 // Back-to-back MFMAs from registers on every CU: sustained TFLOP/s and the clock it ran at.
 hipError_t run_mfma_probe(int dtype, int random_bits, int iters, double* tflops, double* ghz, hipStream_t st);
 // Slot of (query i, key j) inside a 4096-element attention bias tile.

@@ -96,6 +96,7 @@ Model::Model(const crl_model_config& c) : cfg(c) {
 }
 
 Model::~Model() {
+  for (void* p : gen_allocs) (void)hipFree(p);
   for (void* p : allocs) (void)hipFree(p);
   for (void* p : ws_allocs) (void)hipFree(p);
   for (auto& e : prof_events) { (void)hipEventDestroy(e.a); (void)hipEventDestroy(e.b); }
@@ -465,7 +466,7 @@ int Model::forward_chunk(const float* planes, const uint8_t* ids, const uint8_t*
   const int C = cfg.d_model, F = cfg.d_ff, H = cfg.n_head, L = cfg.n_layer, hs = C / H;
   const int T = 64 + t;          // tokens per position: the board, then t move tokens (CRL_ARCH_GPT64 only)
   const int M = mb * T;
-  const bool f8 = cfg.fp8 && !calibrate;
+  const bool f8 = cfg.fp8 && !calibrate && !force_16bit;
   const int hd = cfg.head_dtype, ad = cfg.act_dtype;
   const bool gpt = cfg.arch == CRL_ARCH_GPT64;
   const bool sf32 = gpt && cfg.stream_f32;
@@ -522,6 +523,7 @@ int Model::forward_chunk(const float* planes, const uint8_t* ids, const uint8_t*
       if (cfg.arch == CRL_ARCH_BT4CLASS) { o.C2 = ws.comp; o.ldc2 = cfg.smolgen_compress; o.nsplit = 3 * C; }
       RUN(gemm(ly.qkv, a_in, C, a_dt, ws.qkv, 3 * C, ad, M, o, st));
     }
+    if (kv_capture) HIPCHK(launch_kv_store(ws.qkv, kv_layers[l], mb, T, kv_Tmax, C, st));
     const void* bias_tile = nullptr;
     if (cfg.arch == CRL_ARCH_BT4CLASS) {
       const int sc = cfg.smolgen_compress, sh = cfg.smolgen_hidden, sg = cfg.smolgen_gen;
@@ -643,6 +645,87 @@ int Model::calibrate(const float* planes, int B, hipStream_t st) {
   (void)hipFree(pol);
   if (rc) return rc;
   HIPCHK(e);
+  return CRL_OK;
+}
+
+int Model::generate(const float* planes, int B, int steps, float temperature, uint64_t seed, int rules, int64_t* seq, float* step_out,
+                    int out_logits, hipStream_t st) {
+  if (!finalized) { set_error("generate: call crl_model_finalize first"); return CRL_ERR_STATE; }
+  if (cfg.arch != CRL_ARCH_GPT64) { set_error("generate: only CRL_ARCH_GPT64 generates sequences"); return CRL_ERR_ARG; }
+  if (!planes || !seq || B <= 0 || steps < 1 || temperature < 0.f) { set_error("generate: bad arguments"); return CRL_ERR_ARG; }
+  const int C = cfg.d_model, F = cfg.d_ff, H = cfg.n_head, L = cfg.n_layer, hs = C / H;
+  const int Tmax = 64 + steps;   // the last sampled token is never fed back
+  if (Tmax > pe_rows || Tmax > 1024) { set_error("generate: 64 + steps exceeds the positional table or 1024 tokens"); return CRL_ERR_ARG; }
+  if ((long)B * 65 > (long)cfg.micro_batch * 64) { set_error("generate: batch too large for one micro-batch"); return CRL_ERR_ARG; }
+  int rc = ensure_ws((int)(((long)B * 65 + 63) / 64));
+  if (rc) return rc;
+  if (B > kv_B || Tmax > kv_Tmax || (int)kv_layers.size() != L) {
+    for (void* p : gen_allocs) (void)hipFree(p);
+    gen_allocs.clear();
+    kv_layers.assign(L, nullptr);
+    kv_B = kv_Tmax = 0;
+    auto galloc = [&](void** p, size_t bytes) -> int {
+      hipError_t e = hipMalloc(p, bytes ? bytes : 16);
+      if (e != hipSuccess) { set_error(std::string("generate: ") + hipGetErrorString(e)); return CRL_ERR_HIP; }
+      gen_allocs.push_back(*p);
+      return CRL_OK;
+    };
+    for (int l = 0; l < L; ++l) { rc = galloc(&kv_layers[l], (size_t)B * Tmax * 2 * C * 2); if (rc) return rc; }
+    rc = galloc((void**)&gen_tok, sizeof(int64_t) * B); if (rc) return rc;
+    rc = galloc((void**)&gen_zeros, sizeof(int32_t) * B); if (rc) return rc;
+    rc = galloc((void**)&gen_logits, sizeof(float) * (size_t)B * VOCAB_RL); if (rc) return rc;
+    kv_B = B; kv_Tmax = Tmax;
+  }
+  const int hd = cfg.head_dtype, ad = cfg.act_dtype;
+  const int xdt = cfg.stream_f32 ? DT_F32 : ad;
+  const long START_THINK = 1924, END_THINK = 1925, END_VARIATION = 1926, END = 1927;
+  // <thinking> opens every sequence (model_bis.py:221-224); gen_zeros doubles as the fill source via a tiny host copy.
+  {
+    std::vector<int64_t> first(B, START_THINK);
+    std::vector<int32_t> zeros(B, 0);
+    HIPCHK(hipMemcpyAsync(gen_tok, first.data(), sizeof(int64_t) * B, hipMemcpyHostToDevice, st));
+    HIPCHK(hipMemcpyAsync(gen_zeros, zeros.data(), sizeof(int32_t) * B, hipMemcpyHostToDevice, st));
+    HIPCHK(hipMemcpy2DAsync(seq, sizeof(int64_t) * (steps + 1), gen_tok, sizeof(int64_t), sizeof(int64_t), B, hipMemcpyDeviceToDevice, st));
+    HIPCHK(hipStreamSynchronize(st));   // the host vectors go out of scope
+  }
+#define RUN(call) do { rc = (call); if (rc) { kv_capture = false; force_16bit = false; return rc; } } while (0)
+  // Prefix of 65 tokens: fills the cache and gives the logits of the first sampled token.
+  kv_capture = true; force_16bit = true;
+  RUN(forward_chunk(planes, nullptr, nullptr, gen_tok, 1, B, gen_logits, nullptr, nullptr, false, st));
+  kv_capture = false;
+  const float attn_scale = 1.0f / std::sqrt((float)hs);
+  for (int k = 1; k <= steps; ++k) {
+    SampleArgs sa;
+    std::memset(&sa, 0, sizeof(sa));
+    sa.logits = gen_logits; sa.ldl = VOCAB_RL; sa.seq = seq; sa.ld_seq = steps + 1; sa.tok_out = gen_tok; sa.num_zeros = gen_zeros;
+    sa.step_out = step_out ? step_out + (size_t)(k - 1) * VOCAB_RL : nullptr; sa.ld_out = (long)steps * VOCAB_RL;
+    sa.B = B; sa.V = VOCAB_RL; sa.k = k; sa.step = k; sa.rules = rules; sa.out_logits = out_logits;
+    sa.end_think = END_THINK; sa.end_tok = END; sa.end_variation = END_VARIATION; sa.temperature = temperature; sa.seed = seed;
+    hipError_t he = launch_sample(sa, st);
+    if (he != hipSuccess) { force_16bit = false; HIPCHK(he); }
+    if (k == steps) break;
+    const int pos = 64 + k;    // sequence position of token k
+    he = launch_decode_embed(gen_tok, wte_f32, pe_f32 + (size_t)pos * C, ws.x, B, C, VOCAB_RL, xdt, st);
+    if (he != hipSuccess) { force_16bit = false; HIPCHK(he); }
+    for (int l = 0; l < L; ++l) {
+      const Layer& ly = layers[l];
+      RUN(lnorm(ws.x, C, xdt, ly.ln1_g, ly.ln1_b, ws.h, ad, nullptr, 1.f, C, B, C, nullptr, st));
+      { // q -> ws.qkv [B,C]; k|v -> row `pos` of every sequence's cache
+        GOpt o; o.C2 = reinterpret_cast<uint16_t*>(kv_layers[l]) + (size_t)pos * 2 * C; o.ldc2 = (long)kv_Tmax * 2 * C; o.nsplit = C;
+        RUN(gemm(ly.qkv, ws.h, C, ad, ws.qkv, C, ad, B, o, st)); }
+      he = launch_decode_attention(ws.qkv, C, kv_layers[l], kv_Tmax, C, pos + 1, ws.ao, C, B, H, hs, ad, attn_scale, st);
+      if (he != hipSuccess) { force_16bit = false; HIPCHK(he); }
+      { GOpt o; o.res = ws.x; o.ldr = C; o.res_dt = xdt; RUN(gemm(ly.proj, ws.ao, C, ad, ws.x, C, xdt, B, o, st)); }
+      RUN(lnorm(ws.x, C, xdt, ly.ln2_g, ly.ln2_b, ws.h, ad, nullptr, 1.f, C, B, C, nullptr, st));
+      { GOpt o; o.act = ACT_GELU; RUN(gemm(ly.ff1, ws.h, C, ad, ws.f, F, ad, B, o, st)); }
+      { GOpt o; o.res = ws.x; o.ldr = C; o.res_dt = xdt; RUN(gemm(ly.ff2, ws.f, F, ad, ws.x, C, xdt, B, o, st)); }
+    }
+    RUN(lnorm(ws.x, C, xdt, lnf_g, lnf_b, ws.hl, hd, nullptr, 1.f, C, B, C, nullptr, st));
+    { GOpt o; RUN(gemm(lm_head, ws.hl, C, hd, gen_logits, VOCAB_RL, DT_F32, B, o, st)); }
+  }
+#undef RUN
+  force_16bit = false;
+  prof_collect(st);
   return CRL_OK;
 }
 

@@ -61,6 +61,15 @@ struct Model {
   std::vector<float> amax_host;
   Workspace ws;
   int ws_mb = 0;
+  // generation state, grown on demand: per layer [B, Tmax, 2C] 16-bit keys|values, newest tokens, counters, logits
+  std::vector<void*> kv_layers;
+  std::vector<void*> gen_allocs;
+  int kv_B = 0, kv_Tmax = 0;
+  int64_t* gen_tok = nullptr;
+  int32_t* gen_zeros = nullptr;
+  float* gen_logits = nullptr;
+  bool kv_capture = false;     // forward_chunk copies every layer's keys|values into the cache
+  bool force_16bit = false;    // forward_chunk ignores cfg.fp8
 
   struct ProfEvent { hipEvent_t a, b; int fam; };
   bool profiling = false;
@@ -80,6 +89,11 @@ struct Model {
   int forward_tokens(const float* planes, const uint8_t* ids, const uint8_t* flags, const int64_t* idx, int t, int B, float* policy,
                      float* all_logits, float* wdl, bool calibrate, hipStream_t st);
   int calibrate(const float* planes, int B, hipStream_t st);
+  // Sequence generation with cached keys/values (model_bis.py:213-263 with rules, 266-311 without): seq [B, steps+1]
+  // receives <thinking> and then `steps` sampled tokens; step_out [B, steps, V] (optional) the probabilities of
+  // every step, or its logits when out_logits. Runs in the 16-bit element type whatever cfg.fp8 says.
+  int generate(const float* planes, int B, int steps, float temperature, uint64_t seed, int rules, int64_t* seq, float* step_out,
+               int out_logits, hipStream_t st);
   double flops_per_position() const;
 
  private:

@@ -260,6 +260,19 @@ class _Engine:
               "crl_model_forward_tokens")
         return lastl, alll
 
+    def generate(self, planes, steps, T=1.0, seed=0, rules=True, want_step_out=False, out_logits=False):
+        """CRL_ARCH_GPT64 sequence generation with cached keys/values: (sequences [B, steps+1] int64,
+        per-step probabilities or logits [B, steps, V] or None)."""
+        if not self.ready:
+            self.finalize()
+        planes = _as_planes(planes)
+        B = planes.shape[0]
+        seq = torch.empty((B, steps + 1), dtype=torch.int64, device=planes.device)
+        out = torch.empty((B, steps, self.vocab), dtype=torch.float32, device=planes.device) if want_step_out else None
+        check(lib().crl_model_generate(self.handle, _ptr(planes), B, int(steps), float(T), int(seed) & (2 ** 64 - 1), 1 if rules else 0,
+                                       _ptr(seq), _ptr(out), 1 if out_logits else 0, _stream_ptr()), "crl_model_generate")
+        return seq, out
+
     def evaluate_fens(self, fens, T=1.0, chunk=4096, want_probs=True, want_wdl=True, threads=0):
         """FEN strings -> (probs [n,V] or None, wdl logits [n,3] or None, best move index [n]) as CPU tensors.
         Host encoding, upload and device work of consecutive chunks overlap inside the library."""
@@ -488,6 +501,19 @@ class GPT(_ModelBase):
     __call__ = forward
 
     @torch.no_grad()
+    def generate_sequence(self, board, T=1, seed=0):
+        """model_bis.py:213-263: (sequences [B,192], probs [B,191,1929] or None for T == 0), with the forced
+        </thinking> and end tokens. Keys and values of the prefix are cached instead of recomputed per token."""
+        seq, probs = self._engine.generate(board, self.config.block_size - 65, T, seed, rules=True, want_step_out=T != 0)
+        return seq, probs
+
+    @torch.no_grad()
+    def generate_sequence_raw(self, board, T=1, return_logits=False, seed=0):
+        """model_bis.py:266-311: as generate_sequence without the forced tokens; the per-step output is the
+        probabilities or, with return_logits, the logits."""
+        return self._engine.generate(board, self.config.block_size - 65, T, seed, rules=False, want_step_out=T != 0, out_logits=return_logits)
+
+    @torch.no_grad()
     def get_move_from_fen_no_thinking(self, fen, T=1, device="cuda", force_legal=True, return_probs=False):
         planes = board.encode_fens([fen]).to(device)
         logits, _ = self._engine.forward(planes)
@@ -518,6 +544,19 @@ class BT4(_ModelBase):
         return pol.view(b, s, VOCAB_RL)
 
     __call__ = forward
+
+    @torch.no_grad()
+    def generate_sequence(self, board, T=1, seed=0):
+        """model_bis.py:213-263: (sequences [B,192], probs [B,191,1929] or None for T == 0), with the forced
+        </thinking> and end tokens. Keys and values of the prefix are cached instead of recomputed per token."""
+        seq, probs = self._engine.generate(board, self.config.block_size - 65, T, seed, rules=True, want_step_out=T != 0)
+        return seq, probs
+
+    @torch.no_grad()
+    def generate_sequence_raw(self, board, T=1, return_logits=False, seed=0):
+        """model_bis.py:266-311: as generate_sequence without the forced tokens; the per-step output is the
+        probabilities or, with return_logits, the logits."""
+        return self._engine.generate(board, self.config.block_size - 65, T, seed, rules=False, want_step_out=T != 0, out_logits=return_logits)
 
     @torch.no_grad()
     def get_move_from_fen_no_thinking(self, fen, T=1, device="cuda", force_legal=True, return_probs=False):
@@ -582,6 +621,19 @@ class BT4Class(_ModelBase):
         return self._engine.forward(board_tokens)
 
     __call__ = forward
+
+    @torch.no_grad()
+    def generate_sequence(self, board, T=1, seed=0):
+        """model_bis.py:213-263: (sequences [B,192], probs [B,191,1929] or None for T == 0), with the forced
+        </thinking> and end tokens. Keys and values of the prefix are cached instead of recomputed per token."""
+        seq, probs = self._engine.generate(board, self.config.block_size - 65, T, seed, rules=True, want_step_out=T != 0)
+        return seq, probs
+
+    @torch.no_grad()
+    def generate_sequence_raw(self, board, T=1, return_logits=False, seed=0):
+        """model_bis.py:266-311: as generate_sequence without the forced tokens; the per-step output is the
+        probabilities or, with return_logits, the logits."""
+        return self._engine.generate(board, self.config.block_size - 65, T, seed, rules=False, want_step_out=T != 0, out_logits=return_logits)
 
     @torch.no_grad()
     def get_move_from_fen_no_thinking(self, fen, T=1, device="cuda", force_legal=True, return_probs=False):

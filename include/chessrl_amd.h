@@ -177,6 +177,17 @@ int crl_model_forward_compact(crl_model* m, const uint8_t* ids, const uint8_t* f
  * may be NULL. Attention is causal over all 64+t tokens. */
 int crl_model_forward_tokens(crl_model* m, const float* planes, const int64_t* idx, int B, int t, float* last_logits,
                              float* all_logits, void* stream);
+/* Sequence generation for CRL_ARCH_GPT64 with cached keys and values: GPT.generate_sequence (rules = 1,
+ * model_bis.py:213-263) and GPT.generate_sequence_raw (rules = 0, :266-311). sequences [B, steps+1] int64 receives
+ * <thinking> (1924) followed by `steps` tokens: arg-max for temperature 0, else one draw from softmax(logits/temperature)
+ * (inverse CDF with a counter-based generator keyed by seed, sequence and step: reproducible, not torch's stream).
+ * With rules the forced tokens of :252-259 apply: after five end_variation tokens the next is </thinking>, and the
+ * token two places after a </thinking> is end. step_out [B, steps, 1929] (optional) receives every step's
+ * probabilities, or its logits when out_logits != 0 (return_logits of :266). The 65-token prefix is run once; every
+ * later token costs one row per sequence against the cache (the reference re-runs the whole prefix per token).
+ * steps <= rows(pe) - 64 and <= 960; B*65 tokens must fit one micro-batch. Runs in the 16-bit type also for fp8 models. */
+int crl_model_generate(crl_model* m, const float* planes, int B, int steps, float temperature, uint64_t seed, int rules,
+                       int64_t* sequences, float* step_out, int out_logits, void* stream);
 /* Host front-end of leaf evaluation: n FEN strings in host memory -> results in host memory. Replaces the per-FEN
  * Python of model_bis.py:358-398 and new_paradigm/value.py:214-243,275-317 (encode_fens, the legal-move loop with
  * policy_index.index per move, mask, softmax/arg-max) for whole batches. The positions are walked in chunks of
@@ -203,6 +214,12 @@ int crl_model_get_profile(crl_model* m, double* ms6, int64_t* launches6, double*
  * position b are b*T .. b*T+T-1. */
 int crl_attention_causal(const void* q, int64_t ldq, const void* k, int64_t ldk, const void* v, int64_t ldv, int in_dtype, void* out,
                          int64_t ldo, int out_dtype, float out_scale, int B, int H, int head_dim, int T, float scale, float* amax, void* stream);
+/* One token per row of logits [B, V] (V <= 2048): arg-max (lowest index among equals) for temperature 0, else one
+ * draw from softmax(logits/temperature), i.e. torch.argmax / F.softmax + torch.multinomial of model_bis.py:242-247,
+ * 385-392. The draw is the inverse CDF at a uniform number that depends only on (seed, row, step). probs [B, V]
+ * (optional) receives the softmax. */
+int crl_sample(const float* logits, int64_t ldl, int B, int V, float temperature, uint64_t seed, int step, int64_t* tokens, float* probs,
+               void* stream);
 /* Per-row log-softmax statistics of logits [rows, V] (V <= 2048), each output optional:
  *   logp[r]     = log_softmax(logits[r])[target[r]]      (0 where target[r] == ignore_index or outside 0..V-1)
  *   ref_logp[r] = log_softmax(ref_logits[r])[target[r]]

@@ -198,6 +198,26 @@ class GPTOracle(nn.Module):
         return self.lm_head(x[:, [-1], :]), None, targets
 
 
+def apply_generation_rules(raw):
+    """The token bookkeeping of GPT.generate_sequence (model_bis.py:221-260) for already chosen tokens:
+    raw [B, steps] are the tokens the sampler picked at every step; returns sequences [B, steps+1] that open with
+    <thinking> and carry the forced </thinking> (after five end_variation) and end (two places after </thinking>)."""
+    START_THINK, END_THINK, END_VARIATION, END = 1924, 1925, 1926, 1927
+    B, steps = raw.shape
+    seq = torch.full((B, steps + 1), START_THINK, dtype=torch.int64)
+    for b in range(B):
+        nz = 0
+        for k in range(1, steps + 1):
+            tok = int(raw[b, k - 1])
+            if nz == 5:
+                tok, nz = END_THINK, 6
+            if k >= 2 and int(seq[b, k - 2]) == END_THINK:
+                tok = END
+            nz += 1 if tok == END_VARIATION else 0
+            seq[b, k] = tok
+    return seq
+
+
 # ------------------------------------------------------------------ Model B
 def rel_shift(s):
     """new_paradigm/attn.py:525-533 in closed form for a [..., T, T] score:

@@ -324,3 +324,30 @@ def test_token_scores_and_cross_entropy(cuda, V):
     assert torch.allclose(lp2, F.log_softmax(sl.reshape(-1, V), -1)[:, 0], atol=2e-5)
     assert models.cross_entropy(x, torch.full((rows,), ign, device=cuda), ignore_index=ign).item() == 0.0
     assert lib().crl_token_scores(p(x), V, None, 0, None, rows, 4096, 0, None, None, None, None) != 0
+
+
+def test_sample_distribution_and_argmax(cuda):
+    """crl_sample draws from softmax(logits/T): empirical frequencies over 200k rows, arg-max for T=0."""
+    V, B = 37, 200000
+    torch.manual_seed(0)
+    row = torch.randn(V, device=cuda) * 2
+    logits = row.expand(B, V).contiguous()
+    toks = torch.empty(B, dtype=torch.int64, device=cuda)
+    probs = torch.empty(B, V, device=cuda)
+    st = C.c_void_p(torch.cuda.current_stream().cuda_stream)
+    check(lib().crl_sample(p(logits), V, B, V, 0.7, 123, 5, p(toks), p(probs), st))
+    want = F.softmax(row / 0.7, -1)
+    assert torch.allclose(probs[17], want, atol=1e-6)
+    freq = torch.bincount(toks, minlength=V).float() / B
+    # binomial standard deviation of a frequency is at most sqrt(p/B): allow five of them
+    assert bool(((freq - want).abs() <= 5 * (want / B).sqrt() + 1e-5).all()), (freq - want).abs().max()
+    toks2 = torch.empty_like(toks)
+    check(lib().crl_sample(p(logits), V, B, V, 0.7, 123, 5, p(toks2), None, st))
+    assert torch.equal(toks, toks2)
+    check(lib().crl_sample(p(logits), V, B, V, 0.7, 123, 6, p(toks2), None, st))
+    assert not torch.equal(toks, toks2)
+    x = torch.randn(64, 1929, device=cuda)
+    x[:, 100] = x[:, 7] = 9.0      # a tie: the lower index wins
+    t0 = torch.empty(64, dtype=torch.int64, device=cuda)
+    check(lib().crl_sample(p(x), 1929, 64, 1929, 0.0, 0, 0, p(t0), None, st))
+    assert bool((t0 == 7).all())

@@ -280,3 +280,53 @@ def test_gpt_forward_with_move_tokens(cuda, t):
     assert torch.allclose(alll[:, :64], base, atol=1e-6, rtol=0)
     with pytest.raises(ValueError):
         m.forward((planes.to(cuda), torch.zeros(B, 193, dtype=torch.int64, device=cuda)))
+
+
+def test_generate_cached_equals_teacher_forced_forward(cuda):
+    """Greedy generation with cached keys/values: every step's logits equal the logits the full (uncached) forward
+    gives at that position when it is fed the generated tokens, and every token is the arg-max of its step."""
+    B, steps = 5, 70
+    oracle = om.test_init_(om.GPTOracle(3, 8, 256), seed=6)
+    planes, _ = positions(B, seed=4)
+    m = models.GPT(models.GPTConfig(block_size=256, vocab_size=1929, n_layer=3, n_head=8, n_embd=256))
+    m.load_state_dict(oracle.state_dict())
+    seq, logits = m._engine.generate(planes.to(cuda), steps, T=0.0, rules=False, want_step_out=True, out_logits=True)
+    assert seq.shape == (B, steps + 1) and bool((seq[:, 0] == 1924).all())
+    assert torch.equal(seq[:, 1:], logits.argmax(-1))
+    full = m._engine.forward_tokens(planes.to(cuda), seq[:, :steps].contiguous(), last=False, every=True)[1]
+    err = rel_rms(logits.cpu(), full[:, 64:64 + steps].cpu())
+    print("generate: cached vs recomputed logits rel-rms %.2e" % err)
+    assert err < 3e-3
+    # and against the fp32 oracle fed the same tokens
+    ra, _, _ = oracle.forward_tokens(planes, seq[:, :steps].cpu(), compute_loss=True)
+    assert rel_rms(logits.cpu(), ra[:, 64:64 + steps]) < 1e-2
+    # the reference's entry points: full length, probabilities that sum to one, reproducible draws
+    s1, p1 = m.generate_sequence(planes.to(cuda), T=1, seed=3)
+    s2, _ = m.generate_sequence(planes.to(cuda), T=1, seed=3)
+    s3, _ = m.generate_sequence(planes.to(cuda), T=1, seed=4)
+    assert s1.shape == (B, 192) and p1.shape == (B, 191, 1929) and torch.equal(s1, s2) and not torch.equal(s1, s3)
+    assert torch.allclose(p1.sum(-1), torch.ones(B, 191, device=cuda), atol=1e-4)
+    assert bool((p1.gather(2, s1[:, 1:, None]) > 0).all())
+    s0, p0 = m.generate_sequence_raw(planes.to(cuda), T=0)
+    assert p0 is None and s0.shape == (B, 192)
+
+
+def test_generate_forced_tokens(cuda):
+    """generate_sequence's bookkeeping (model_bis.py:252-259) on a model rigged to prefer end_variation: the sequences
+    equal the rule application of the oracle to the arg-max of the recorded step logits."""
+    B, steps = 3, 20
+    oracle = om.test_init_(om.GPTOracle(2, 8, 256), seed=7)
+    sd = oracle.state_dict()
+    u = sd["transformer.ln_f.bias"].clone()
+    sd["lm_head.weight"][1926] = 40.0 * u / u.pow(2).sum()
+    sd["transformer.wte.weight"] = sd["lm_head.weight"]
+    planes, _ = positions(B, seed=8)
+    m = models.GPT(models.GPTConfig(block_size=256, vocab_size=1929, n_layer=2, n_head=8, n_embd=256))
+    m.load_state_dict(sd)
+    seq, logits = m._engine.generate(planes.to(cuda), steps, T=0.0, rules=True, want_step_out=True, out_logits=True)
+    want = om.apply_generation_rules(logits.argmax(-1).cpu())
+    assert torch.equal(seq.cpu(), want)
+    row = seq[0].tolist()
+    assert row.count(1926) >= 5 and 1925 in row
+    i = row.index(1925)
+    assert row[1:i].count(1926) == 5 and row[i + 2] == 1927
