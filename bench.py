@@ -32,7 +32,7 @@ def parse():
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--workload", default="bt4class_fp8_b4096",
                     choices=["bt4class_fp8_b4096", "bt4class_bf16_b1024", "bt4class_fp8_b16384", "bt4class_bf16_b8192",
-                             "grpo_scoring_gpt6x768_g8_b16_t256"])
+                             "grpo_scoring_gpt6x768_g8_b16_t256", "grpo_rollout_gpt6x768_g8_b16_t256"])
     ap.add_argument("--micro-batch", type=int, default=0)
     ap.add_argument("--layers", type=int, default=15, help=argparse.SUPPRESS)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
@@ -77,6 +77,39 @@ def grpo_scoring(a, torch, models, board, dev):
                       "roofline": None, "cpu_baseline": None}))
 
 
+def grpo_rollout(a, torch, models, board, dev):
+    """The rollout half of a GRPO step (grpo_refactored.py:398, model_bis.py:213-263): G*B = 128 sequences of 191 sampled
+    tokens after the 64 board tokens and <thinking>, T = 1, forced-token rules on, keys and values cached."""
+    G, Bp = 8, 16
+    n = G * Bp
+    cfg = models.GPTConfig(block_size=256, vocab_size=1929, n_layer=6, n_head=12, n_embd=768)
+    policy = models.GPT(cfg, seed=0)
+    planes = torch.from_numpy(board.random_positions(1, Bp)["planes"]).to(dev).reshape(Bp, 64, 19).repeat(G, 1, 1)
+    for i in range(a.warmup):
+        policy.generate_sequence(planes, T=1, seed=i)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for i in range(a.steps):
+        policy.generate_sequence(planes, T=1, seed=100 + i)
+    torch.cuda.synchronize()
+    dt = (time.perf_counter() - t0) / a.steps
+    # what the reference's loop costs on the same kernels: one full forward per sampled token over the growing prefix
+    seq = torch.randint(0, 1924, (n, 191), generator=torch.Generator().manual_seed(0)).to(dev)
+    torch.cuda.synchronize()
+    t1 = time.perf_counter()
+    for t in range(1, 192, 10):
+        policy._engine.forward_tokens(planes, seq[:, :t].contiguous(), last=True)
+    torch.cuda.synchronize()
+    naive = (time.perf_counter() - t1) * 10
+    print(json.dumps({"metric": "generated sequences/sec, GRPO rollout (191 sampled tokens per sequence, cached keys/values)",
+                      "value": round(n / dt, 1), "unit": "sequences/s", "n_gpus": 1, "steps": a.steps, "warmup": a.warmup,
+                      "ms_per_step": round(dt * 1e3, 3), "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "bf16",
+                      "data": "synthetic", "config": {"workload": a.workload, "layers": 6, "d_model": 768, "heads": 12, "G": G, "batch": Bp,
+                                                      "sampled_tokens_per_s": round(n * 191 / dt, 1),
+                                                      "full_recompute_per_token_ms_estimate": round(naive * 1e3, 1)},
+                      "roofline": None, "cpu_baseline": None}))
+
+
 def main():
     a = parse()
     if a.gpus != 1:
@@ -93,6 +126,8 @@ def main():
     dev = torch.device("cuda:0")
     if a.workload.startswith("grpo_scoring"):
         return grpo_scoring(a, torch, models, board, dev)
+    if a.workload.startswith("grpo_rollout"):
+        return grpo_rollout(a, torch, models, board, dev)
     fp8 = "fp8" in a.workload
     B = int(a.workload.rsplit("_b", 1)[1])
     late = 0.3 if B >= 8192 else 0.0
