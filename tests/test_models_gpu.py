@@ -34,7 +34,7 @@ def report(name, pol, rpol, mask, wdl=None, rwdl=None):
 
 
 def test_gpt_plumbing_config(cuda):
-    """BASELINE config 1: 6 layers, d=256, 8 heads, FFN 1024 GELU, B=256."""
+    """The small plumbing configuration: 6 layers, d=256, 8 heads, FFN 1024 GELU, B=256."""
     oracle = om.test_init_(om.GPTOracle(6, 8, 256), seed=0)
     planes, mask = positions(256)
     ref = oracle.forward_last(planes)
