@@ -109,6 +109,7 @@ struct GemmArgs {
   float out_scale;    // multiplies the final value before an fp8 store
   int vec_ok;         // 1 if 4-wide stores/loads along N are aligned for C, C2 and res
   int res_rows;       // >0: the residual has this many rows and row m reads row m % res_rows
+  int stream_out;     // 1: the output is far larger than the L2 caches: store it with the non-temporal hint
 };
 
 struct LayerNormArgs {
