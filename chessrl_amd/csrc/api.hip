@@ -422,12 +422,12 @@ int crl_model_calibrate(crl_model* m, const float* planes, int B, void* stream) 
   return m->impl.calibrate(planes, B, (hipStream_t)stream);
 }
 int crl_model_get_amax(crl_model* m, float* out, int n) {
-  if (!m || !out || n != (int)m->impl.amax_host.size()) return arg_fail("crl_model_get_amax: n must be n_layer*4");
+  if (!m || !out || n != (int)m->impl.amax_host.size()) return arg_fail("crl_model_get_amax: n must be n_layer*5");
   std::memcpy(out, m->impl.amax_host.data(), sizeof(float) * n);
   return CRL_OK;
 }
 int crl_model_set_amax(crl_model* m, const float* in, int n) {
-  if (!m || !in || n != (int)m->impl.amax_host.size()) return arg_fail("crl_model_set_amax: n must be n_layer*4");
+  if (!m || !in || n != (int)m->impl.amax_host.size()) return arg_fail("crl_model_set_amax: n must be n_layer*5");
   std::memcpy(m->impl.amax_host.data(), in, sizeof(float) * n);
   return CRL_OK;
 }

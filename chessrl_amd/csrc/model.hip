@@ -92,7 +92,7 @@ Model::Model(const crl_model_config& c) : cfg(c) {
     }
     lin("value_head.dense1", 128, C); lin("value_head.dense2", 128, 128 * 64); lin("value_head.dense3", 3, 128);
   }
-  amax_host.assign((size_t)L * 4, 0.f);
+  amax_host.assign((size_t)L * AMAX_SLOTS, 0.f);
 }
 
 Model::~Model() {
@@ -277,7 +277,7 @@ int Model::finalize() {
       for (int i = 0; i < 64; ++i)
         for (int j = 0; j < 64; ++j)
           std::memcpy(&perm[(size_t)attn_bias_slot_host(i, j) * sg], &gw[(size_t)(i * 64 + j) * sg], sizeof(float) * sg);
-      LIN(sm_weight_gen, perm, nullptr, 4096, sg, ad, false);
+      LIN(sm_weight_gen, perm, nullptr, 4096, sg, ad, f8);
       UP(w("promotion_offsets.weight"), DT_F32, promo_w);
       // Gather tables: Leela move v -> (from_token*64+to_token) for black / white rows.
       std::vector<int16_t> gi((size_t)2 * VOCAB_LEELA);
@@ -335,6 +335,7 @@ int Model::ensure_ws(int mb) {
     WS(ws.sh2, (size_t)mb * cfg.smolgen_hidden * 2);
     WS(ws.sg1, (size_t)mb * H * cfg.smolgen_gen * 2);
     WS(ws.sg2, (size_t)mb * H * cfg.smolgen_gen * 2);
+    WS(ws.sg2_8, (size_t)mb * H * cfg.smolgen_gen);
     WS(ws.bias, (size_t)mb * H * 4096 * 2);
   }
   if (cfg.arch == CRL_ARCH_GPT64) {
@@ -426,7 +427,7 @@ int Model::lnorm(const void* x, long ldx, int in_dt, const float* g, const float
 }
 
 float Model::act_scale(int layer, int slot) const {
-  const float am = amax_host[(size_t)layer * 4 + slot];
+  const float am = amax_host[(size_t)layer * AMAX_SLOTS + slot];
   return am > 0.f ? 448.f / am : 1.f;
 }
 
@@ -471,7 +472,7 @@ int Model::forward_chunk(const float* planes, const uint8_t* ids, const uint8_t*
   const bool gpt = cfg.arch == CRL_ARCH_GPT64;
   const bool sf32 = gpt && cfg.stream_f32;
   const int xdt = sf32 ? DT_F32 : ad;
-  auto am = [&](int l, int slot) -> float* { return calibrate ? amax_dev + (size_t)l * 4 + slot : nullptr; };
+  auto am = [&](int l, int slot) -> float* { return calibrate ? amax_dev + (size_t)l * AMAX_SLOTS + slot : nullptr; };
   int rc;
 #define RUN(call) do { rc = (call); if (rc) return rc; } while (0)
 
@@ -531,9 +532,12 @@ int Model::forward_chunk(const float* planes, const uint8_t* ids, const uint8_t*
       RUN(gemm(ly.sm_hidden, ws.comp, 64 * sc, ad, ws.sh1, sh, ad, mb, o, st));
       RUN(lnorm(ws.sh1, sh, ad, ly.sm_ln1_g, ly.sm_ln1_b, ws.sh2, ad, nullptr, 1.f, sh, mb, sh, nullptr, st));
       RUN(gemm(ly.sm_gen, ws.sh2, sh, ad, ws.sg1, H * sg, ad, mb, o, st));
-      RUN(lnorm(ws.sg1, H * sg, ad, ly.sm_ln2_g, ly.sm_ln2_b, ws.sg2, ad, nullptr, 1.f, H * sg, mb, H * sg, nullptr, st));
-      GOpt o2;
-      RUN(gemm(sm_weight_gen, ws.sg2, sg, ad, ws.bias, 4096, ad, mb * H, o2, st));
+      // The shared 256 -> 4096 generator is the largest smolgen product (2*B*H*256*4096 per layer): in the fp8
+      // configuration it takes e4m3 inputs like the trunk linears; the two small layers before it stay 16-bit.
+      RUN(lnorm(ws.sg1, H * sg, ad, ly.sm_ln2_g, ly.sm_ln2_b, f8 ? nullptr : ws.sg2, ad, f8 ? ws.sg2_8 : nullptr, f8 ? act_scale(l, 4) : 1.f,
+                H * sg, mb, H * sg, am(l, 4), st));
+      GOpt o2; o2.a_scale = f8 ? act_scale(l, 4) : 1.f;
+      RUN(gemm(sm_weight_gen, f8 ? (const void*)ws.sg2_8 : (const void*)ws.sg2, sg, f8 ? DT_FP8 : ad, ws.bias, 4096, ad, mb * H, o2, st));
       bias_tile = ws.bias;
     }
     // attention

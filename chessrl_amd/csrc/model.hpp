@@ -36,6 +36,7 @@ struct Workspace {
   void *x = nullptr, *t = nullptr, *h = nullptr, *qkv = nullptr, *ao = nullptr, *f = nullptr;
   uint8_t *x8 = nullptr, *h8 = nullptr, *ao8 = nullptr, *f8 = nullptr, *stm = nullptr;
   void *comp = nullptr, *sh1 = nullptr, *sh2 = nullptr, *sg1 = nullptr, *sg2 = nullptr, *bias = nullptr;
+  uint8_t* sg2_8 = nullptr;
   void *hl = nullptr, *tok = nullptr, *pqk = nullptr, *v1 = nullptr, *v2 = nullptr, *dense = nullptr;
 };
 
@@ -57,6 +58,9 @@ struct Model {
   Lin lm_head, pol_tok, pol_qk, pol_head, val1, val2, val3, sm_weight_gen;
   int16_t* gidx = nullptr;
   int8_t* gpromo = nullptr;
+  // Activation amax table [n_layer][AMAX_SLOTS]: input of q|k|v, attention output, input of FFN-1, input of FFN-2,
+  // input of the shared bias generator (BT4-class only).
+  static constexpr int AMAX_SLOTS = 5;
   float* amax_dev = nullptr;
   std::vector<float> amax_host;
   Workspace ws;

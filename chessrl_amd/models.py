@@ -216,9 +216,9 @@ class _Engine:
         check(lib().crl_model_calibrate(self.handle, _ptr(planes), planes.shape[0], _stream_ptr()), "crl_model_calibrate")
 
     def get_amax(self):
-        a = np.zeros(self.n_layer * 4, np.float32)
+        a = np.zeros(self.n_layer * 5, np.float32)
         check(lib().crl_model_get_amax(self.handle, a.ctypes.data, a.size), "crl_model_get_amax")
-        return a.reshape(self.n_layer, 4)
+        return a.reshape(self.n_layer, 5)
 
     def set_amax(self, a):
         a = np.ascontiguousarray(np.asarray(a, np.float32).reshape(-1))

@@ -159,7 +159,8 @@ int crl_model_finalize(crl_model* m);
  * scales 448/amax (pretrain_fp8.py:75-79 uses DelayedScaling amax history; here the history
  * is one calibration batch). Synchronises the stream. */
 int crl_model_calibrate(crl_model* m, const float* planes, int B, void* stream);
-/* Read / overwrite the activation amax table (float[n_layer*4]). */
+/* Read / overwrite the activation amax table, float[n_layer*5]: per layer the input of q|k|v, the attention output,
+ * the inputs of the two FFN linears and the input of the shared attention-bias generator (BT4-class only, else 0). */
 int crl_model_get_amax(crl_model* m, float* out, int n);
 int crl_model_set_amax(crl_model* m, const float* in, int n);
 /* The forward pass. planes: device f32 [B,64,19] (GPT.forward batch[0] / BT4.forward inp[0]).

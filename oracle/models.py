@@ -47,11 +47,12 @@ def amax_scale(amax):
 
 
 class Fp8Plan:
-    """Activation amax table [n_layer, 4]: slot 0 = input of the q/k/v linear, 1 = attention
-    output, 2 = input of the first FFN linear, 3 = input of the second FFN linear."""
+    """Activation amax table [n_layer, 5]: slot 0 = input of the q/k/v linear, 1 = attention
+    output, 2 = input of the first FFN linear, 3 = input of the second FFN linear, 4 = input of the
+    shared attention-bias generator (BT4-class)."""
 
     def __init__(self, n_layer):
-        self.amax = torch.zeros(n_layer, 4)
+        self.amax = torch.zeros(n_layer, 5)
         self.recording = False
 
     def lin(self, x, layer, slot, weight, bias):
@@ -399,7 +400,7 @@ class BT4ClassOracle(nn.Module):
                 q, k, v, comp = out.split([C, C, C, sm.compress.weight.shape[0]], dim=-1)
             hid = sm.hidden_ln(F.silu(sm.hidden(comp.reshape(B, -1))))
             gen = sm.gen_from_ln(F.silu(sm.gen_from(hid))).view(B, H, -1)
-            bias = self.smol_weight_gen(gen).view(B, H, 64, 64)
+            bias = _lin(plan, gen, li, 4, self.smol_weight_gen).view(B, H, 64, 64)
             q, k, v = (t.view(B, T, H, hs).transpose(1, 2) for t in (q, k, v))
             score = torch.matmul(q, k.transpose(-2, -1)) / math.sqrt(hs) + bias
             ctx = torch.matmul(F.softmax(score, -1), v).transpose(1, 2).reshape(B, T, C)
