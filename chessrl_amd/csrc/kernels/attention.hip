@@ -86,6 +86,20 @@ __global__ void __launch_bounds__(64 * AttnWaves<MODE>::N) attention_kernel(cons
   const uint16_t* kp = reinterpret_cast<const uint16_t*>(a.k) + (long)b * 64 * a.ldk + h * HS;
   const uint16_t* vp = reinterpret_cast<const uint16_t*>(a.v) + (long)b * 64 * a.ldv + h * HS;
 
+  // The bias tile is the largest operand (8 KB per wave): request it first so it travels while V is
+  // transposed and the scores are formed.
+  uint4 braw[2][2][2];
+  if constexpr (MODE == ATTN_BIAS) {
+    const uint16_t* bp = reinterpret_cast<const uint16_t*>(a.bias) + (long)unit * 4096;
+#pragma unroll
+    for (int it = 0; it < 2; ++it)
+#pragma unroll
+      for (int jt = 0; jt < 2; ++jt)
+#pragma unroll
+        for (int rh = 0; rh < 2; ++rh)
+          braw[it][jt][rh] = *reinterpret_cast<const uint4*>(bp + ((((it * 2 + jt) * 2 + rh) * 64 + lane) << 3));
+  }
+
   // ---- V -> V^T in LDS ------------------------------------------------------------
   uint16_t* vt = s_vt[wave];
   {
@@ -203,14 +217,13 @@ __global__ void __launch_bounds__(64 * AttnWaves<MODE>::N) attention_kernel(cons
           s[jt][it] = H16::mfma(kf[jt][ks], qf[it][ks], s[jt][it]);
 
     if constexpr (MODE == ATTN_BIAS) {
-      const uint16_t* bp = reinterpret_cast<const uint16_t*>(a.bias) + (long)unit * 4096;
 #pragma unroll
       for (int it = 0; it < 2; ++it)
 #pragma unroll
         for (int jt = 0; jt < 2; ++jt)
 #pragma unroll
           for (int rh = 0; rh < 2; ++rh) {
-            const uint4 u = *reinterpret_cast<const uint4*>(bp + ((((it * 2 + jt) * 2 + rh) * 64 + lane) << 3));
+            const uint4 u = braw[it][jt][rh];
             const uint32_t w[4] = {u.x, u.y, u.z, u.w};
 #pragma unroll
             for (int e = 0; e < 8; ++e) {
