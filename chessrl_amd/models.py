@@ -514,6 +514,24 @@ class GPT(_ModelBase):
         return self._engine.generate(board, self.config.block_size - 65, T, seed, rules=False, want_step_out=T != 0, out_logits=return_logits)
 
     @torch.no_grad()
+    def get_move_from_fen(self, fen, T=1, device="cuda", force_legal=True, return_probs=False, seed=0):
+        """model_bis.py:321-356: generate a thinking sequence, take the logits of the step that produced the token
+        before the first `end` (the last step's if there is none), mask them to the legal moves and sample.
+        T must be positive (the reference divides by T and needs the per-step logits)."""
+        if not T > 0:
+            raise ValueError("get_move_from_fen needs T > 0")
+        planes = board.encode_fens([fen]).to(device)
+        seq, logits = self.generate_sequence_raw(planes, T=T, return_logits=True, seed=seed)
+        ids = seq[0].tolist()
+        end = policy_index.index("end")
+        i = ids.index(end) if end in ids else len(ids) - 1
+        row = logits[0, i - 2].unsqueeze(0)          # negative i-2 wraps like the reference's indexing
+        mask = torch.from_numpy(board.legal_move_mask(fen)).to(device).unsqueeze(0) if force_legal else None
+        idx, probs = self._sample(row, mask, T)
+        move = policy_index[idx]
+        return (move, probs[0]) if return_probs else move
+
+    @torch.no_grad()
     def get_move_from_fen_no_thinking(self, fen, T=1, device="cuda", force_legal=True, return_probs=False):
         planes = board.encode_fens([fen]).to(device)
         logits, _ = self._engine.forward(planes)

@@ -309,6 +309,14 @@ def test_generate_cached_equals_teacher_forced_forward(cuda):
     assert bool((p1.gather(2, s1[:, 1:, None]) > 0).all())
     s0, p0 = m.generate_sequence_raw(planes.to(cuda), T=0)
     assert p0 is None and s0.shape == (B, 192)
+    # the thinking-mode move picker built on it (model_bis.py:321-356)
+    fen = "r1bq1rk1/2pp1ppp/p1n2n2/2b1p3/1pP1P3/1B1P1N2/PP3PPP/RNBQR1K1 b - c3 0 9"
+    legal = {mv[:-1] if mv.endswith("n") else mv for mv in board.legal_moves(fen)}
+    mv, probs = m.get_move_from_fen(fen, T=1, return_probs=True)
+    assert mv in legal and abs(probs.sum().item() - 1) < 1e-4
+    assert torch.equal((probs > 0).cpu(), torch.from_numpy(board.legal_move_mask(fen)).bool())
+    with pytest.raises(ValueError):
+        m.get_move_from_fen(fen, T=0)
 
 
 def test_generate_forced_tokens(cuda):
