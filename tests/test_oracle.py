@@ -131,3 +131,44 @@ def test_masked_policy_matches_reference_formula():
     want = F.softmax((logits + (1 - mask) * -999) / 0.7, -1)
     assert torch.allclose(p, want) and torch.equal(p > 0, mask.bool())
     assert len(policy_index) == 1929
+
+
+def test_gpt_oracle_forward_tokens():
+    """model_bis.py:171-199: targets are the input shifted left with 1928 over the board, the loss ignores 1928,
+    move tokens use the tied embedding plus the positional rows 64.., and nothing before a token depends on it."""
+    torch.manual_seed(1)
+    m = om.test_init_(om.GPTOracle(2, 8, 256), 1)
+    x = torch.rand(2, 8, 8, 19)
+    idx = torch.tensor([[5, 1928, 7], [9, 11, 1927]])
+    logits, loss, targets = m.forward_tokens(x, idx, compute_loss=True)
+    assert logits.shape == (2, 67, 1929)
+    assert targets[0].tolist() == [1928] * 63 + [5, 1928, 7, 1928]          # rolled: the last target wraps to the board filler
+    assert targets[1].tolist() == [1928] * 63 + [9, 11, 1927, 1928]
+    # the mean runs over the 5 counted targets: positions 63 (both rows), 64 (row 1 only), 65 (both)
+    lp = F.log_softmax(logits, -1)
+    want = -(lp[0, 63, 5] + lp[0, 65, 7] + lp[1, 63, 9] + lp[1, 64, 11] + lp[1, 65, 1927]) / 5
+    assert abs(loss.item() - want.item()) < 1e-5
+    # no move tokens: the last-token logits are forward_last's
+    last, none, _ = m.forward_tokens(x, idx[:, :0])
+    assert none is None and torch.allclose(last[:, 0], m.forward_last(x), atol=1e-5)
+    # causality: changing the last move token leaves every earlier position's logits alone
+    idx2 = idx.clone()
+    idx2[:, 2] = 3
+    l2, _, _ = m.forward_tokens(x, idx2, compute_loss=True)
+    assert torch.allclose(l2[:, :66], logits[:, :66], atol=1e-5) and not torch.allclose(l2[:, 66], logits[:, 66])
+    # the embedding of a move token is the tied lm_head row plus pe[64 + j]
+    h = torch.cat((m.FenEncoder(x), m.lm_head.weight[idx]), 1) + m.pe[:67]
+    assert torch.allclose(m.lm_head(m._trunk(h)), logits, atol=1e-5)
+
+
+def test_generation_rules():
+    """model_bis.py:252-259 on hand-made sampler outputs: five end_variation tokens force </thinking> next, the token
+    two places after </thinking> is forced to end, and the counter keeps running afterwards."""
+    EV, ET, END, TH = 1926, 1925, 1927, 1924
+    raw = torch.tensor([[EV, 10, EV, EV, EV, EV, 20, 21, 22, 23, EV, 24],
+                        [1, 2, ET, 3, 4, 5, 6, 7, 8, 9, 10, 11]])
+    seq = om.apply_generation_rules(raw)
+    #            0   1   2   3   4   5   6  7(forced)  8  9(forced)
+    assert seq[0].tolist() == [TH, EV, 10, EV, EV, EV, EV, ET, 21, END, 23, EV, 24]
+    # a sampled </thinking> (no counter involved) also forces end two places later
+    assert seq[1].tolist() == [TH, 1, 2, ET, 3, END, 5, 6, 7, 8, 9, 10, 11]
