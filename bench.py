@@ -93,6 +93,16 @@ def grpo_rollout(a, torch, models, board, dev):
         policy.generate_sequence(planes, T=1, seed=100 + i)
     torch.cuda.synchronize()
     dt = (time.perf_counter() - t0) / a.steps
+    # the same rollout with the token step recorded once into a HIP graph and replayed instead of launched kernel by kernel
+    policy._engine.set_decode_graph(True)
+    policy.generate_sequence(planes, T=1, seed=0)
+    torch.cuda.synchronize()
+    t2 = time.perf_counter()
+    for i in range(a.steps):
+        policy.generate_sequence(planes, T=1, seed=100 + i)
+    torch.cuda.synchronize()
+    replayed = (time.perf_counter() - t2) / a.steps
+    policy._engine.set_decode_graph(False)
     # what the reference's loop costs on the same kernels: one full forward per sampled token over the growing prefix
     seq = torch.randint(0, 1924, (n, 191), generator=torch.Generator().manual_seed(0)).to(dev)
     torch.cuda.synchronize()
@@ -106,6 +116,7 @@ def grpo_rollout(a, torch, models, board, dev):
                       "ms_per_step": round(dt * 1e3, 3), "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "bf16",
                       "data": "synthetic", "config": {"workload": a.workload, "layers": 6, "d_model": 768, "heads": 12, "G": G, "batch": Bp,
                                                       "sampled_tokens_per_s": round(n * 191 / dt, 1),
+                                                      "replayed_graph_ms": round(replayed * 1e3, 3),
                                                       "full_recompute_per_token_ms_estimate": round(naive * 1e3, 1)},
                       "roofline": None, "cpu_baseline": None}))
 

@@ -69,6 +69,7 @@ SIGNATURES = {
     "crl_model_vocab": (_i, [_vp]),
     "crl_model_flops_per_position": (C.c_double, [_vp]),
     "crl_model_set_profiling": (_i, [_vp, _i]),
+    "crl_model_set_decode_graph": (_i, [_vp, _i]),
     "crl_model_get_profile": (_i, [_vp, _vp, _vp, _vp]),
     "crl_model_evaluate_fens": (_i, [_vp, C.POINTER(C.c_char_p), _i, _i, _f, _vp, _vp, _vp, _i]),
     "crl_model_forward_tokens": (_i, [_vp, _vp, _vp, _i, _i, _vp, _vp, _vp]),

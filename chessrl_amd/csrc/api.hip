@@ -195,14 +195,15 @@ int crl_gemm(const void* A, int64_t lda, const void* W, int64_t ldw, void* C, in
              float out_scale, float* amax, int tile, void* stream) {
   if (!A || !W || !C || M < 0 || N < 0 || K <= 0) return arg_fail("crl_gemm: bad arguments");
   if (in_dtype != DT_BF16 && in_dtype != DT_F16 && in_dtype != DT_FP8) return arg_fail("crl_gemm: in_dtype must be bf16, f16 or fp8");
-  if (out_dtype < 0 || out_dtype > 3 || tile < 0 || tile > 3) return arg_fail("crl_gemm: bad out_dtype or tile");
+  if (out_dtype < 0 || out_dtype > 3 || tile < 0 || tile > 4) return arg_fail("crl_gemm: bad out_dtype or tile");
   GemmArgs g;
   std::memset(&g, 0, sizeof(g));
   g.A = A; g.lda = lda; g.W = W; g.ldw = ldw; g.C = C; g.ldc = ldc; g.M = M; g.N = N; g.K = K; g.nsplit = N;
   g.bias = bias; g.act = act; g.descale = descale; g.alpha = alpha; g.res = res; g.ldr = ldr; g.res_dtype = res_dtype;
   g.out_scale = out_scale; g.amax = amax;
   hipError_t e = launch_gemm(g, in_dtype, out_dtype, tile, (hipStream_t)stream);
-  if (e == hipErrorInvalidValue) return arg_fail("crl_gemm: operands must be 16-byte aligned with K*elem_size a multiple of 16");
+  if (e == hipErrorInvalidValue)
+    return arg_fail("crl_gemm: operands must be 16-byte aligned with K*elem_size a multiple of 16");
   return e == hipSuccess ? CRL_OK : hip_fail("crl_gemm", e);
 }
 
@@ -535,6 +536,11 @@ int crl_model_set_profiling(crl_model* m, int on) {
   if (!m) return arg_fail("null model");
   m->impl.profiling = on != 0;
   for (int i = 0; i < 6; ++i) { m->impl.prof_ms[i] = 0; m->impl.prof_n[i] = 0; m->impl.prof_flops[i] = 0; }
+  return CRL_OK;
+}
+int crl_model_set_decode_graph(crl_model* m, int on) {
+  if (!m) return arg_fail("null model");
+  m->impl.decode_graph = on != 0;
   return CRL_OK;
 }
 int crl_model_get_profile(crl_model* m, double* ms6, int64_t* launches6, double* flops6) {

@@ -110,6 +110,8 @@ struct GemmArgs {
   int vec_ok;         // 1 if 4-wide stores/loads along N are aligned for C, C2 and res
   int res_rows;       // >0: the residual has this many rows and row m reads row m % res_rows
   int stream_out;     // 1: the output is far larger than the L2 caches: store it with the non-temporal hint
+  int k_slices;       // >1: workgroup (tile, slice) covers slabs_per_slice 128-byte slabs of K and writes slice `slice` of C [k_slices, M, ldc]
+  int slabs_per_slice;
 };
 
 struct LayerNormArgs {
@@ -219,6 +221,7 @@ struct SampleArgs {
   long end_think, end_tok, end_variation;
   float temperature;
   uint64_t seed;
+  const int* dyn_k;                  // optional device counter: k and step are read from it (graph replays), step_out advances with it
 };
 
 struct ScatterArgs {
@@ -232,8 +235,11 @@ struct ScatterArgs {
 
 // ---- launchers (one per kernel family) -------------------------------------------------
 // in_dt: element type of A and W; out_dt: element type of C/C2; tile: 0 auto, 1 = 64x64,
-// 2 = 128x128, 3 = 256x256 workgroup tile.
+// 2 = 128x128, 3 = 256x256 workgroup tile, 4 = 64x64 tiles with K cut into slices (what 0 picks for few tiles and long K).
 hipError_t launch_gemm(GemmArgs a, int in_dt, int out_dt, int tile, hipStream_t st);
+// Allocates the stream's workspace for K-sliced GEMMs now (it is otherwise allocated by the first launch that needs
+// it, which must not happen while the stream is being recorded into a graph).
+hipError_t gemm_prepare_stream(hipStream_t st);
 hipError_t launch_layernorm(const LayerNormArgs& a, hipStream_t st);
 hipError_t launch_embed(const EmbedArgs& a, hipStream_t st);
 hipError_t launch_token_embed(const TokenEmbedArgs& a, hipStream_t st);
@@ -248,9 +254,15 @@ hipError_t launch_extract_stm(const float* planes, const uint8_t* flags, uint8_t
 hipError_t launch_fill_f32(float* p, float v, long n, hipStream_t st);
 hipError_t launch_convert(const float* src, void* dst, long n, int dt, float scale, hipStream_t st);
 hipError_t launch_kv_store(const void* qkv, void* cache, int B, int T, int Tmax, int C, hipStream_t st);
-hipError_t launch_decode_embed(const int64_t* tok, const float* wte, const float* pe_row, void* out, int B, int C, int V, int out_dtype, hipStream_t st);
-hipError_t launch_decode_attention(const void* q, long ldq, const void* cache, int Tmax, int C, int n, void* out, long ldo, int B, int H,
-                                   int head_dim, int in_dtype, float scale, hipStream_t st);
+// dyn_k (optional, device): the kernels take the token index k from it instead of from their arguments, so one captured
+// graph serves every step: position = 64 + k, keys = 65 + k.
+hipError_t launch_decode_embed(const int64_t* tok, const float* wte, const float* pe, int pos, const int* dyn_k, void* out, int B, int C, int V,
+                               int out_dtype, hipStream_t st);
+hipError_t launch_decode_attention(const void* q, long ldq, const void* cache, int Tmax, int C, int n, const int* dyn_k, void* out, long ldo,
+                                   int B, int H, int head_dim, int in_dtype, float scale, hipStream_t st);
+// staging [B, 2C] -> row (pos or 64 + *dyn_k) of every sequence's [Tmax, 2C] cache
+hipError_t launch_kv_append(const void* staging, void* cache, int B, int Tmax, int C, int pos, const int* dyn_k, hipStream_t st);
+hipError_t launch_add_int(int* p, int v, hipStream_t st);
 hipError_t launch_sample(const SampleArgs& a, hipStream_t st);
 // Back-to-back MFMAs from registers on every CU: sustained TFLOP/s and the clock it ran at.
 hipError_t run_mfma_probe(int dtype, int random_bits, int iters, double* tflops, double* ghz, hipStream_t st);

@@ -22,7 +22,9 @@
 //  * Workgroup ids are remapped so each XCD (ids round-robin over 8 XCDs) walks a
 //    contiguous range of tiles, N fastest: the weight matrix stays in that XCD's L2
 //    and every activation slab is fetched from HBM by one XCD only.
+#include <mutex>
 #include <type_traits>
+#include <unordered_map>
 
 #include "common.hpp"
 
@@ -330,11 +332,16 @@ __global__ void __launch_bounds__(Cfg::NT, Cfg::MIN_WAVES) gemm_kernel(const Gem
     const int per = nblk >> 3;  // full groups of 8
     if (pid < (per << 3)) pid = (pid & 7) * per + (pid >> 3);
   }
+  int slice = 0;
+  if (a.k_slices > 1) { slice = pid % a.k_slices; pid /= a.k_slices; }
   const int tile_m = pid / tiles_n, tile_n = pid - tile_m * tiles_n;
   const int m0 = tile_m * BM, n0 = tile_n * BN;
 
   const long kbytes = (long)a.K * ESZ;
-  const int nslab = (int)((kbytes + 127) >> 7);
+  const int nslab_all = (int)((kbytes + 127) >> 7);
+  // A K-sliced launch walks only this workgroup's slabs and leaves the raw fp32 sums in its own copy of C.
+  const int slab0 = a.k_slices > 1 ? slice * a.slabs_per_slice : 0;
+  const int nslab = a.k_slices > 1 ? min(nslab_all, slab0 + a.slabs_per_slice) : nslab_all;
   const uint8_t* Ab = reinterpret_cast<const uint8_t*>(a.A);
   const uint8_t* Wb = reinterpret_cast<const uint8_t*>(a.W);
   const long lda_b = a.lda * ESZ, ldw_b = a.ldw * ESZ;
@@ -411,8 +418,8 @@ __global__ void __launch_bounds__(Cfg::NT, Cfg::MIN_WAVES) gemm_kernel(const Gem
     arow_sw[tm] = lds_swizzle(ar);
   }
 
-  gload(0);
-  sstore(0, 0);
+  gload(slab0);
+  sstore(0, slab0);
   __syncthreads();
 
   // With FRAG_DB two fragment sets alternate: while the MFMAs of k-step ks run on one set,
@@ -436,8 +443,8 @@ __global__ void __launch_bounds__(Cfg::NT, Cfg::MIN_WAVES) gemm_kernel(const Gem
       for (int tm = 0; tm < TM; ++tm) acc[tn][tm] = mfma_frag<IN_DT>(wf[set][tn], xf[set][tm], acc[tn][tm]);
   };
 
-  for (int slab = 0; slab < nslab; ++slab) {
-    const int stage = Cfg::STAGES == 2 ? (slab & 1) : 0;
+  for (int slab = slab0; slab < nslab; ++slab) {
+    const int stage = Cfg::STAGES == 2 ? ((slab - slab0) & 1) : 0;
     const uint8_t* st = smem + stage * Cfg::STAGE_BYTES;
     const bool more = slab + 1 < nslab;
     if (more) gload(slab + 1);
@@ -468,8 +475,68 @@ __global__ void __launch_bounds__(Cfg::NT, Cfg::MIN_WAVES) gemm_kernel(const Gem
     }
   }
 
+  if (a.k_slices > 1) {
+    GemmArgs b = a;
+    b.C = b.C2 = reinterpret_cast<char*>(a.C) + (size_t)slice * a.M * a.ldc * dtype_size(OUT_DT);
+    gemm_epilogue<Cfg::WM, Cfg::WN, OUT_DT>(b, acc, reinterpret_cast<float*>(smem) + wave * (32 * Cfg::WN),
+                                           m0 + wm * Cfg::WM, n0 + wn * Cfg::WN, lane);
+    return;
+  }
   gemm_epilogue<Cfg::WM, Cfg::WN, OUT_DT>(a, acc, reinterpret_cast<float*>(smem) + wave * (32 * Cfg::WN),
                                          m0 + wm * Cfg::WM, n0 + wn * Cfg::WN, lane);
+}
+
+// ---- second pass of a K-sliced GEMM -------------------------------------------------------------
+// partial [ks, M, ldp] holds the raw fp32 sums of the slices. One thread per output row and group of four columns
+// adds them in slice order (so the result does not depend on which workgroup finished first) and applies the
+// epilogue of the one-pass kernels: C = res + alpha*act(descale*sum + bias), amax, the fp8 output scale, the C/C2 split.
+template <int OUT_DT>
+__global__ void __launch_bounds__(256) splitk_reduce_kernel(const GemmArgs a, const float* partial, int ks, long ldp) {
+  const int groups = (a.N + 3) / 4;
+  const long idx = (long)blockIdx.x * 256 + threadIdx.x;
+  const int m = (int)(idx / groups), n = (int)(idx - (long)m * groups) * 4;
+  float local_amax = 0.f;
+  if (m < a.M) {
+    f32x4_t acc = {0.f, 0.f, 0.f, 0.f};
+    const float* pp = partial + (long)m * ldp + n;
+    for (int s = 0; s < ks; ++s) acc += *reinterpret_cast<const f32x4_t*>(pp + (long)s * a.M * ldp);   // ldp is a multiple of 4 and >= N rounded up
+    float v[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const float b = (a.bias && n + i < a.N) ? a.bias[n + i] : 0.f;
+      v[i] = apply_act(fmaf(acc[i], a.descale, b), a.act);
+    }
+    if (a.res) {
+      const long ro = (long)(a.res_rows > 0 ? m % a.res_rows : m) * a.ldr + n;
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        float rv = 0.f;
+        if (n + i < a.N) {
+          if (a.res_dtype == DT_F32) rv = reinterpret_cast<const float*>(a.res)[ro + i];
+          else {
+            const uint16_t h = reinterpret_cast<const uint16_t*>(a.res)[ro + i];
+            rv = a.res_dtype == DT_F16 ? f16_bits_to_f32(h) : bf16_bits_to_f32(h);
+          }
+        }
+        v[i] = fmaf(v[i], a.alpha, rv);
+      }
+    } else {
+#pragma unroll
+      for (int i = 0; i < 4; ++i) v[i] *= a.alpha;
+    }
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      if (n + i >= a.N) continue;
+      local_amax = fmaxf(local_amax, fabsf(v[i]));
+      const float o = OUT_DT == DT_FP8 ? v[i] * a.out_scale : v[i];
+      if (n + i < a.nsplit) store1<OUT_DT>(a.C, (long)m * a.ldc + n + i, o);
+      else store1<OUT_DT>(a.C2, (long)m * a.ldc2 + (n + i - a.nsplit), o);
+    }
+  }
+  if (a.amax) {
+    local_amax = wave_max(local_amax);
+    if ((threadIdx.x & 63) == 0) atomic_amax(a.amax, local_amax);
+  }
 }
 
 // ---- 256x256 tile fed by direct global->LDS loads ------------------------------------------
@@ -716,8 +783,84 @@ static hipError_t launch_dma(const GemmArgs& a, hipStream_t st) {
   return hipGetLastError();
 }
 
+// Workspace of the K-sliced GEMMs: one per (device, stream a launch is issued or recorded on), so launches that may
+// run at the same time never share one. Lives until the process ends.
+constexpr size_t SPLITK_WS_BYTES = 16u << 20;
+static std::mutex g_ws_mutex;
+static std::unordered_map<uint64_t, float*> g_ws;
+static hipError_t workspace_for(hipStream_t st, float** out) {
+  int dev = 0;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess) return e;
+  const uint64_t key = (reinterpret_cast<uint64_t>(st) << 4) ^ (uint64_t)(dev & 15);
+  std::lock_guard<std::mutex> lock(g_ws_mutex);
+  auto it = g_ws.find(key);
+  if (it != g_ws.end()) { *out = it->second; return hipSuccess; }
+  float* p = nullptr;
+  e = hipMalloc((void**)&p, SPLITK_WS_BYTES);
+  if (e != hipSuccess) return e;
+  g_ws.emplace(key, p);
+  *out = p;
+  return hipSuccess;
+}
+hipError_t gemm_prepare_stream(hipStream_t st) {
+  float* p = nullptr;
+  return workspace_for(st, &p);
+}
+
+// Few output tiles and a long K leave most CUs idle while a few walk K alone (M=128, N=768, K=3072: 24 workgroups
+// of 48 slabs each). Then K is cut into slices, one workgroup per (tile, slice) writes its raw sums, and a second
+// small kernel adds the slices and applies the epilogue. Returns the number of slices (1: not worth it / no room).
+static int splitk_plan(const GemmArgs& a, int esz, bool forced, int* slabs_per_slice) {
+  const long tiles = (long)((a.M + 63) / 64) * ((a.N + 63) / 64);
+  const int nslab = (int)(((long)a.K * esz + 127) >> 7);
+  if (!forced && (tiles > 64 || nslab < 16)) return 1;
+  int ks = (int)std::min<long>(std::max(nslab / 4, 1), (256 + tiles - 1) / tiles);
+  if (forced) ks = std::max(ks, std::min(nslab, 2));
+  const int per = (nslab + ks - 1) / ks;
+  ks = (nslab + per - 1) / per;
+  const long ldp = (a.N + 7) / 8 * 8;
+  if (ks < 2 || (size_t)ks * a.M * ldp * sizeof(float) > SPLITK_WS_BYTES) return 1;
+  *slabs_per_slice = per;
+  return ks;
+}
+
+template <int IN_DT, int OUT_DT>
+static hipError_t launch_splitk(const GemmArgs& a, int ks, int per, hipStream_t st) {
+  float* ws = nullptr;
+  hipError_t e = workspace_for(st, &ws);
+  if (e != hipSuccess) return e;
+  const long ldp = (a.N + 7) / 8 * 8;
+  GemmArgs b = a;
+  b.C = b.C2 = ws; b.ldc = b.ldc2 = ldp; b.nsplit = a.N;
+  b.bias = nullptr; b.res = nullptr; b.amax = nullptr; b.act = ACT_NONE; b.descale = 1.f; b.alpha = 1.f; b.out_scale = 1.f;
+  b.vec_ok = 1; b.stream_out = 0; b.k_slices = ks; b.slabs_per_slice = per;
+  static bool attr_set[16] = {};
+  int dev = 0;
+  (void)hipGetDevice(&dev);
+  auto kern = gemm_kernel<CfgSmall, IN_DT, DT_F32>;
+  if (dev >= 0 && dev < 16 && !attr_set[dev]) {
+    e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, CfgSmall::LDS_BYTES);
+    if (e != hipSuccess) return e;
+    attr_set[dev] = true;
+  }
+  const int tiles = ((a.M + 63) / 64) * ((a.N + 63) / 64);
+  hipLaunchKernelGGL(kern, dim3(tiles * ks), dim3(CfgSmall::NT), CfgSmall::LDS_BYTES, st, b);
+  e = hipGetLastError();
+  if (e != hipSuccess) return e;
+  const long threads = (long)a.M * ((a.N + 3) / 4);
+  hipLaunchKernelGGL((splitk_reduce_kernel<OUT_DT>), dim3((unsigned)((threads + 255) / 256)), dim3(256), 0, st, a, ws, ks, ldp);
+  return hipGetLastError();
+}
+
 template <int IN_DT, int OUT_DT>
 static hipError_t launch_in_out(const GemmArgs& a, int tile, hipStream_t st) {
+  if (tile == 0 || tile == 4) {
+    int per = 0;
+    const int ks = splitk_plan(a, IN_DT == DT_FP8 ? 1 : 2, tile == 4, &per);
+    if (ks > 1) return launch_splitk<IN_DT, OUT_DT>(a, ks, per, st);
+    if (tile == 4) tile = 1;
+  }
   if (tile == 0) {
     // Largest tile that still gives every CU a workgroup.
     const long big = (long)((a.M + 255) / 256) * ((a.N + 255) / 256);
@@ -741,7 +884,7 @@ static hipError_t launch_in(const GemmArgs& a, int out_dt, int tile, hipStream_t
 }
 
 // in_dt: element type of A and W; out_dt: element type of C/C2; tile: 0 auto, 1 = 64x64,
-// 2 = 128x128, 3 = 256x256 (direct-to-LDS loads).
+// 2 = 128x128, 3 = 256x256 (direct-to-LDS loads), 4 = 64x64 tiles with K cut into slices.
 hipError_t launch_gemm(GemmArgs a, int in_dt, int out_dt, int tile, hipStream_t st) {
   if (a.M <= 0 || a.N <= 0) return hipSuccess;
   const int esz = in_dt == DT_FP8 ? 1 : 2;

@@ -97,6 +97,7 @@ Model::Model(const crl_model_config& c) : cfg(c) {
 
 Model::~Model() {
   for (void* p : gen_allocs) (void)hipFree(p);
+  if (cap_stream) (void)hipStreamDestroy(cap_stream);
   for (void* p : allocs) (void)hipFree(p);
   for (void* p : ws_allocs) (void)hipFree(p);
   for (auto& e : prof_events) { (void)hipEventDestroy(e.a); (void)hipEventDestroy(e.b); }
@@ -678,6 +679,8 @@ int Model::generate(const float* planes, int B, int steps, float temperature, ui
     rc = galloc((void**)&gen_tok, sizeof(int64_t) * B); if (rc) return rc;
     rc = galloc((void**)&gen_zeros, sizeof(int32_t) * B); if (rc) return rc;
     rc = galloc((void**)&gen_logits, sizeof(float) * (size_t)B * VOCAB_RL); if (rc) return rc;
+    rc = galloc((void**)&gen_kv_stage, (size_t)B * 2 * C * 2); if (rc) return rc;
+    rc = galloc((void**)&gen_k, 256); if (rc) return rc;
     kv_B = B; kv_Tmax = Tmax;
   }
   const int hd = cfg.head_dtype, ad = cfg.act_dtype;
@@ -687,6 +690,8 @@ int Model::generate(const float* planes, int B, int steps, float temperature, ui
   {
     std::vector<int64_t> first(B, START_THINK);
     std::vector<int32_t> zeros(B, 0);
+    const int first_replayed = 2;
+    HIPCHK(hipMemcpyAsync(gen_k, &first_replayed, sizeof(int), hipMemcpyHostToDevice, st));
     HIPCHK(hipMemcpyAsync(gen_tok, first.data(), sizeof(int64_t) * B, hipMemcpyHostToDevice, st));
     HIPCHK(hipMemcpyAsync(gen_zeros, zeros.data(), sizeof(int32_t) * B, hipMemcpyHostToDevice, st));
     HIPCHK(hipMemcpy2DAsync(seq, sizeof(int64_t) * (steps + 1), gen_tok, sizeof(int64_t), sizeof(int64_t), B, hipMemcpyDeviceToDevice, st));
@@ -698,35 +703,76 @@ int Model::generate(const float* planes, int B, int steps, float temperature, ui
   RUN(forward_chunk(planes, nullptr, nullptr, gen_tok, 1, B, gen_logits, nullptr, nullptr, false, st));
   kv_capture = false;
   const float attn_scale = 1.0f / std::sqrt((float)hs);
-  for (int k = 1; k <= steps; ++k) {
+  // One token step: sample token k from gen_logits, then (unless it is the last) run it through the trunk at position
+  // 64 + k against the cache and leave the next logits in gen_logits. With `dyn` the kernels read k from device memory
+  // and the step ends by advancing it, so the same launches serve every k (the body of the replayed graph).
+  auto token_step = [&](int k, const int* dyn, bool sample_only, hipStream_t s) -> int {
+    int rc = CRL_OK;
+#define STEP_HIP(expr) do { hipError_t he_ = (expr); if (he_ != hipSuccess) { set_error(std::string("generate: ") + hipGetErrorString(he_)); return CRL_ERR_HIP; } } while (0)
+#define STEP_RUN(call) do { rc = (call); if (rc) return rc; } while (0)
     SampleArgs sa;
     std::memset(&sa, 0, sizeof(sa));
     sa.logits = gen_logits; sa.ldl = VOCAB_RL; sa.seq = seq; sa.ld_seq = steps + 1; sa.tok_out = gen_tok; sa.num_zeros = gen_zeros;
-    sa.step_out = step_out ? step_out + (size_t)(k - 1) * VOCAB_RL : nullptr; sa.ld_out = (long)steps * VOCAB_RL;
-    sa.B = B; sa.V = VOCAB_RL; sa.k = k; sa.step = k; sa.rules = rules; sa.out_logits = out_logits;
+    sa.step_out = !step_out ? nullptr : dyn ? step_out : step_out + (size_t)(k - 1) * VOCAB_RL;
+    sa.ld_out = (long)steps * VOCAB_RL;
+    sa.B = B; sa.V = VOCAB_RL; sa.k = k; sa.step = k; sa.rules = rules; sa.out_logits = out_logits; sa.dyn_k = dyn;
     sa.end_think = END_THINK; sa.end_tok = END; sa.end_variation = END_VARIATION; sa.temperature = temperature; sa.seed = seed;
-    hipError_t he = launch_sample(sa, st);
-    if (he != hipSuccess) { force_16bit = false; HIPCHK(he); }
-    if (k == steps) break;
+    STEP_HIP(launch_sample(sa, s));
+    if (sample_only) return CRL_OK;
     const int pos = 64 + k;    // sequence position of token k
-    he = launch_decode_embed(gen_tok, wte_f32, pe_f32 + (size_t)pos * C, ws.x, B, C, VOCAB_RL, xdt, st);
-    if (he != hipSuccess) { force_16bit = false; HIPCHK(he); }
+    STEP_HIP(launch_decode_embed(gen_tok, wte_f32, pe_f32, pos, dyn, ws.x, B, C, VOCAB_RL, xdt, s));
     for (int l = 0; l < L; ++l) {
       const Layer& ly = layers[l];
-      RUN(lnorm(ws.x, C, xdt, ly.ln1_g, ly.ln1_b, ws.h, ad, nullptr, 1.f, C, B, C, nullptr, st));
-      { // q -> ws.qkv [B,C]; k|v -> row `pos` of every sequence's cache
+      STEP_RUN(lnorm(ws.x, C, xdt, ly.ln1_g, ly.ln1_b, ws.h, ad, nullptr, 1.f, C, B, C, nullptr, s));
+      if (dyn) {
+        // q -> ws.qkv [B,C]; k|v -> staging, then to the row the counter names
+        GOpt o; o.C2 = gen_kv_stage; o.ldc2 = 2 * C; o.nsplit = C;
+        STEP_RUN(gemm(ly.qkv, ws.h, C, ad, ws.qkv, C, ad, B, o, s));
+        STEP_HIP(launch_kv_append(gen_kv_stage, kv_layers[l], B, kv_Tmax, C, 0, dyn, s));
+      } else {
+        // q -> ws.qkv [B,C]; k|v -> row `pos` of every sequence's cache
         GOpt o; o.C2 = reinterpret_cast<uint16_t*>(kv_layers[l]) + (size_t)pos * 2 * C; o.ldc2 = (long)kv_Tmax * 2 * C; o.nsplit = C;
-        RUN(gemm(ly.qkv, ws.h, C, ad, ws.qkv, C, ad, B, o, st)); }
-      he = launch_decode_attention(ws.qkv, C, kv_layers[l], kv_Tmax, C, pos + 1, ws.ao, C, B, H, hs, ad, attn_scale, st);
-      if (he != hipSuccess) { force_16bit = false; HIPCHK(he); }
-      { GOpt o; o.res = ws.x; o.ldr = C; o.res_dt = xdt; RUN(gemm(ly.proj, ws.ao, C, ad, ws.x, C, xdt, B, o, st)); }
-      RUN(lnorm(ws.x, C, xdt, ly.ln2_g, ly.ln2_b, ws.h, ad, nullptr, 1.f, C, B, C, nullptr, st));
-      { GOpt o; o.act = ACT_GELU; RUN(gemm(ly.ff1, ws.h, C, ad, ws.f, F, ad, B, o, st)); }
-      { GOpt o; o.res = ws.x; o.ldr = C; o.res_dt = xdt; RUN(gemm(ly.ff2, ws.f, F, ad, ws.x, C, xdt, B, o, st)); }
+        STEP_RUN(gemm(ly.qkv, ws.h, C, ad, ws.qkv, C, ad, B, o, s));
+      }
+      STEP_HIP(launch_decode_attention(ws.qkv, C, kv_layers[l], kv_Tmax, C, pos + 1, dyn, ws.ao, C, B, H, hs, ad, attn_scale, s));
+      { GOpt o; o.res = ws.x; o.ldr = C; o.res_dt = xdt; STEP_RUN(gemm(ly.proj, ws.ao, C, ad, ws.x, C, xdt, B, o, s)); }
+      STEP_RUN(lnorm(ws.x, C, xdt, ly.ln2_g, ly.ln2_b, ws.h, ad, nullptr, 1.f, C, B, C, nullptr, s));
+      { GOpt o; o.act = ACT_GELU; STEP_RUN(gemm(ly.ff1, ws.h, C, ad, ws.f, F, ad, B, o, s)); }
+      { GOpt o; o.res = ws.x; o.ldr = C; o.res_dt = xdt; STEP_RUN(gemm(ly.ff2, ws.f, F, ad, ws.x, C, xdt, B, o, s)); }
     }
-    RUN(lnorm(ws.x, C, xdt, lnf_g, lnf_b, ws.hl, hd, nullptr, 1.f, C, B, C, nullptr, st));
-    { GOpt o; RUN(gemm(lm_head, ws.hl, C, hd, gen_logits, VOCAB_RL, DT_F32, B, o, st)); }
+    STEP_RUN(lnorm(ws.x, C, xdt, lnf_g, lnf_b, ws.hl, hd, nullptr, 1.f, C, B, C, nullptr, s));
+    { GOpt o; STEP_RUN(gemm(lm_head, ws.hl, C, hd, gen_logits, VOCAB_RL, DT_F32, B, o, s)); }
+    if (dyn) STEP_HIP(launch_add_int(gen_k, 1, s));
+    return CRL_OK;
+#undef STEP_HIP
+#undef STEP_RUN
+  };
+  // Steps 2 .. steps-1 are identical launches apart from k: they are recorded once and replayed, which takes the host's
+  // launch cost (some 8 launches per layer) off the critical path. Step 1 runs eagerly first so that every kernel's
+  // one-time set-up has happened before the recording; the timers of the profiling mode cannot be recorded, so that
+  // mode stays on plain launches.
+  const bool graphed = decode_graph && !profiling && steps >= 4;
+  int k = 1;
+  if (graphed) {
+    RUN(token_step(1, nullptr, false, st));
+    if (!cap_stream) HIPCHK(hipStreamCreateWithFlags(&cap_stream, hipStreamNonBlocking));
+    HIPCHK(gemm_prepare_stream(cap_stream));
+    hipGraph_t graph = nullptr;
+    hipGraphExec_t exec = nullptr;
+    hipError_t he = hipStreamBeginCapture(cap_stream, hipStreamCaptureModeRelaxed);
+    if (he != hipSuccess) { force_16bit = false; HIPCHK(he); }
+    rc = token_step(2, gen_k, false, cap_stream);
+    he = hipStreamEndCapture(cap_stream, &graph);   // always ends the recording, also after a failed launch
+    if (rc == CRL_OK && he == hipSuccess) he = hipGraphInstantiate(&exec, graph, nullptr, nullptr, 0);
+    for (k = 2; rc == CRL_OK && he == hipSuccess && k < steps; ++k) he = hipGraphLaunch(exec, st);
+    if (rc == CRL_OK && he == hipSuccess) he = hipStreamSynchronize(st);   // the graph is destroyed below
+    if (exec) (void)hipGraphExecDestroy(exec);
+    if (graph) (void)hipGraphDestroy(graph);
+    if (rc) { force_16bit = false; return rc; }
+    if (he != hipSuccess) { force_16bit = false; HIPCHK(he); }
+    k = steps;
   }
+  for (; k <= steps; ++k) RUN(token_step(k, nullptr, k == steps, st));
 #undef RUN
   force_16bit = false;
   prof_collect(st);

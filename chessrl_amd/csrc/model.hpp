@@ -72,6 +72,10 @@ struct Model {
   int64_t* gen_tok = nullptr;
   int32_t* gen_zeros = nullptr;
   float* gen_logits = nullptr;
+  void* gen_kv_stage = nullptr;     // [B, 2C] k|v of the newest token inside a replayed step
+  int* gen_k = nullptr;             // device counter: index of the token a replayed step samples
+  hipStream_t cap_stream = nullptr; // records the step graph (nothing executes on it)
+  bool decode_graph = false;
   bool kv_capture = false;     // forward_chunk copies every layer's keys|values into the cache
   bool force_16bit = false;    // forward_chunk ignores cfg.fp8
 

@@ -294,6 +294,9 @@ class _Engine:
     def set_profiling(self, on):
         check(lib().crl_model_set_profiling(self.handle, 1 if on else 0), "crl_model_set_profiling")
 
+    def set_decode_graph(self, on):
+        check(lib().crl_model_set_decode_graph(self.handle, 1 if on else 0), "crl_model_set_decode_graph")
+
     def get_profile(self):
         ms = (C.c_double * 6)()
         n = (C.c_int64 * 6)()

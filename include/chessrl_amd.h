@@ -97,7 +97,10 @@ int crl_random_positions(uint64_t seed, int n, int max_plies, double late_fracti
  * A [M,K] (lda), W [N,K] (ldw) of in_dtype (bf16/f16/fp8); C [M,N] (ldc) of out_dtype;
  * bias fp32[N] or NULL; res [M,N] of res_dtype (f32/bf16) or NULL; for an fp8 output the
  * value is multiplied by out_scale before conversion; amax (device float, optional)
- * accumulates max|value|. tile: 0 = automatic. */
+ * accumulates max|value|. tile: 0 = automatic, 1-3 = the 64x64 / 128x128 / 256x256 workgroup tile, 4 = 64x64 tiles
+ * with K cut into slices (what 0 picks when at most 64 tiles would each walk 1 KB or more of K per row): one workgroup
+ * per (tile, slice) leaves raw fp32 sums in a workspace of 16 MB that the library keeps per stream, and a second
+ * kernel adds them in slice order and applies the epilogue, so results do not vary from launch to launch. */
 int crl_gemm(const void* A, int64_t lda, const void* W, int64_t ldw, void* C, int64_t ldc,
              int M, int N, int K, int in_dtype, int out_dtype,
              const float* bias, int act, float descale, float alpha,
@@ -186,9 +189,15 @@ int crl_model_forward_tokens(crl_model* m, const float* planes, const int64_t* i
  * token two places after a </thinking> is end. step_out [B, steps, 1929] (optional) receives every step's
  * probabilities, or its logits when out_logits != 0 (return_logits of :266). The 65-token prefix is run once; every
  * later token costs one row per sequence against the cache (the reference re-runs the whole prefix per token).
- * steps <= rows(pe) - 64 and <= 960; B*65 tokens must fit one micro-batch. Runs in the 16-bit type also for fp8 models. */
+ * steps <= rows(pe) - 64 and <= 960; B*65 tokens must fit one micro-batch. Runs in the 16-bit type also for fp8 models.
+ * crl_model_set_decode_graph(m, 1) records the per-token launches once into a HIP graph (from the second token on;
+ * the kernels then read the token index from a device counter) and replays it; results are bit-identical, the call
+ * returns after the stream has drained, and the stream must not itself be under capture. It is off by default: a
+ * token step is bound by its kernels' run time on the device, not by the host's launches (measured: no gain at 128
+ * sequences), so the option is for hosts that cannot keep up. The profiling mode always launches plainly. */
 int crl_model_generate(crl_model* m, const float* planes, int B, int steps, float temperature, uint64_t seed, int rules,
                        int64_t* sequences, float* step_out, int out_logits, void* stream);
+int crl_model_set_decode_graph(crl_model* m, int on);
 /* Host front-end of leaf evaluation: n FEN strings in host memory -> results in host memory. Replaces the per-FEN
  * Python of model_bis.py:358-398 and new_paradigm/value.py:214-243,275-317 (encode_fens, the legal-move loop with
  * policy_index.index per move, mask, softmax/arg-max) for whole batches. The positions are walked in chunks of

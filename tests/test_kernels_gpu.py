@@ -59,6 +59,74 @@ def test_gemm_bf16(cuda, M, N, K, tile):
     assert torch.allclose(out, ref, rtol=1e-4, atol=1e-3 * math.sqrt(K / 64)), (out - ref).abs().max()
 
 
+@pytest.mark.parametrize("M,N,K", [
+    (128, 768, 3072), (128, 2304, 768), (1, 1929, 768), (16, 1929, 256), (100, 1929, 256), (37, 3, 128), (8, 128, 8192),
+    (200, 768, 1000), (256, 16, 40), (300, 100, 264), (129, 250, 8), (64, 3072, 768), (64, 128, 8192),
+])
+@pytest.mark.parametrize("dt", [torch.bfloat16, torch.float16])
+def test_gemm_k_slices(cuda, M, N, K, dt):
+    """64x64 tiles with K cut into slices and a second pass that adds them (tile 4; tile 0 picks it for few tiles and
+    long K): against the fp32 product of the same 16-bit operands, bit-identical from launch to launch, and equal to
+    the one-pass kernel up to summation order."""
+    torch.manual_seed(M * 11 + K)
+    A = torch.randn(M, K, device=cuda).to(dt)
+    W = (torch.randn(N, K, device=cuda) * 0.05).to(dt)
+    bias = torch.randn(N, device=cuda)
+    ldc = ((N + 7) // 8) * 8
+    outs = [run_gemm(A, W, _lib.F32, bias=bias, tile=4, ldc=ldc).clone() for _ in range(3)]
+    ref = A.float() @ W.float().t() + bias
+    assert torch.allclose(outs[0], ref, rtol=1e-4, atol=1e-3 * math.sqrt(max(K, 64) / 64)), (outs[0] - ref).abs().max()
+    assert torch.equal(outs[0], outs[1]) and torch.equal(outs[0], outs[2])
+    other = run_gemm(A, W, _lib.F32, bias=bias, tile=1, ldc=ldc)
+    assert torch.allclose(outs[0], other, rtol=1e-4, atol=1e-3 * math.sqrt(max(K, 64) / 64))
+    auto = run_gemm(A, W, _lib.F32, bias=bias, tile=0, ldc=ldc)
+    if (M, N, K) in ((128, 768, 3072), (8, 128, 8192), (64, 128, 8192)):
+        assert torch.equal(auto, outs[0])          # the automatic choice slices these
+    assert torch.allclose(auto, ref, rtol=1e-4, atol=1e-3 * math.sqrt(max(K, 64) / 64))
+    # a row stride of C that rules out vector stores
+    assert torch.equal(run_gemm(A, W, _lib.F32, bias=bias, tile=4, ldc=N + 1), outs[0])
+
+
+@pytest.mark.parametrize("act", [0, 1, 2, 3])
+@pytest.mark.parametrize("out_dt", [_lib.BF16, _lib.F16, _lib.F32])
+def test_gemm_k_slices_epilogue(cuda, act, out_dt):
+    torch.manual_seed(act + 10)
+    M, N, K = 150, 388, 1536
+    A = torch.randn(M, K, device=cuda).bfloat16()
+    W = (torch.randn(N, K, device=cuda) * 0.03).bfloat16()
+    bias = torch.randn(N, device=cuda)
+    tol = {_lib.BF16: 2 ** -8, _lib.F16: 2 ** -10, _lib.F32: 1e-4}[out_dt]
+    for res_dt in (TORCH_DT[out_dt], torch.float32):
+        res = torch.randn(M, N, device=cuda).to(res_dt)
+        amax = torch.zeros(1, device=cuda)
+        out = run_gemm(A, W, out_dt, bias=bias, act=act, alpha=0.43, res=res, amax=amax, tile=4)
+        ref = res.float() + 0.43 * ref_act(A.float() @ W.float().t() + bias, act)
+        assert torch.allclose(out.float(), ref, rtol=tol, atol=tol * 4), (out.float() - ref).abs().max()
+        assert abs(amax.item() - ref.abs().max().item()) <= 1e-3 * ref.abs().max().item()
+    out = run_gemm(A, W, out_dt, act=act, alpha=-1.5, tile=4)
+    ref = -1.5 * ref_act(A.float() @ W.float().t(), act)
+    assert torch.allclose(out.float(), ref, rtol=tol, atol=tol * 4)
+
+
+def test_gemm_k_slices_fp8(cuda):
+    torch.manual_seed(3)
+    M, N, K = 96, 256, 4096
+    x = torch.randn(M, K, device=cuda)
+    w = torch.randn(N, K, device=cuda) * 0.02
+    sx, sw = 448.0 / x.abs().max().item(), 448.0 / w.abs().max().item()
+    A = (x * sx).to(torch.float8_e4m3fn)
+    W = (w * sw).to(torch.float8_e4m3fn)
+    bias = torch.randn(N, device=cuda) * 0.1
+    ref = (A.float() @ W.float().t()) / (sx * sw) + bias
+    for tile in (4, 0):
+        out = run_gemm(A, W, _lib.F32, bias=bias, descale=1.0 / (sx * sw), tile=tile)
+        assert torch.allclose(out, ref, rtol=1e-4, atol=1e-4), (out - ref).abs().max()
+    so = 448.0 / ref.abs().max().item()
+    q = run_gemm(A, W, _lib.FP8, bias=bias, descale=1.0 / (sx * sw), out_scale=so, tile=4)
+    deq = q.view(torch.float8_e4m3fn).float() / so
+    assert (deq - ref).abs().max() <= ref.abs().max() * 2 ** -3
+
+
 @pytest.mark.parametrize("act", [0, 1, 2, 3])
 @pytest.mark.parametrize("out_dt", [_lib.BF16, _lib.F16, _lib.F32])
 def test_gemm_epilogue(cuda, act, out_dt):

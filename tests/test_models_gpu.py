@@ -319,6 +319,33 @@ def test_generate_cached_equals_teacher_forced_forward(cuda):
         m.get_move_from_fen(fen, T=0)
 
 
+def test_generate_replayed_graph_equals_plain_launches(cuda):
+    """The recorded-and-replayed token step gives bit-identical sequences and per-step probabilities to plain
+    launches: temperature sampling with the forced-token rules, on the default stream and on a side stream, twice
+    in a row with a different length (the graph is recorded per call)."""
+    B = 6
+    oracle = om.test_init_(om.GPTOracle(3, 8, 256), seed=9)
+    planes, _ = positions(B, seed=10)
+    m = models.GPT(models.GPTConfig(block_size=256, vocab_size=1929, n_layer=3, n_head=8, n_embd=256))
+    m.load_state_dict(oracle.state_dict())
+    x = planes.to(cuda)
+    for steps, stream in ((60, None), (33, torch.cuda.Stream()), (4, None)):
+        out = {}
+        for graph in (False, True):
+            m._engine.set_decode_graph(graph)
+            if stream is None:
+                out[graph] = m._engine.generate(x, steps, T=1.0, seed=21, rules=True, want_step_out=True)
+            else:
+                stream.wait_stream(torch.cuda.current_stream())
+                with torch.cuda.stream(stream):
+                    out[graph] = m._engine.generate(x, steps, T=1.0, seed=21, rules=True, want_step_out=True)
+                stream.synchronize()
+        torch.cuda.synchronize()
+        assert torch.equal(out[False][0], out[True][0]), steps
+        assert torch.equal(out[False][1], out[True][1]), steps
+    m._engine.set_decode_graph(False)
+
+
 def test_generate_forced_tokens(cuda):
     """generate_sequence's bookkeeping (model_bis.py:252-259) on a model rigged to prefer end_variation: the sequences
     equal the rule application of the oracle to the arg-max of the recorded step logits."""
