@@ -16,6 +16,7 @@ LIB = os.path.join(HERE, "libchessrl_amd.so")
 SOURCES = [
     "host/chess.cpp",
     "kernels/gemm.hip",
+    "kernels/gemm_dma.hip",
     "kernels/norm_embed.hip",
     "kernels/attention.hip",
     "kernels/heads.hip",

@@ -112,6 +112,7 @@ struct GemmArgs {
   int stream_out;     // 1: the output is far larger than the L2 caches: store it with the non-temporal hint
   int k_slices;       // >1: workgroup (tile, slice) covers slabs_per_slice 128-byte slabs of K and writes slice `slice` of C [k_slices, M, ldc]
   int slabs_per_slice;
+  int k_parallel;     // 1: tile 0 may pick the K-sliced / K-grouped kernels, whose summation order over K differs from the tiled kernels'
 };
 
 struct LayerNormArgs {
@@ -235,7 +236,10 @@ struct ScatterArgs {
 
 // ---- launchers (one per kernel family) -------------------------------------------------
 // in_dt: element type of A and W; out_dt: element type of C/C2; tile: 0 auto, 1 = 64x64,
-// 2 = 128x128, 3 = 256x256 workgroup tile, 4 = 64x64 tiles with K cut into slices (what 0 picks for few tiles and long K).
+// 2 = 128x128, 3 = 256x256 workgroup tile, 4 = 64x64 tiles with K cut into slices, 5 = 64x64 tiles whose K slabs four
+// groups of waves take in turn. Tiles 1-3 add up K in the same order, so with tile 0 a row's result does not depend on
+// how many other rows the call has; 4 and 5 are picked by tile 0 only when a.k_parallel is set (few tiles, where they
+// are faster).
 hipError_t launch_gemm(GemmArgs a, int in_dt, int out_dt, int tile, hipStream_t st);
 // Allocates the stream's workspace for K-sliced GEMMs now (it is otherwise allocated by the first launch that needs
 // it, which must not happen while the stream is being recorded into a graph).

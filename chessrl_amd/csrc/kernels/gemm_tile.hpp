@@ -1,0 +1,296 @@
+// Device code shared by the GEMM kernels of gemm.hip (register-staged 64x64 / 128x128 tiles) and gemm_dma.hip
+// (256x256 tile fed by direct global->LDS loads): MFMA operand fragments read from swizzled LDS rows, the output
+// stores, and the epilogue C = res + alpha*act(descale*acc + bias) with its amax, fp8 scaling and C/C2 split.
+#pragma once
+#include <type_traits>
+
+#include "common.hpp"
+
+namespace crl {
+
+__device__ __forceinline__ int lds_swizzle(int row) { return (row ^ (row >> 3)) & 7; }
+
+// Compile-time loop: f is called with std::integral_constant<int, I> for I in [0, N), so
+// register arrays indexed by I never need dynamic indexing whatever the body size.
+template <int I, int N, typename F>
+__device__ __forceinline__ void static_for(F&& f) {
+  if constexpr (I < N) {
+    f(std::integral_constant<int, I>{});
+    static_for<I + 1, N>(f);
+  }
+}
+
+// One MFMA operand fragment of a lane: 16 bytes (2-byte types, 8 k-elements) or
+// 32 bytes (fp8, 32 k-elements) of one LDS row.
+template <int IN_DT>
+struct Frag {
+  i32x4_t lo;
+};
+template <>
+struct Frag<DT_FP8> {
+  i32x4_t lo, hi;
+};
+
+template <int IN_DT>
+__device__ __forceinline__ Frag<IN_DT> load_frag(const uint8_t* row, int sw, int ks, int g) {
+  Frag<IN_DT> f;
+  if constexpr (IN_DT == DT_FP8) {
+    const int c0 = 4 * ks + 2 * g;
+    f.lo = *reinterpret_cast<const i32x4_t*>(row + ((c0 ^ sw) << 4));
+    f.hi = *reinterpret_cast<const i32x4_t*>(row + (((c0 + 1) ^ sw) << 4));
+  } else {
+    const int c0 = 2 * ks + g;
+    f.lo = *reinterpret_cast<const i32x4_t*>(row + ((c0 ^ sw) << 4));
+  }
+  return f;
+}
+
+template <int IN_DT>
+__device__ __forceinline__ f32x16_t mfma_frag(const Frag<IN_DT>& w, const Frag<IN_DT>& x, f32x16_t acc) {
+  if constexpr (IN_DT == DT_FP8) {
+    i32x8_t wv = {w.lo[0], w.lo[1], w.lo[2], w.lo[3], w.hi[0], w.hi[1], w.hi[2], w.hi[3]};
+    i32x8_t xv = {x.lo[0], x.lo[1], x.lo[2], x.lo[3], x.hi[0], x.hi[1], x.hi[2], x.hi[3]};
+    return __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(wv, xv, acc, 0, 0, 0, 0, 0, 0);
+  } else if constexpr (IN_DT == DT_BF16) {
+    return __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, w.lo), __builtin_bit_cast(bf16x8_t, x.lo), acc, 0, 0, 0);
+  } else {
+    return __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8_t, w.lo), __builtin_bit_cast(f16x8_t, x.lo), acc, 0, 0, 0);
+  }
+}
+
+template <int OUT_DT>
+__device__ __forceinline__ void store1(void* base, long off, float v) {
+  if constexpr (OUT_DT == DT_F32) reinterpret_cast<float*>(base)[off] = v;
+  else if constexpr (OUT_DT == DT_BF16) reinterpret_cast<uint16_t*>(base)[off] = f32_to_bf16_bits(v);
+  else if constexpr (OUT_DT == DT_F16) reinterpret_cast<uint16_t*>(base)[off] = f32_to_f16_bits(v);
+  else reinterpret_cast<uint8_t*>(base)[off] = f32_to_fp8(v);
+}
+
+// Orders this wave's LDS traffic (LDS executes one wave's operations in issue order) and
+// keeps the compiler from moving accesses across the point.
+__device__ __forceinline__ void wave_lds_fence() {
+  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+  __builtin_amdgcn_wave_barrier();
+  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+}
+
+// NT: store with the non-temporal hint, so a streamed output does not evict the operands from L2.
+template <int OUT_DT, int NT = 0>
+__device__ __forceinline__ void store8(void* base, long off, const float v[8]) {
+  auto put = [](i32x4_t* p, i32x4_t x) {
+    if constexpr (NT) __builtin_nontemporal_store(x, p);
+    else *p = x;
+  };
+  if constexpr (OUT_DT == DT_F32) {
+    i32x4_t* p = reinterpret_cast<i32x4_t*>(reinterpret_cast<float*>(base) + off);
+    put(p, i32x4_t{(int)__float_as_uint(v[0]), (int)__float_as_uint(v[1]), (int)__float_as_uint(v[2]), (int)__float_as_uint(v[3])});
+    put(p + 1, i32x4_t{(int)__float_as_uint(v[4]), (int)__float_as_uint(v[5]), (int)__float_as_uint(v[6]), (int)__float_as_uint(v[7])});
+  } else if constexpr (OUT_DT == DT_BF16) {
+    put(reinterpret_cast<i32x4_t*>(reinterpret_cast<uint16_t*>(base) + off),
+        i32x4_t{(int)pack_bf16x2(v[0], v[1]), (int)pack_bf16x2(v[2], v[3]), (int)pack_bf16x2(v[4], v[5]), (int)pack_bf16x2(v[6], v[7])});
+  } else if constexpr (OUT_DT == DT_F16) {
+    uint32_t w[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) w[i] = (uint32_t)f32_to_f16_bits(v[2 * i]) | ((uint32_t)f32_to_f16_bits(v[2 * i + 1]) << 16);
+    put(reinterpret_cast<i32x4_t*>(reinterpret_cast<uint16_t*>(base) + off), i32x4_t{(int)w[0], (int)w[1], (int)w[2], (int)w[3]});
+  } else {
+    typedef int i32x2_t __attribute__((ext_vector_type(2)));
+    const i32x2_t x = {(int)pack_fp8x4(v[0], v[1], v[2], v[3]), (int)pack_fp8x4(v[4], v[5], v[6], v[7])};
+    i32x2_t* p = reinterpret_cast<i32x2_t*>(reinterpret_cast<uint8_t*>(base) + off);
+    if constexpr (NT) __builtin_nontemporal_store(x, p);
+    else *p = x;
+  }
+}
+
+// Shared epilogue. acc[tn][tm][r] is output row m = mw0 + tm*32 + lr, column
+// n = nw0 + tn*32 + 8*(r/4) + 4*g + (r%4) (lr = lane%32, g = lane/32); sC is this wave's
+// private LDS patch of 32 x WN floats.
+//
+// Each 32 x WN strip of the wave tile goes through the patch (16-byte chunks XOR-swizzled by
+// row) so that a lane ends up with 8 consecutive columns of one row: stores, residual loads
+// and bias loads are 16-byte vectors (32 for fp32) and every store instruction writes whole
+// row segments. A lane keeps the same 8 columns for all rows, so its bias is loaded once. The
+// residual of strip t+1 is requested before strip t is processed (two register sets), which
+// takes its memory latency off the critical path; the activation is selected once per strip.
+//
+// The branches for tiles that hang over an edge of C or meet an unaligned row stride are marked unlikely, so that the
+// compiler moves them out of the straight path. Left inline between the vector accesses they put a taken jump over a
+// kilobyte of cold code in front of every store and residual load; identical kernels then ran 5-10 % apart depending
+// on where the code object happened to place them (instruction-cache misses at the jump targets), and 5 % slower than
+// this form at best. (A second, compile-time variant of the epilogue for tiles entirely inside C was tried on top:
+// two inlined copies push the 256x256 kernel into register spills.)
+template <int WM, int WN, int OUT_DT>
+__device__ __forceinline__ void gemm_epilogue(const GemmArgs& a, f32x16_t (&acc)[WN / 32][WM / 32], float* sC, int mw0, int nw0, int lane) {
+  constexpr int TM = WM / 32, TN = WN / 32, CH4 = WN / 4, CP = WN / 8, RSTEP = 64 / CP, ITERS = 32 / RSTEP;
+  const int lr = lane & 31, g = lane >> 5;
+  const int ec = lane % CP, er = lane / CP;
+  const int n = nw0 + ec * 8;
+  const bool n_ok = n < a.N;
+  const bool full = a.vec_ok && (n + 7 < a.N) && ((n < a.nsplit) == (n + 7 < a.nsplit));
+  float bias8[8];
+  if (__builtin_expect(a.bias != nullptr && n + 7 < a.N && (reinterpret_cast<uintptr_t>(a.bias) & 15) == 0, 1)) {
+    const f32x4_t b0 = *reinterpret_cast<const f32x4_t*>(a.bias + n), b1 = *reinterpret_cast<const f32x4_t*>(a.bias + n + 4);
+#pragma unroll
+    for (int e = 0; e < 4; ++e) { bias8[e] = b0[e]; bias8[4 + e] = b1[e]; }
+  } else {
+#pragma unroll
+    for (int e = 0; e < 8; ++e) bias8[e] = (a.bias && n + e < a.N) ? a.bias[n + e] : 0.f;
+  }
+  const int res_dt = a.res_dtype;
+  const float descale = a.descale, alpha = a.alpha;
+  float local_amax = 0.f;
+
+  // Raw residual bits, 16 bytes per step and set. 16-bit residuals use the two sets as a double
+  // buffer over strips; an fp32 residual (8 values = 32 bytes) uses both sets for the current
+  // strip (low and high half), i.e. it is fetched at the start of its own strip.
+  const bool res32 = res_dt == DT_F32;
+  uint4 rraw[2][ITERS];
+  auto load_res = [&](int tm, int set, int half) {
+#pragma unroll
+    for (int it = 0; it < ITERS; ++it) {
+      const int m = mw0 + tm * 32 + er + it * RSTEP;
+      uint4 val = make_uint4(0, 0, 0, 0);
+      if (__builtin_expect(m < a.M && n_ok, 1)) {
+        const long ro = (long)(a.res_rows > 0 ? m % a.res_rows : m) * a.ldr + n;
+        if (res32) {
+          const float* rp = reinterpret_cast<const float*>(a.res) + ro + 4 * half;
+          if (__builtin_expect(full, 1)) val = *reinterpret_cast<const uint4*>(rp);
+          else {
+            uint32_t w[4];
+#pragma unroll
+            for (int e = 0; e < 4; ++e) w[e] = (n + 4 * half + e < a.N) ? __float_as_uint(rp[e]) : 0u;
+            val = make_uint4(w[0], w[1], w[2], w[3]);
+          }
+        } else {
+          const uint16_t* rp = reinterpret_cast<const uint16_t*>(a.res) + ro;
+          if (__builtin_expect(full, 1)) val = *reinterpret_cast<const uint4*>(rp);
+          else {
+            uint32_t h[8];
+#pragma unroll
+            for (int e = 0; e < 8; ++e) h[e] = (n + e < a.N) ? (uint32_t)rp[e] : 0u;
+            val = make_uint4(h[0] | (h[1] << 16), h[2] | (h[3] << 16), h[4] | (h[5] << 16), h[6] | (h[7] << 16));
+          }
+        }
+      }
+      rraw[set][it] = val;
+    }
+  };
+  auto res_value = [&](int tm, int it, int e) -> float {
+    if (res32) {
+      const uint4 q = rraw[e >> 2][it];
+      const uint32_t w[4] = {q.x, q.y, q.z, q.w};
+      return __uint_as_float(w[e & 3]);
+    }
+    const uint4 q = rraw[tm & 1][it];
+    const uint32_t w[4] = {q.x, q.y, q.z, q.w};
+    const uint16_t h = (uint16_t)((e & 1) ? (w[e >> 1] >> 16) : (w[e >> 1] & 0xffff));
+    return res_dt == DT_F16 ? f16_bits_to_f32(h) : bf16_bits_to_f32(h);
+  };
+
+  if (a.res && !res32) load_res(0, 0, 0);
+  static_for<0, TM>([&](auto tmc) {
+    constexpr int tm = decltype(tmc)::value;
+    if (a.res) {
+      if (res32) { load_res(tm, 0, 0); load_res(tm, 1, 1); }
+      else if constexpr (tm + 1 < TM) load_res(tm + 1, (tm + 1) & 1, 0);
+    }
+#pragma unroll
+    for (int tn = 0; tn < TN; ++tn)
+#pragma unroll
+      for (int rq = 0; rq < 4; ++rq) {
+        const int chunk = tn * 8 + 2 * rq + g;
+        f32x4_t v4 = {acc[tn][tm][4 * rq], acc[tn][tm][4 * rq + 1], acc[tn][tm][4 * rq + 2], acc[tn][tm][4 * rq + 3]};
+        *reinterpret_cast<f32x4_t*>(sC + lr * WN + ((chunk ^ (lr & (CH4 - 1))) << 2)) = v4;
+      }
+    wave_lds_fence();
+    float v[ITERS][8];
+#pragma unroll
+    for (int it = 0; it < ITERS; ++it) {
+      const int r = er + it * RSTEP;
+      const int sw = r & (CH4 - 1);
+      const f32x4_t lo = *reinterpret_cast<const f32x4_t*>(sC + r * WN + (((2 * ec) ^ sw) << 2));
+      const f32x4_t hi = *reinterpret_cast<const f32x4_t*>(sC + r * WN + (((2 * ec + 1) ^ sw) << 2));
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        v[it][e] = fmaf(lo[e], descale, bias8[e]);
+        v[it][4 + e] = fmaf(hi[e], descale, bias8[4 + e]);
+      }
+    }
+    switch (a.act) {  // uniform
+      case ACT_GELU:
+#pragma unroll
+        for (int it = 0; it < ITERS; ++it)
+#pragma unroll
+          for (int e = 0; e < 8; ++e) v[it][e] = act_gelu(v[it][e]);
+        break;
+      case ACT_MISH:
+#pragma unroll
+        for (int it = 0; it < ITERS; ++it)
+#pragma unroll
+          for (int e = 0; e < 8; ++e) v[it][e] = act_mish(v[it][e]);
+        break;
+      case ACT_SWISH:
+#pragma unroll
+        for (int it = 0; it < ITERS; ++it)
+#pragma unroll
+          for (int e = 0; e < 8; ++e) v[it][e] = act_swish(v[it][e]);
+        break;
+      default: break;
+    }
+    if (a.res) {
+#pragma unroll
+      for (int it = 0; it < ITERS; ++it)
+#pragma unroll
+        for (int e = 0; e < 8; ++e) v[it][e] = fmaf(v[it][e], alpha, res_value(tm, it, e));
+    } else {
+#pragma unroll
+      for (int it = 0; it < ITERS; ++it)
+#pragma unroll
+        for (int e = 0; e < 8; ++e) v[it][e] *= alpha;
+    }
+    if (a.amax) {
+#pragma unroll
+      for (int it = 0; it < ITERS; ++it)
+#pragma unroll
+        for (int e = 0; e < 8; ++e)
+          if (mw0 + tm * 32 + er + it * RSTEP < a.M && n + e < a.N) local_amax = fmaxf(local_amax, fabsf(v[it][e]));
+    }
+    if constexpr (OUT_DT == DT_FP8) {
+      const float os = a.out_scale;
+#pragma unroll
+      for (int it = 0; it < ITERS; ++it)
+#pragma unroll
+        for (int e = 0; e < 8; ++e) v[it][e] *= os;
+    }
+#pragma unroll
+    for (int it = 0; it < ITERS; ++it) {
+      const int m = mw0 + tm * 32 + er + it * RSTEP;
+      if (__builtin_expect(m >= a.M || !n_ok, 0)) continue;
+      if (__builtin_expect(full, 1)) {
+        void* dst = n < a.nsplit ? a.C : a.C2;
+        const long off = n < a.nsplit ? (long)m * a.ldc + n : (long)m * a.ldc2 + (n - a.nsplit);
+        if (a.stream_out) store8<OUT_DT, 1>(dst, off, v[it]);
+        else store8<OUT_DT, 0>(dst, off, v[it]);
+      } else {
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+          if (n + e >= a.N) continue;
+          if (n + e < a.nsplit) store1<OUT_DT>(a.C, (long)m * a.ldc + n + e, v[it][e]);
+          else store1<OUT_DT>(a.C2, (long)m * a.ldc2 + (n + e - a.nsplit), v[it][e]);
+        }
+      }
+    }
+    wave_lds_fence();
+  });
+  if (a.amax) {
+    local_amax = wave_max(local_amax);
+    if (lane == 0) atomic_amax(a.amax, local_amax);
+  }
+}
+
+// The 256x256 direct-to-LDS tile (gemm_dma.hip). It lives in a translation unit, and so a device code object, of its
+// own: its speed depends measurably on where its code lands (identical instructions ran 3-8 % slower after unrelated
+// kernels were added to the same code object), and alone it stays where it was measured.
+hipError_t launch_gemm_dma(const GemmArgs& a, int in_dt, int out_dt, hipStream_t st);
+
+}  // namespace crl

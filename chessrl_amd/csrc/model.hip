@@ -392,6 +392,7 @@ struct GOpt {
   float out_scale = 1.f;
   float* amax = nullptr;
   void* C2 = nullptr; long ldc2 = 0; int nsplit = 0;
+  bool k_parallel = false;  // token steps of generation: few rows, so K is spread over more waves (different summation order)
 };
 
 int Model::gemm(const Lin& L, const void* A, long lda, int in_dt, void* C, long ldc, int out_dt, int M, const GOpt& o, hipStream_t st) {
@@ -404,7 +405,7 @@ int Model::gemm(const Lin& L, const void* A, long lda, int in_dt, void* C, long 
   g.bias = L.b; g.res = o.res; g.ldr = o.ldr; g.res_dtype = o.res_dt; g.res_rows = o.res_rows;
   g.amax = o.amax; g.M = M; g.N = L.N; g.K = L.K; g.act = o.act;
   g.descale = in_dt == DT_FP8 ? 1.f / (o.a_scale * L.wscale) : 1.f;
-  g.alpha = o.alpha; g.out_scale = o.out_scale;
+  g.alpha = o.alpha; g.out_scale = o.out_scale; g.k_parallel = o.k_parallel ? 1 : 0;
   const int fam = in_dt == DT_FP8 ? 0 : 5;
   if (profiling) prof_flops[fam] += 2.0 * M * (double)L.N * L.K;
   prof_begin(fam, st);
@@ -726,22 +727,22 @@ int Model::generate(const float* planes, int B, int steps, float temperature, ui
       STEP_RUN(lnorm(ws.x, C, xdt, ly.ln1_g, ly.ln1_b, ws.h, ad, nullptr, 1.f, C, B, C, nullptr, s));
       if (dyn) {
         // q -> ws.qkv [B,C]; k|v -> staging, then to the row the counter names
-        GOpt o; o.C2 = gen_kv_stage; o.ldc2 = 2 * C; o.nsplit = C;
+        GOpt o; o.k_parallel = true; o.C2 = gen_kv_stage; o.ldc2 = 2 * C; o.nsplit = C;
         STEP_RUN(gemm(ly.qkv, ws.h, C, ad, ws.qkv, C, ad, B, o, s));
         STEP_HIP(launch_kv_append(gen_kv_stage, kv_layers[l], B, kv_Tmax, C, 0, dyn, s));
       } else {
         // q -> ws.qkv [B,C]; k|v -> row `pos` of every sequence's cache
-        GOpt o; o.C2 = reinterpret_cast<uint16_t*>(kv_layers[l]) + (size_t)pos * 2 * C; o.ldc2 = (long)kv_Tmax * 2 * C; o.nsplit = C;
+        GOpt o; o.k_parallel = true; o.C2 = reinterpret_cast<uint16_t*>(kv_layers[l]) + (size_t)pos * 2 * C; o.ldc2 = (long)kv_Tmax * 2 * C; o.nsplit = C;
         STEP_RUN(gemm(ly.qkv, ws.h, C, ad, ws.qkv, C, ad, B, o, s));
       }
       STEP_HIP(launch_decode_attention(ws.qkv, C, kv_layers[l], kv_Tmax, C, pos + 1, dyn, ws.ao, C, B, H, hs, ad, attn_scale, s));
-      { GOpt o; o.res = ws.x; o.ldr = C; o.res_dt = xdt; STEP_RUN(gemm(ly.proj, ws.ao, C, ad, ws.x, C, xdt, B, o, s)); }
+      { GOpt o; o.k_parallel = true; o.res = ws.x; o.ldr = C; o.res_dt = xdt; STEP_RUN(gemm(ly.proj, ws.ao, C, ad, ws.x, C, xdt, B, o, s)); }
       STEP_RUN(lnorm(ws.x, C, xdt, ly.ln2_g, ly.ln2_b, ws.h, ad, nullptr, 1.f, C, B, C, nullptr, s));
-      { GOpt o; o.act = ACT_GELU; STEP_RUN(gemm(ly.ff1, ws.h, C, ad, ws.f, F, ad, B, o, s)); }
-      { GOpt o; o.res = ws.x; o.ldr = C; o.res_dt = xdt; STEP_RUN(gemm(ly.ff2, ws.f, F, ad, ws.x, C, xdt, B, o, s)); }
+      { GOpt o; o.k_parallel = true; o.act = ACT_GELU; STEP_RUN(gemm(ly.ff1, ws.h, C, ad, ws.f, F, ad, B, o, s)); }
+      { GOpt o; o.k_parallel = true; o.res = ws.x; o.ldr = C; o.res_dt = xdt; STEP_RUN(gemm(ly.ff2, ws.f, F, ad, ws.x, C, xdt, B, o, s)); }
     }
     STEP_RUN(lnorm(ws.x, C, xdt, lnf_g, lnf_b, ws.hl, hd, nullptr, 1.f, C, B, C, nullptr, s));
-    { GOpt o; STEP_RUN(gemm(lm_head, ws.hl, C, hd, gen_logits, VOCAB_RL, DT_F32, B, o, s)); }
+    { GOpt o; o.k_parallel = true; STEP_RUN(gemm(lm_head, ws.hl, C, hd, gen_logits, VOCAB_RL, DT_F32, B, o, s)); }
     if (dyn) STEP_HIP(launch_add_int(gen_k, 1, s));
     return CRL_OK;
 #undef STEP_HIP
