@@ -55,15 +55,30 @@ __device__ __forceinline__ uint8_t f32_to_fp8(float a) {
 __device__ __forceinline__ float fp8_to_f32(uint8_t b) { return __builtin_amdgcn_cvt_f32_fp8((int)b, 0); }
 
 // ---- activations ---------------------------------------------------------------
-__device__ __forceinline__ float act_gelu(float x) { return 0.5f * x * (1.0f + erff(x * 0.70710678118654752f)); }
-// mish(x) = x * tanh(softplus(x)); with n = e^x, tanh(log(1+n)) = (n^2+2n)/(n^2+2n+2).
-__device__ __forceinline__ float act_mish(float x) {
-  if (x > 20.f) return x;
-  float n = __expf(x);
-  float t = n * (n + 2.f);
-  return x * (t / (t + 2.f));
+// All three are straight-line code (no per-lane branch, hardware reciprocal instead of the IEEE division sequence):
+// they run on every element of the GEMM epilogues, where the library forms (erff with its two divergent ranges,
+// the early return of mish, precise division) cost 20-50 instructions and a branch per element.
+__device__ __forceinline__ float fast_rcp(float x) { return __builtin_amdgcn_rcpf(x); }
+// erf by Abramowitz & Stegun 7.1.26: |error| <= 1.5e-7 over the whole line.
+__device__ __forceinline__ float erf_as(float x) {
+  const float ax = fabsf(x);
+  const float t = fast_rcp(fmaf(0.3275911f, ax, 1.0f));
+  float p = fmaf(1.061405429f, t, -1.453152027f);
+  p = fmaf(p, t, 1.421413741f);
+  p = fmaf(p, t, -0.284496736f);
+  p = fmaf(p, t, 0.254829592f);
+  const float y = 1.0f - p * t * __expf(-ax * ax);
+  return copysignf(y, x);
 }
-__device__ __forceinline__ float act_swish(float x) { return x / (1.0f + __expf(-x)); }
+__device__ __forceinline__ float act_gelu(float x) { return 0.5f * x * (1.0f + erf_as(x * 0.70710678118654752f)); }
+// mish(x) = x * tanh(softplus(x)); with n = e^x, tanh(log(1+n)) = (n^2+2n)/(n^2+2n+2). Past x = 20 the ratio is 1 in
+// fp32, so the exponent is clamped there (n^2 would overflow from x = 44).
+__device__ __forceinline__ float act_mish(float x) {
+  const float n = __expf(fminf(x, 20.f));
+  const float t = n * (n + 2.f);
+  return x * (t * fast_rcp(t + 2.f));
+}
+__device__ __forceinline__ float act_swish(float x) { return x * fast_rcp(1.0f + __expf(-x)); }
 __device__ __forceinline__ float apply_act(float x, int act) {
   switch (act) {
     case ACT_GELU: return act_gelu(x);

@@ -175,18 +175,6 @@ __device__ __forceinline__ void gemm_epilogue(const GemmArgs& a, f32x16_t (&acc)
       rraw[set][it] = val;
     }
   };
-  auto res_value = [&](int tm, int it, int e) -> float {
-    if (res32) {
-      const uint4 q = rraw[e >> 2][it];
-      const uint32_t w[4] = {q.x, q.y, q.z, q.w};
-      return __uint_as_float(w[e & 3]);
-    }
-    const uint4 q = rraw[tm & 1][it];
-    const uint32_t w[4] = {q.x, q.y, q.z, q.w};
-    const uint16_t h = (uint16_t)((e & 1) ? (w[e >> 1] >> 16) : (w[e >> 1] & 0xffff));
-    return res_dt == DT_F16 ? f16_bits_to_f32(h) : bf16_bits_to_f32(h);
-  };
-
   if (a.res && !res32) load_res(0, 0, 0);
   static_for<0, TM>([&](auto tmc) {
     constexpr int tm = decltype(tmc)::value;
@@ -238,10 +226,34 @@ __device__ __forceinline__ void gemm_epilogue(const GemmArgs& a, f32x16_t (&acc)
       default: break;
     }
     if (a.res) {
+      // One straight block per residual type (the type test per element compiles to a chain of branches).
+      if (res32) {
 #pragma unroll
-      for (int it = 0; it < ITERS; ++it)
+        for (int it = 0; it < ITERS; ++it) {
+          const uint4 lo = rraw[0][it], hi = rraw[1][it];
+          const uint32_t w[8] = {lo.x, lo.y, lo.z, lo.w, hi.x, hi.y, hi.z, hi.w};
 #pragma unroll
-        for (int e = 0; e < 8; ++e) v[it][e] = fmaf(v[it][e], alpha, res_value(tm, it, e));
+          for (int e = 0; e < 8; ++e) v[it][e] = fmaf(v[it][e], alpha, __uint_as_float(w[e]));
+        }
+      } else if (res_dt == DT_F16) {
+#pragma unroll
+        for (int it = 0; it < ITERS; ++it) {
+          const uint4 q = rraw[tm & 1][it];
+          const uint32_t w[4] = {q.x, q.y, q.z, q.w};
+#pragma unroll
+          for (int e = 0; e < 8; ++e)
+            v[it][e] = fmaf(v[it][e], alpha, f16_bits_to_f32((uint16_t)((e & 1) ? (w[e >> 1] >> 16) : (w[e >> 1] & 0xffff))));
+        }
+      } else {
+#pragma unroll
+        for (int it = 0; it < ITERS; ++it) {
+          const uint4 q = rraw[tm & 1][it];
+          const uint32_t w[4] = {q.x, q.y, q.z, q.w};
+#pragma unroll
+          for (int e = 0; e < 8; ++e)
+            v[it][e] = fmaf(v[it][e], alpha, __uint_as_float((e & 1) ? (w[e >> 1] & 0xffff0000u) : (w[e >> 1] << 16)));
+        }
+      }
     } else {
 #pragma unroll
       for (int it = 0; it < ITERS; ++it)
