@@ -77,8 +77,10 @@ __device__ __forceinline__ void wave_lds_fence() {
 // NT: store with the non-temporal hint, so a streamed output does not evict the operands from L2.
 template <int OUT_DT, int NT = 0>
 __device__ __forceinline__ void store8(void* base, long off, const float v[8]) {
+  // The hint is written as an instruction: __builtin_nontemporal_store beside a plain store of the same value in the
+  // other arm of a branch is merged with it by the compiler, and the hint is dropped.
   auto put = [](i32x4_t* p, i32x4_t x) {
-    if constexpr (NT) __builtin_nontemporal_store(x, p);
+    if constexpr (NT) asm volatile("global_store_dwordx4 %0, %1, off nt" ::"v"(p), "v"(x) : "memory");
     else *p = x;
   };
   if constexpr (OUT_DT == DT_F32) {
@@ -97,7 +99,7 @@ __device__ __forceinline__ void store8(void* base, long off, const float v[8]) {
     typedef int i32x2_t __attribute__((ext_vector_type(2)));
     const i32x2_t x = {(int)pack_fp8x4(v[0], v[1], v[2], v[3]), (int)pack_fp8x4(v[4], v[5], v[6], v[7])};
     i32x2_t* p = reinterpret_cast<i32x2_t*>(reinterpret_cast<uint8_t*>(base) + off);
-    if constexpr (NT) __builtin_nontemporal_store(x, p);
+    if constexpr (NT) asm volatile("global_store_dwordx2 %0, %1, off nt" ::"v"(p), "v"(x) : "memory");
     else *p = x;
   }
 }
