@@ -141,6 +141,15 @@ __device__ __forceinline__ void gemm_epilogue(const GemmArgs& a, f32x16_t (&acc)
   const int res_dt = a.res_dtype;
   const float descale = a.descale, alpha = a.alpha;
   float local_amax = 0.f;
+  // A lane keeps its 8 columns for every row, so which output (C or C2), the column inside it and the row stride are
+  // fixed per lane: the vector paths address row m as base + m * stride.
+  constexpr int OUT_SZ = OUT_DT == DT_F32 ? 4 : OUT_DT == DT_FP8 ? 1 : 2;
+  const bool first = n < a.nsplit;
+  char* const out_base = reinterpret_cast<char*>(first ? a.C : a.C2) + (long)(first ? n : n - a.nsplit) * OUT_SZ;
+  const long out_stride = (first ? a.ldc : a.ldc2) * OUT_SZ;
+  const int res_sz = res_dt == DT_F32 ? 4 : 2;
+  const char* const res_base = reinterpret_cast<const char*>(a.res) + (long)n * res_sz;
+  const long res_stride = a.ldr * res_sz;
 
   // Raw residual bits, 16 bytes per step and set. 16-bit residuals use the two sets as a double
   // buffer over strips; an fp32 residual (8 values = 32 bytes) uses both sets for the current
@@ -153,10 +162,11 @@ __device__ __forceinline__ void gemm_epilogue(const GemmArgs& a, f32x16_t (&acc)
       const int m = mw0 + tm * 32 + er + it * RSTEP;
       uint4 val = make_uint4(0, 0, 0, 0);
       if (__builtin_expect(m < a.M && n_ok, 1)) {
-        const long ro = (long)(a.res_rows > 0 ? m % a.res_rows : m) * a.ldr + n;
+        const long rrow = a.res_rows > 0 ? m % a.res_rows : m;
+        const long ro = rrow * a.ldr + n;
         if (res32) {
           const float* rp = reinterpret_cast<const float*>(a.res) + ro + 4 * half;
-          if (__builtin_expect(full, 1)) val = *reinterpret_cast<const uint4*>(rp);
+          if (__builtin_expect(full, 1)) val = *reinterpret_cast<const uint4*>(res_base + rrow * res_stride + 16 * half);
           else {
             uint32_t w[4];
 #pragma unroll
@@ -165,7 +175,7 @@ __device__ __forceinline__ void gemm_epilogue(const GemmArgs& a, f32x16_t (&acc)
           }
         } else {
           const uint16_t* rp = reinterpret_cast<const uint16_t*>(a.res) + ro;
-          if (__builtin_expect(full, 1)) val = *reinterpret_cast<const uint4*>(rp);
+          if (__builtin_expect(full, 1)) val = *reinterpret_cast<const uint4*>(res_base + rrow * res_stride);
           else {
             uint32_t h[8];
 #pragma unroll
@@ -281,10 +291,9 @@ __device__ __forceinline__ void gemm_epilogue(const GemmArgs& a, f32x16_t (&acc)
       const int m = mw0 + tm * 32 + er + it * RSTEP;
       if (__builtin_expect(m >= a.M || !n_ok, 0)) continue;
       if (__builtin_expect(full, 1)) {
-        void* dst = n < a.nsplit ? a.C : a.C2;
-        const long off = n < a.nsplit ? (long)m * a.ldc + n : (long)m * a.ldc2 + (n - a.nsplit);
-        if (a.stream_out) store8<OUT_DT, 1>(dst, off, v[it]);
-        else store8<OUT_DT, 0>(dst, off, v[it]);
+        char* dst = out_base + m * out_stride;
+        if (a.stream_out) store8<OUT_DT, 1>(dst, 0, v[it]);
+        else store8<OUT_DT, 0>(dst, 0, v[it]);
       } else {
 #pragma unroll
         for (int e = 0; e < 8; ++e) {
