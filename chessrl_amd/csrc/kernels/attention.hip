@@ -65,9 +65,16 @@ __device__ __forceinline__ typename H::vec add_bias_h(typename H::vec q, const f
 template <int MODE>
 struct AttnWaves { static constexpr int N = MODE == ATTN_RELSHIFT ? 2 : 4; };
 
+// Waves per SIMD the register allocation is held to (0: the compiler's own choice). The kernel is a chain of load,
+// compute and store phases, so resident waves are what hides its memory latency: at head size 32 with a generated
+// bias it fits 4 waves in 122 registers without spilling (152 and 3 waves left alone; measured 10.8 -> 9.6 ms per
+// 4096-position forward; 5 waves spill and are slower). The other instances spill at that bound and keep theirs.
+template <int HS, int MODE>
+struct AttnMinWaves { static constexpr int N = (HS == 32 && MODE == ATTN_BIAS) ? 4 : 0; };
+
 // OUT_FP8: write e4m3 (value*out_scale) instead of the input element type.
 template <int HS, int MODE, int OUT_FP8, int IN_DT>
-__global__ void __launch_bounds__(64 * AttnWaves<MODE>::N) attention_kernel(const AttnArgs a) {
+__global__ void __launch_bounds__(64 * AttnWaves<MODE>::N, (AttnMinWaves<HS, MODE>::N)) attention_kernel(const AttnArgs a) {
   typedef Half16<IN_DT> H16;
   typedef typename H16::vec hvec;
   constexpr int KS = HS / 16;   // k-steps of the score product
