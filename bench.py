@@ -252,6 +252,15 @@ def main():
             res[name] = round(nf / (time.perf_counter() - t1), 1)
         pipeline = {"positions": nf, "chunk": min(B, 4096), "unit": "positions/s", "positions_per_s": res,
                     "includes": "FEN parse + encode + legal masks on host threads, PCIe both ways, forward, masked softmax"}
+        # batched 1-ply value search (new_paradigm/value.py:319-400): every legal move of every root evaluated by the value head
+        roots = fens[:512]
+        model.get_best_moves_value(roots[:32])
+        t1 = time.perf_counter()
+        _, per_root = model.get_best_moves_value(roots, T=0, return_values=True)
+        dt1 = time.perf_counter() - t1
+        children = sum(len(mv) for mv, _ in per_root)
+        pipeline["search_1ply"] = {"roots": len(roots), "child_positions": children, "roots_per_s": round(len(roots) / dt1, 1),
+                                   "child_positions_per_s": round(children / dt1, 1)}
 
     cpu = None
     if not a.no_cpu:

@@ -72,6 +72,7 @@ SIGNATURES = {
     "crl_model_set_decode_graph": (_i, [_vp, _i]),
     "crl_model_get_profile": (_i, [_vp, _vp, _vp, _vp]),
     "crl_model_evaluate_fens": (_i, [_vp, C.POINTER(C.c_char_p), _i, _i, _f, _vp, _vp, _vp, _i]),
+    "crl_model_search_1ply": (_i, [_vp, C.POINTER(C.c_char_p), _i, _i, _f, C.c_uint64, _vp, _vp, _vp, _vp, _i64, _i]),
     "crl_model_forward_tokens": (_i, [_vp, _vp, _vp, _i, _i, _vp, _vp, _vp]),
     "crl_attention_causal": (_i, [_vp, _i64, _vp, _i64, _vp, _i64, _i, _vp, _i64, _i, _f, _i, _i, _i, _i, _f, _vp, _vp]),
     "crl_token_scores": (_i, [_vp, _i64, _vp, _i64, _vp, _i, _i, _i64, _vp, _vp, _vp, _vp]),

@@ -451,18 +451,22 @@ int crl_model_generate(crl_model* m, const float* planes, int B, int steps, floa
   if (!m) return arg_fail("crl_model_generate: null model");
   return m->impl.generate(planes, B, steps, temperature, seed, rules, sequences, step_out, out_logits, (hipStream_t)stream);
 }
-int crl_model_evaluate_fens(crl_model* m, const char* const* fens, int n, int chunk, float temperature, float* probs,
-                            float* wdl, int32_t* best, int threads) {
-  if (!m || n < 0 || (n && !fens) || chunk <= 0) return arg_fail("crl_model_evaluate_fens: bad arguments");
-  if (!m->impl.finalized) { set_error("crl_model_evaluate_fens: call crl_model_finalize first"); return CRL_ERR_STATE; }
+}  // extern "C"
+
+// The chunked host -> device -> host pipeline behind crl_model_evaluate_fens and crl_model_search_1ply: position i of
+// the job is produced by get(i, board) on the host threads. The legal-move masks and the masked softmax are skipped
+// when neither probabilities nor best moves are asked for (value-only evaluation).
+template <typename GetBoard>
+static int evaluate_boards(crl_model* m, int n, int chunk, float temperature, float* probs, float* wdl, int32_t* best, int threads,
+                           GetBoard get) {
   const int V = m->impl.vocab;
   const bool leela = m->impl.cfg.arch == CRL_ARCH_BT4CLASS, has_wdl = m->impl.cfg.arch != CRL_ARCH_GPT64;
-  if (wdl && !has_wdl) return arg_fail("crl_model_evaluate_fens: this architecture has no value head");
+  const bool need_policy = probs || best;
   if (n == 0) return CRL_OK;
   if (chunk > n) chunk = n;
   FenPipeline& P = m->pipe;
   hipError_t e = P.ensure(chunk, V);
-  if (e != hipSuccess) return hip_fail("crl_model_evaluate_fens: staging buffers", e);
+  if (e != hipSuccess) return hip_fail("evaluate: staging buffers", e);
   // Results of a finished slot go from pinned staging to the caller's arrays.
   auto drain = [&](FenPipeline::Slot& s) -> hipError_t {
     if (s.count == 0) return hipSuccess;
@@ -479,33 +483,36 @@ int crl_model_evaluate_fens(crl_model* m, const char* const* fens, int n, int ch
   for (int first = 0; first < n && rc == CRL_OK; first += chunk, ++k) {
     FenPipeline::Slot& s = P.slot[k & 1];
     e = drain(s);  // the chunk that used this slot two steps ago
-    if (e != hipSuccess) { rc = hip_fail("crl_model_evaluate_fens: wait", e); break; }
+    if (e != hipSuccess) { rc = hip_fail("evaluate: wait", e); break; }
     const int cnt = std::min(chunk, n - first);
     // Host work of this chunk overlaps the device work of the previous one.
     rc = parallel_for(cnt, threads, [&](int i) {
       Board b;
-      int prc = parse(fens[first + i], b);
+      int prc = get(first + i, b);
       if (prc) return prc;
       b.compact(s.h_ids + (size_t)i * 64, s.h_flags + (size_t)i * 4);
+      if (!need_policy) return 0;
       if (leela) legal_mask_leela(b, s.h_mask + (size_t)i * V);
       else legal_mask_rl(b, s.h_mask + (size_t)i * V);
       return 0;
     });
     if (rc) break;
-#define PIPE_HIP(call) do { e = (call); if (e != hipSuccess) { rc = hip_fail("crl_model_evaluate_fens", e); } } while (0)
+#define PIPE_HIP(call) do { e = (call); if (e != hipSuccess) { rc = hip_fail("evaluate", e); } } while (0)
     PIPE_HIP(hipMemcpyAsync(s.d_ids, s.h_ids, (size_t)cnt * 64, hipMemcpyHostToDevice, P.copy_st));
     if (rc == CRL_OK) PIPE_HIP(hipMemcpyAsync(s.d_flags, s.h_flags, (size_t)cnt * 4, hipMemcpyHostToDevice, P.copy_st));
-    if (rc == CRL_OK) PIPE_HIP(hipMemcpyAsync(s.d_mask, s.h_mask, (size_t)cnt * V, hipMemcpyHostToDevice, P.copy_st));
+    if (rc == CRL_OK && need_policy) PIPE_HIP(hipMemcpyAsync(s.d_mask, s.h_mask, (size_t)cnt * V, hipMemcpyHostToDevice, P.copy_st));
     if (rc == CRL_OK) PIPE_HIP(hipEventRecord(s.uploaded, P.copy_st));
     if (rc == CRL_OK) PIPE_HIP(hipStreamWaitEvent(P.comp_st, s.uploaded, 0));
     if (rc) break;
     rc = m->impl.forward(nullptr, s.d_ids, s.d_flags, cnt, s.d_logits, has_wdl ? s.d_wdl : nullptr, false, P.comp_st);
     if (rc) break;
-    SoftmaxArgs a;
-    std::memset(&a, 0, sizeof(a));
-    a.logits = s.d_logits; a.ldl = V; a.mask = s.d_mask; a.ldm = V; a.probs = probs ? s.d_probs : nullptr; a.ldp = V;
-    a.argmax = s.d_best; a.B = cnt; a.V = V; a.temperature = temperature;
-    PIPE_HIP(launch_masked_softmax(a, P.comp_st));
+    if (need_policy) {
+      SoftmaxArgs a;
+      std::memset(&a, 0, sizeof(a));
+      a.logits = s.d_logits; a.ldl = V; a.mask = s.d_mask; a.ldm = V; a.probs = probs ? s.d_probs : nullptr; a.ldp = V;
+      a.argmax = s.d_best; a.B = cnt; a.V = V; a.temperature = temperature;
+      PIPE_HIP(launch_masked_softmax(a, P.comp_st));
+    }
     if (rc == CRL_OK && probs) PIPE_HIP(hipMemcpyAsync(s.h_probs, s.d_probs, sizeof(float) * (size_t)cnt * V, hipMemcpyDeviceToHost, P.comp_st));
     if (rc == CRL_OK && wdl) PIPE_HIP(hipMemcpyAsync(s.h_wdl, s.d_wdl, sizeof(float) * (size_t)cnt * 3, hipMemcpyDeviceToHost, P.comp_st));
     if (rc == CRL_OK && best) PIPE_HIP(hipMemcpyAsync(s.h_best, s.d_best, sizeof(int32_t) * (size_t)cnt, hipMemcpyDeviceToHost, P.comp_st));
@@ -518,7 +525,7 @@ int crl_model_evaluate_fens(crl_model* m, const char* const* fens, int n, int ch
   for (FenPipeline::Slot& s : P.slot) {
     if (rc == CRL_OK) {
       e = drain(s);
-      if (e != hipSuccess) rc = hip_fail("crl_model_evaluate_fens: wait", e);
+      if (e != hipSuccess) rc = hip_fail("evaluate: wait", e);
     } else {
       s.count = 0;
     }
@@ -529,6 +536,88 @@ int crl_model_evaluate_fens(crl_model* m, const char* const* fens, int n, int ch
     if (!err.empty()) set_error(err);
   }
   return rc;
+}
+extern "C" {
+
+int crl_model_evaluate_fens(crl_model* m, const char* const* fens, int n, int chunk, float temperature, float* probs,
+                            float* wdl, int32_t* best, int threads) {
+  if (!m || n < 0 || (n && !fens) || chunk <= 0) return arg_fail("crl_model_evaluate_fens: bad arguments");
+  if (!m->impl.finalized) { set_error("crl_model_evaluate_fens: call crl_model_finalize first"); return CRL_ERR_STATE; }
+  if (wdl && m->impl.cfg.arch == CRL_ARCH_GPT64) return arg_fail("crl_model_evaluate_fens: this architecture has no value head");
+  return evaluate_boards(m, n, chunk, temperature, probs, wdl, best, threads, [&](int i, Board& b) { return parse(fens[i], b); });
+}
+
+int crl_model_search_1ply(crl_model* m, const char* const* fens, int n, int chunk, float temperature, uint64_t seed, char* best_uci6,
+                          int32_t* n_moves, char* moves_uci6, float* values, int64_t capacity, int threads) {
+  if (!m || n < 0 || (n && !fens) || chunk <= 0 || temperature < 0.f || capacity < 0)
+    return arg_fail("crl_model_search_1ply: bad arguments");
+  if (!m->impl.finalized) { set_error("crl_model_search_1ply: call crl_model_finalize first"); return CRL_ERR_STATE; }
+  if (m->impl.cfg.arch == CRL_ARCH_GPT64) return arg_fail("crl_model_search_1ply: this architecture has no value head");
+  // Roots -> children on the host threads.
+  std::vector<Board> roots(n);
+  std::vector<std::vector<Move>> moves(n);
+  int rc = parallel_for(n, threads, [&](int i) {
+    int prc = parse(fens[i], roots[i]);
+    if (prc) return prc;
+    roots[i].legal(moves[i]);
+    return 0;
+  });
+  if (rc) return rc;
+  std::vector<int64_t> first(n + 1, 0);
+  for (int i = 0; i < n; ++i) first[i + 1] = first[i] + (int64_t)moves[i].size();
+  const int64_t total = first[n];
+  if ((moves_uci6 || values) && total > capacity) {
+    set_error("crl_model_search_1ply: " + std::to_string(total) + " child positions, room for " + std::to_string(capacity));
+    return CRL_ERR_ARG;
+  }
+  if (total > INT32_MAX) return arg_fail("crl_model_search_1ply: too many child positions for one call");
+  std::vector<int32_t> root_of((size_t)total);
+  for (int i = 0; i < n; ++i)
+    for (int64_t c = first[i]; c < first[i + 1]; ++c) root_of[(size_t)c] = i;
+  std::vector<float> wdl((size_t)total * 3);
+  rc = evaluate_boards(m, (int)total, chunk, 1.0f, nullptr, wdl.data(), nullptr, threads, [&](int c, Board& b) {
+    // board.push(move); board.fen() and back (value.py:336-340, 288): the en-passant square survives only where a
+    // capture is legal, which is what the planes of the child position are then built from.
+    const int i = root_of[(size_t)c];
+    Board child = roots[i];
+    child.make(moves[i][(size_t)(c - first[i])]);
+    return parse(child.fen(true).c_str(), b);
+  });
+  if (rc) return rc;
+  // Per root: value of each child for the side to move at the root, then the pick (value.py:343-352, 372-395).
+  for (int i = 0; i < n; ++i) {
+    const int nm = (int)moves[i].size();
+    if (n_moves) n_moves[i] = nm;
+    if (best_uci6) std::memset(best_uci6 + (size_t)i * 6, 0, 6);
+    if (nm == 0) continue;
+    std::vector<float> val((size_t)nm);
+    for (int c = 0; c < nm; ++c) {
+      const float* w = wdl.data() + (size_t)(first[i] + c) * 3;
+      const float mx = std::max(w[0], std::max(w[1], w[2]));
+      const float e0 = std::exp(w[0] - mx), e1 = std::exp(w[1] - mx), e2 = std::exp(w[2] - mx);
+      const float inv = 1.0f / (e0 + e1 + e2);
+      val[(size_t)c] = 0.5f * e1 * inv + (roots[i].white_to_move ? e2 : e0) * inv;
+      if (values) values[first[i] + c] = val[(size_t)c];
+      if (moves_uci6) put_str(moves_uci6 + (size_t)(first[i] + c) * 6, 6, move_uci(moves[i][(size_t)c]));
+    }
+    int pick = 0;
+    for (int c = 1; c < nm; ++c)
+      if (val[(size_t)c] > val[(size_t)pick]) pick = c;
+    if (temperature > 0.f) {
+      // one draw from softmax(values / T): inverse CDF with a generator keyed by (seed, root)
+      double sum = 0.0;
+      std::vector<double> p((size_t)nm);
+      for (int c = 0; c < nm; ++c) { p[(size_t)c] = std::exp((double)(val[(size_t)c] - val[(size_t)pick]) / temperature); sum += p[(size_t)c]; }
+      SplitMix64 rng(seed ^ (0x9E3779B97F4A7C15ull * (uint64_t)(i + 1)));
+      const double u = (double)(rng.next() >> 11) * (1.0 / 9007199254740992.0) * sum;
+      double acc = 0.0;
+      int drawn = nm - 1;
+      for (int c = 0; c < nm; ++c) { acc += p[(size_t)c]; if (u < acc) { drawn = c; break; } }
+      pick = drawn;
+    }
+    if (best_uci6) put_str(best_uci6 + (size_t)i * 6, 6, move_uci(moves[i][(size_t)pick]));
+  }
+  return CRL_OK;
 }
 int crl_model_vocab(const crl_model* m) { return m ? m->impl.vocab : 0; }
 double crl_model_flops_per_position(const crl_model* m) { return m ? m->impl.flops_per_position() : 0.0; }

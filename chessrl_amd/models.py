@@ -288,6 +288,29 @@ class _Engine:
               "crl_model_evaluate_fens")
         return probs, wdl, best
 
+    def search_1ply(self, fens, T=0.0, seed=0, chunk=4096, want_values=False, threads=0):
+        """Batched 1-ply value search: (best move per root, and with want_values the per-root (moves, values) lists)."""
+        if not self.ready:
+            self.finalize()
+        n = len(fens)
+        arr = _lib.str_array(fens)
+        best = C.create_string_buffer(max(n, 1) * 6)
+        counts = (C.c_int32 * max(n, 1))()
+        cap = 256 * n if want_values else 0
+        mv = C.create_string_buffer(max(cap, 1) * 6) if want_values else None
+        vals = torch.empty((max(cap, 1),), dtype=torch.float32) if want_values else None
+        check(lib().crl_model_search_1ply(self.handle, arr, n, int(chunk), float(T), int(seed) & (2 ** 64 - 1), best, counts,
+                                          mv, _ptr(vals), cap, int(threads)), "crl_model_search_1ply")
+        moves = [best.raw[6 * i:6 * i + 6].split(b"\0")[0].decode() for i in range(n)]
+        if not want_values:
+            return moves
+        per_root, o = [], 0
+        for i in range(n):
+            k = counts[i]
+            per_root.append(([mv.raw[6 * (o + c):6 * (o + c) + 6].split(b"\0")[0].decode() for c in range(k)], vals[o:o + k].clone()))
+            o += k
+        return moves, per_root
+
     def flops_per_position(self):
         return lib().crl_model_flops_per_position(self.handle)
 
@@ -389,6 +412,13 @@ class _ModelBase:
         legal masks, upload (overlapped with the device work of the previous chunk), masked softmax, download.
         Returns CPU tensors (probs [n,V] or None, wdl logits [n,3] or None, best legal move index [n])."""
         return self._engine.evaluate_fens(list(fens), T, chunk, want_probs, want_wdl)
+
+    @torch.no_grad()
+    def get_best_moves_value(self, fens, T=0.0, seed=0, return_values=False):
+        """get_best_move_value (new_paradigm/value.py:356-400) for a list of positions in one call: every child of
+        every root goes through the library's chunked pipeline. Returns the chosen move per root ('' where a root has
+        no legal move) and, with return_values, per root (moves, value of each move for the side to move)."""
+        return self._engine.search_1ply(list(fens), T=T, seed=seed, want_values=return_values)
 
     def graphed_evaluator(self, batch, T=1.0, device="cuda"):
         """Leaf evaluation for a fixed batch size captured in a HIP graph (launch-bound small batches)."""

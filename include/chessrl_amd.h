@@ -211,6 +211,17 @@ int crl_model_set_decode_graph(crl_model* m, int on);
  * per model; the staging buffers (2 chunks, pinned + device) stay with the model until it is destroyed. */
 int crl_model_evaluate_fens(crl_model* m, const char* const* fens, int n, int chunk, float temperature, float* probs,
                             float* wdl, int32_t* best, int threads);
+/* Batched 1-ply value search: BT4.calculate_move_values / get_best_move_value (new_paradigm/value.py:319-400) for n root
+ * positions at once. Every legal move of every root is made on the host, all child positions go through the same
+ * chunked pipeline as crl_model_evaluate_fens (value head only: no masks, no policy download), and per root the value
+ * of a child for the side to move at the root is 0.5*P(draw) + P(win for that side) with P = softmax of the child's
+ * [black win, draw, white win] logits (:343-352). best_uci6 [n,6] receives the move with the largest value
+ * (temperature 0) or one draw from softmax(values/temperature) (:384-394; inverse CDF with a generator keyed by seed and
+ * root index, not torch's stream); a root without legal moves gets an empty string (the reference raises there).
+ * Optional: n_moves [n]; moves_uci6 [total,6] and values [total], the children of root i at
+ * sum(n_moves[0..i)) onwards in move-generation order, total <= capacity or the call fails. Not for CRL_ARCH_GPT64. */
+int crl_model_search_1ply(crl_model* m, const char* const* fens, int n, int chunk, float temperature, uint64_t seed,
+                          char* best_uci6, int32_t* n_moves, char* moves_uci6, float* values, int64_t capacity, int threads);
 int crl_model_vocab(const crl_model* m);
 /* 2*MAC count of one position through this model (for roofline accounting). */
 double crl_model_flops_per_position(const crl_model* m);

@@ -252,6 +252,58 @@ def test_evaluate_fens_pipeline_equals_direct(cuda, arch):
     assert m.evaluate_fens([], chunk=4)[2].numel() == 0
 
 
+def test_search_1ply_batched(cuda):
+    """crl_model_search_1ply (calculate_move_values / get_best_move_value of new_paradigm/value.py:319-400 for many
+    roots at once): the same moves, values and arg-max move as the per-position path; values against the fp32 oracle
+    evaluated on the child positions; roots without legal moves; reproducible draws; the capacity check."""
+    oracle = om.test_init_(om.BT4Oracle(2, 256, 368, 4), seed=3)
+    m = models.BT4(2, 256, 368, 4)
+    m.load_state_dict(oracle.state_dict())
+    fens = list(board.random_positions(21, 40, fens=True)["fens"])
+    fens += ["7k/P7/8/8/8/8/8/K7 w - - 0 1",                      # promotions among the children
+             "R6k/6pp/8/8/8/8/8/K7 b - - 0 1",                    # checkmated: no legal move
+             "7k/5Q2/6K1/8/8/8/8/8 b - - 0 1",                    # stalemate: no legal move
+             "r1bq1rk1/2pp1ppp/p1n2n2/2b1p3/1pP1P3/1B1P1N2/PP3PPP/RNBQR1K1 b - c3 0 9"]
+    best, per_root = m.get_best_moves_value(fens, T=0, return_values=True)
+    assert len(best) == len(fens) and len(per_root) == len(fens)
+    worst = 0.0
+    for fen, bm, (moves, vals) in zip(fens, best, per_root):
+        ref_moves, ref_vals = m.calculate_move_values(fen)
+        assert moves == list(ref_moves)
+        if not moves:
+            assert bm == "" and vals.numel() == 0
+            continue
+        assert torch.allclose(vals, ref_vals.cpu(), rtol=0, atol=2e-6)
+        assert bm == moves[int(torch.argmax(vals))]
+        # the oracle on the same children (value.py:343-352)
+        _, child = board.child_fens(fen)
+        _, wdl = oracle.forward_pv(board.encode_fens(child))
+        pr = wdl.softmax(-1)
+        want = 0.5 * pr[:, 1] + (pr[:, 2] if board.white_to_move(fen) else pr[:, 0])
+        worst = max(worst, (vals - want).abs().max().item())
+    print("1-ply search: largest |value - oracle| %.2e" % worst)
+    assert worst < 1e-2
+    assert best[-3] == "" and best[-2] == ""
+    # one call without the value arrays, chunked so that several chunks are in flight
+    assert m._engine.search_1ply(fens, T=0.0, chunk=64) == best
+    # draws: legal, reproducible, seed-dependent
+    d1 = m.get_best_moves_value(fens, T=1.0, seed=5)
+    d2 = m.get_best_moves_value(fens, T=1.0, seed=5)
+    d3 = m.get_best_moves_value(fens, T=1.0, seed=6)
+    assert d1 == d2 and d1 != d3
+    for mv, (moves, _) in zip(d1, per_root):
+        assert (mv in moves) if moves else mv == ""
+    # too little room for the per-child arrays is an error, not an overflow
+    import ctypes as C
+    from chessrl_amd import _lib
+    arr = _lib.str_array(fens[:3])
+    vals = torch.empty(4)
+    assert _lib.lib().crl_model_search_1ply(m._engine.handle, arr, 3, 64, 0.0, 0, None, None, None, C.c_void_p(vals.data_ptr()), 4, 0) < 0
+    gpt = models.GPT(models.GPTConfig(block_size=256, vocab_size=1929, n_layer=1, n_head=8, n_embd=256))
+    with pytest.raises(_lib.CrlError):
+        gpt.get_best_moves_value(fens[:2])
+
+
 @pytest.mark.parametrize("t", [1, 37, 192])
 def test_gpt_forward_with_move_tokens(cuda, t):
     """GPT.forward((planes, idx), compute_loss) of model_bis.py:171-199: 64 board tokens followed by t move tokens,
