@@ -254,7 +254,7 @@ def main():
                     "includes": "FEN parse + encode + legal masks on host threads, PCIe both ways, forward, masked softmax"}
         # batched 1-ply value search (new_paradigm/value.py:319-400): every legal move of every root evaluated by the value head
         roots = fens[:512]
-        model.get_best_moves_value(roots[:32])
+        model.get_best_moves_value(roots[:160])   # more than one chunk of children: the staging buffers reach full size
         t1 = time.perf_counter()
         _, per_root = model.get_best_moves_value(roots, T=0, return_values=True)
         dt1 = time.perf_counter() - t1
