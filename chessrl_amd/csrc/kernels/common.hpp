@@ -127,6 +127,8 @@ struct GemmArgs {
   int stream_out;     // 1: the output is far larger than the L2 caches: store it with the non-temporal hint
   int k_slices;       // >1: workgroup (tile, slice) covers slabs_per_slice 128-byte slabs of K and writes slice `slice` of C [k_slices, M, ldc]
   int slabs_per_slice;
+  float* splitk_ws;   // workspace of the K-sliced path owned by the caller (else the library's per-stream one), splitk_ws_bytes long
+  long splitk_ws_bytes;
   int k_parallel;     // 1: tile 0 may pick the K-sliced / K-grouped kernels, whose summation order over K differs from the tiled kernels'
 };
 
@@ -256,9 +258,6 @@ struct ScatterArgs {
 // how many other rows the call has; 4 and 5 are picked by tile 0 only when a.k_parallel is set (few tiles, where they
 // are faster).
 hipError_t launch_gemm(GemmArgs a, int in_dt, int out_dt, int tile, hipStream_t st);
-// Allocates the stream's workspace for K-sliced GEMMs now (it is otherwise allocated by the first launch that needs
-// it, which must not happen while the stream is being recorded into a graph).
-hipError_t gemm_prepare_stream(hipStream_t st);
 hipError_t launch_layernorm(const LayerNormArgs& a, hipStream_t st);
 hipError_t launch_embed(const EmbedArgs& a, hipStream_t st);
 hipError_t launch_token_embed(const TokenEmbedArgs& a, hipStream_t st);

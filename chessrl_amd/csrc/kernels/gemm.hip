@@ -343,7 +343,7 @@ static hipError_t launch_cfg(const GemmArgs& a, hipStream_t st) {
 
 // Workspace of the K-sliced GEMMs: one per (device, stream a launch is issued or recorded on), so launches that may
 // run at the same time never share one. Lives until the process ends.
-constexpr size_t SPLITK_WS_BYTES = 16u << 20;
+constexpr size_t SPLITK_WS_BYTES = 64u << 20;
 static std::mutex g_ws_mutex;
 static std::unordered_map<uint64_t, float*> g_ws;
 static hipError_t workspace_for(hipStream_t st, float** out) {
@@ -361,10 +361,6 @@ static hipError_t workspace_for(hipStream_t st, float** out) {
   *out = p;
   return hipSuccess;
 }
-hipError_t gemm_prepare_stream(hipStream_t st) {
-  float* p = nullptr;
-  return workspace_for(st, &p);
-}
 
 // Few output tiles and a long K leave most CUs idle while a few walk K alone (M=128, N=768, K=3072: 24 workgroups
 // of 48 slabs each). Then K is cut into slices, one workgroup per (tile, slice) writes its raw sums, and a second
@@ -378,21 +374,38 @@ static int splitk_plan(const GemmArgs& a, int esz, bool forced, int* slabs_per_s
   const int per = (nslab + ks - 1) / ks;
   ks = (nslab + per - 1) / per;
   const long ldp = (a.N + 7) / 8 * 8;
-  if (ks < 2 || (size_t)ks * a.M * ldp * sizeof(float) > SPLITK_WS_BYTES) return 1;
+  if (ks < 2 || (size_t)ks * a.M * ldp * sizeof(float) > (a.splitk_ws ? (size_t)a.splitk_ws_bytes : SPLITK_WS_BYTES)) return 1;
+  *slabs_per_slice = per;
+  return ks;
+}
+
+// The same idea for the forward pass, where a row's result must not depend on how many rows the call has: narrow
+// outputs with a long K (the value head's 8192 -> 128 layer, the bias generator's 2048 -> 256 layer, both on one row
+// per position) are always cut into the same slices, a function of N and K alone, whenever the 64x64 tile is the
+// choice (fewer than 256 tiles of 128x128, i.e. under 16384 rows at these widths; the workspace holds that case).
+// At 64 rows the 8192 -> 128 layer otherwise runs on two workgroups for 98 us.
+static int splitk_plan_fixed(const GemmArgs& a, int esz, int* slabs_per_slice) {
+  const int nslab = (int)(((long)a.K * esz + 127) >> 7);
+  if (a.N > 256 || nslab < 32) return 1;
+  int ks = std::min(nslab / 16, 4);
+  const int per = (nslab + ks - 1) / ks;
+  ks = (nslab + per - 1) / per;
+  const long ldp = (a.N + 7) / 8 * 8;
+  if (ks < 2 || (size_t)ks * a.M * ldp * sizeof(float) > (a.splitk_ws ? (size_t)a.splitk_ws_bytes : SPLITK_WS_BYTES)) return 1;
   *slabs_per_slice = per;
   return ks;
 }
 
 template <int IN_DT, int OUT_DT>
 static hipError_t launch_splitk(const GemmArgs& a, int ks, int per, hipStream_t st) {
-  float* ws = nullptr;
-  hipError_t e = workspace_for(st, &ws);
+  float* ws = a.splitk_ws;
+  hipError_t e = ws ? hipSuccess : workspace_for(st, &ws);
   if (e != hipSuccess) return e;
   const long ldp = (a.N + 7) / 8 * 8;
   GemmArgs b = a;
   b.C = b.C2 = ws; b.ldc = b.ldc2 = ldp; b.nsplit = a.N;
   b.bias = nullptr; b.res = nullptr; b.amax = nullptr; b.act = ACT_NONE; b.descale = 1.f; b.alpha = 1.f; b.out_scale = 1.f;
-  b.vec_ok = 1; b.stream_out = 0; b.k_slices = ks; b.slabs_per_slice = per;
+  b.vec_ok = 1; b.stream_out = 0; b.k_slices = ks; b.slabs_per_slice = per; b.splitk_ws = nullptr;
   static bool attr_set[16] = {};
   int dev = 0;
   (void)hipGetDevice(&dev);
@@ -430,6 +443,11 @@ static hipError_t launch_in_out(const GemmArgs& a, int tile, hipStream_t st) {
     const long small = (long)((a.M + 63) / 64) * ((a.N + 63) / 64);
     const long nslab = ((long)a.K * (IN_DT == DT_FP8 ? 1 : 2) + 127) >> 7;
     if (tile == 1 && a.k_parallel && small <= 512 && nslab >= 8) tile = 5;
+    if (tile == 1 && !a.k_parallel) {
+      int per = 0;
+      const int ks = splitk_plan_fixed(a, IN_DT == DT_FP8 ? 1 : 2, &per);
+      if (ks > 1) return launch_splitk<IN_DT, OUT_DT>(a, ks, per, st);
+    }
   }
   if (tile == 3) return launch_gemm_dma(a, IN_DT, OUT_DT, st);
   if (tile == 2) return launch_cfg<CfgMid, IN_DT, OUT_DT>(a, st);

@@ -330,6 +330,7 @@ int Model::ensure_ws(int mb) {
   WS(ws.f, M * F * 2);
   WS(ws.f8, M * F);
   WS(ws.stm, (size_t)mb);
+  WS(ws.splitk, (size_t)Workspace::SPLITK_BYTES);
   if (cfg.arch == CRL_ARCH_BT4CLASS) {
     WS(ws.comp, M * cfg.smolgen_compress * 2);
     WS(ws.sh1, (size_t)mb * cfg.smolgen_hidden * 2);
@@ -406,6 +407,7 @@ int Model::gemm(const Lin& L, const void* A, long lda, int in_dt, void* C, long 
   g.amax = o.amax; g.M = M; g.N = L.N; g.K = L.K; g.act = o.act;
   g.descale = in_dt == DT_FP8 ? 1.f / (o.a_scale * L.wscale) : 1.f;
   g.alpha = o.alpha; g.out_scale = o.out_scale; g.k_parallel = o.k_parallel ? 1 : 0;
+  g.splitk_ws = ws.splitk; g.splitk_ws_bytes = Workspace::SPLITK_BYTES;
   const int fam = in_dt == DT_FP8 ? 0 : 5;
   if (profiling) prof_flops[fam] += 2.0 * M * (double)L.N * L.K;
   prof_begin(fam, st);
@@ -757,7 +759,6 @@ int Model::generate(const float* planes, int B, int steps, float temperature, ui
   if (graphed) {
     RUN(token_step(1, nullptr, false, st));
     if (!cap_stream) HIPCHK(hipStreamCreateWithFlags(&cap_stream, hipStreamNonBlocking));
-    HIPCHK(gemm_prepare_stream(cap_stream));
     hipGraph_t graph = nullptr;
     hipGraphExec_t exec = nullptr;
     hipError_t he = hipStreamBeginCapture(cap_stream, hipStreamCaptureModeRelaxed);

@@ -38,6 +38,8 @@ struct Workspace {
   void *comp = nullptr, *sh1 = nullptr, *sh2 = nullptr, *sg1 = nullptr, *sg2 = nullptr, *bias = nullptr;
   uint8_t* sg2_8 = nullptr;
   void *hl = nullptr, *tok = nullptr, *pqk = nullptr, *v1 = nullptr, *v2 = nullptr, *dense = nullptr;
+  float* splitk = nullptr;    // partial tiles of the K-sliced GEMMs (SPLITK_BYTES)
+  static constexpr long SPLITK_BYTES = 64L << 20;
 };
 
 struct GOpt;

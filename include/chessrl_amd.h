@@ -100,7 +100,7 @@ int crl_random_positions(uint64_t seed, int n, int max_plies, double late_fracti
  * accumulates max|value|. tile: 0 = automatic among 1-3 = the 64x64 / 128x128 / 256x256 workgroup tile; these add up
  * K in one order, so a row's result does not depend on the other rows of the call. For few rows (the token steps of
  * crl_model_generate use them): 4 = 64x64 tiles with K cut into slices, one workgroup per (tile, slice) leaving raw
- * fp32 sums in a workspace of 16 MB that the library keeps per stream, and a second kernel that adds them in slice
+ * fp32 sums in a workspace of 64 MB that the library keeps per stream, and a second kernel that adds them in slice
  * order and applies the epilogue; 5 = 64x64 tiles whose K slabs four groups of four waves take in turn and add up in
  * LDS. Both are deterministic from launch to launch but differ from 1-3 in summation order. */
 int crl_gemm(const void* A, int64_t lda, const void* W, int64_t ldw, void* C, int64_t ldc,

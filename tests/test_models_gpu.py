@@ -126,6 +126,25 @@ def test_bt4class_16bit(cuda, cfg, act):
     assert top1_agreement(pol, rpol, mask) >= 0.98
 
 
+@pytest.mark.parametrize("fp8", [False, True])
+def test_bt4class_batch_invariance(cuda, fp8):
+    """A position's policy and WDL are bit-equal whatever batch it travels in: alone, in 64, in 700 (two GEMM tile
+    regimes, and the narrow long-K layers of the value head and the bias generator, whose K slices are a function of
+    the layer alone), and in any order."""
+    m = models.BT4Class(3, 512, 768, 16, fp8=fp8)
+    planes, _ = positions(700, seed=12, leela=True)
+    x = planes.to(cuda)
+    if fp8:
+        m.calibrate(x[:128])
+    pol, wdl = m(x)
+    for sl in (slice(5, 6), slice(0, 64), slice(100, 357)):
+        p2, w2 = m(x[sl].contiguous())
+        assert torch.equal(p2, pol[sl]) and torch.equal(w2, wdl[sl])
+    perm = torch.randperm(700, generator=torch.Generator().manual_seed(1))
+    p3, w3 = m(x[perm.to(cuda)].contiguous())
+    assert torch.equal(p3.cpu(), pol.cpu()[perm]) and torch.equal(w3.cpu(), wdl.cpu()[perm])
+
+
 @pytest.mark.parametrize("act", ["bf16", "f16"])
 def test_bt4class_full_size(cuda, act):
     """The benchmark model at its real size (15 layers, d=1024, 32 heads, FFN 1536) and its benchmark
