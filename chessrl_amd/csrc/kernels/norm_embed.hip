@@ -127,6 +127,67 @@ __global__ void __launch_bounds__(256) layernorm_kernel(const LayerNormArgs a) {
   }
 }
 
+// Rows longer than 2048 elements (the 8192-wide norm of the bias generator): the four waves of a workgroup share one
+// row, 8 elements per thread and step of 2048, and meet through LDS for the two reductions (wave sums added in wave
+// order). Chosen by the row length alone, so a row's result does not depend on how many rows the call has; with one
+// row per position it also puts four times as many waves on a small batch as one wave per row would.
+template <int IN_DT>
+__global__ void __launch_bounds__(256) layernorm_wide_kernel(const LayerNormArgs a) {
+  constexpr int VPT = 4;
+  __shared__ float s_red[2][4];
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const long row = blockIdx.x;
+  float x[VPT][8];
+  float s = 0.f;
+#pragma unroll
+  for (int i = 0; i < VPT; ++i) {
+    const int col = (i * 256 + tid) * 8;
+    if (col < a.C) {
+      load8<IN_DT>(a.x, row * a.ldx + col, x[i]);
+#pragma unroll
+      for (int e = 0; e < 8; ++e) s += x[i][e];
+    }
+  }
+  s = wave_sum(s);
+  if (lane == 0) s_red[0][wave] = s;
+  __syncthreads();
+  const float mean = (((s_red[0][0] + s_red[0][1]) + s_red[0][2]) + s_red[0][3]) / (float)a.C;
+  float q = 0.f;
+#pragma unroll
+  for (int i = 0; i < VPT; ++i) {
+    if ((i * 256 + tid) * 8 < a.C) {
+#pragma unroll
+      for (int e = 0; e < 8; ++e) { const float d = x[i][e] - mean; q += d * d; }
+    }
+  }
+  q = wave_sum(q);
+  if (lane == 0) s_red[1][wave] = q;
+  __syncthreads();
+  const float rstd = rsqrtf((((s_red[1][0] + s_red[1][1]) + s_red[1][2]) + s_red[1][3]) / (float)a.C + a.eps);
+  float am = 0.f;
+#pragma unroll
+  for (int i = 0; i < VPT; ++i) {
+    const int col = (i * 256 + tid) * 8;
+    if (col < a.C) {
+      float gv[8], bv[8], y[8];
+      load8<DT_F32>(a.gamma, col, gv);
+      if (a.beta) load8<DT_F32>(a.beta, col, bv);
+#pragma unroll
+      for (int e = 0; e < 8; ++e) y[e] = (x[i][e] - mean) * rstd * gv[e] + (a.beta ? bv[e] : 0.f);
+      if (a.out) store8(a.out, row * a.ldo + col, y, a.out_dtype);
+      if (a.out_fp8) store8_fp8(a.out_fp8, row * a.ldo + col, y, a.fp8_scale);
+      if (a.amax) {
+#pragma unroll
+        for (int e = 0; e < 8; ++e) am = fmaxf(am, fabsf(y[e]));
+      }
+    }
+  }
+  if (a.amax) {
+    am = wave_max(am);
+    if (lane == 0) atomic_amax(a.amax, am);
+  }
+}
+
 template <int IN_DT>
 static hipError_t launch_ln_dt(const LayerNormArgs& a, hipStream_t st) {
   const dim3 grid((a.rows + 3) / 4), block(256);
@@ -134,7 +195,7 @@ static hipError_t launch_ln_dt(const LayerNormArgs& a, hipStream_t st) {
   if (vecs <= 1) hipLaunchKernelGGL((layernorm_kernel<IN_DT, 1>), grid, block, 0, st, a);
   else if (vecs <= 2) hipLaunchKernelGGL((layernorm_kernel<IN_DT, 2>), grid, block, 0, st, a);
   else if (vecs <= 4) hipLaunchKernelGGL((layernorm_kernel<IN_DT, 4>), grid, block, 0, st, a);
-  else if (vecs <= 16) hipLaunchKernelGGL((layernorm_kernel<IN_DT, 16>), grid, block, 0, st, a);
+  else if (vecs <= 16) hipLaunchKernelGGL((layernorm_wide_kernel<IN_DT>), dim3(a.rows), block, 0, st, a);
   else return hipErrorInvalidValue;
   return hipGetLastError();
 }
