@@ -433,10 +433,12 @@ static hipError_t launch_in_out(const GemmArgs& a, int tile, hipStream_t st) {
     if (tile == 4) tile = 1;
   }
   if (tile == 0) {
-    // Largest tile that still gives every CU a workgroup.
+    // Largest tile that still gives (nearly) every CU a workgroup. One round of 256x256 tiles takes about as long
+    // whether 160 or 256 CUs have one (33-37 us at K=1024 in bf16), and from about 160 tiles on that is less than the
+    // 128x128 tiles need (M=4096, N=3104: 47 -> 37 us; M=8192, N=1536: 39 -> 35 us; 128 tiles or fewer: slower).
     const long big = (long)((a.M + 255) / 256) * ((a.N + 255) / 256);
     const long mid = (long)((a.M + 127) / 128) * ((a.N + 127) / 128);
-    tile = big >= 256 ? 3 : mid >= 256 ? 2 : 1;
+    tile = big >= 160 ? 3 : mid >= 256 ? 2 : 1;
     // Few 64x64 tiles: nothing else on the CU hides the latency of walking K slab by slab, so four groups of waves
     // share the walk (measured with weights coming from HBM, M=128, K=768: 9.8 -> 8.2 us at N=2304, 12.3 -> 9.0 us at
     // N=3072).
