@@ -396,7 +396,7 @@ static int splitk_plan_fixed(const GemmArgs& a, int esz, int* slabs_per_slice) {
   return ks;
 }
 
-template <int IN_DT, int OUT_DT>
+template <typename Cfg, int IN_DT, int OUT_DT>
 static hipError_t launch_splitk(const GemmArgs& a, int ks, int per, hipStream_t st) {
   float* ws = a.splitk_ws;
   hipError_t e = ws ? hipSuccess : workspace_for(st, &ws);
@@ -409,14 +409,14 @@ static hipError_t launch_splitk(const GemmArgs& a, int ks, int per, hipStream_t 
   static bool attr_set[16] = {};
   int dev = 0;
   (void)hipGetDevice(&dev);
-  auto kern = gemm_kernel<CfgSmall, IN_DT, DT_F32>;
+  auto kern = gemm_kernel<Cfg, IN_DT, DT_F32>;
   if (dev >= 0 && dev < 16 && !attr_set[dev]) {
-    e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, CfgSmall::LDS_BYTES);
+    e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, Cfg::LDS_BYTES);
     if (e != hipSuccess) return e;
     attr_set[dev] = true;
   }
   const int tiles = ((a.M + 63) / 64) * ((a.N + 63) / 64);
-  hipLaunchKernelGGL(kern, dim3(tiles * ks), dim3(CfgSmall::NT), CfgSmall::LDS_BYTES, st, b);
+  hipLaunchKernelGGL(kern, dim3(tiles * ks), dim3(Cfg::NT_ALL), Cfg::LDS_BYTES, st, b);
   e = hipGetLastError();
   if (e != hipSuccess) return e;
   const long threads = (long)a.M * ((a.N + 3) / 4);
@@ -429,7 +429,7 @@ static hipError_t launch_in_out(const GemmArgs& a, int tile, hipStream_t st) {
   if ((tile == 0 && a.k_parallel) || tile == 4) {
     int per = 0;
     const int ks = splitk_plan(a, IN_DT == DT_FP8 ? 1 : 2, tile == 4, &per);
-    if (ks > 1) return launch_splitk<IN_DT, OUT_DT>(a, ks, per, st);
+    if (ks > 1) return launch_splitk<CfgSmall, IN_DT, OUT_DT>(a, ks, per, st);
     if (tile == 4) tile = 1;
   }
   if (tile == 0) {
@@ -448,7 +448,7 @@ static hipError_t launch_in_out(const GemmArgs& a, int tile, hipStream_t st) {
     if (tile == 1 && !a.k_parallel) {
       int per = 0;
       const int ks = splitk_plan_fixed(a, IN_DT == DT_FP8 ? 1 : 2, &per);
-      if (ks > 1) return launch_splitk<IN_DT, OUT_DT>(a, ks, per, st);
+      if (ks > 1) return launch_splitk<CfgSmallK4, IN_DT, OUT_DT>(a, ks, per, st);
     }
   }
   if (tile == 3) return launch_gemm_dma(a, IN_DT, OUT_DT, st);
