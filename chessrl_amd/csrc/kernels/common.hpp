@@ -129,6 +129,8 @@ struct GemmArgs {
   int slabs_per_slice;
   float* splitk_ws;   // workspace of the K-sliced path owned by the caller (else the library's per-stream one), splitk_ws_bytes long
   long splitk_ws_bytes;
+  // Optional LayerNorm over the N columns of the result, written to ln_out (only where gemm_folds_layernorm says so).
+  const float* ln_gamma; const float* ln_beta; void* ln_out; long ln_ldo; int ln_out_dtype; float ln_eps;
   int k_parallel;     // 1: tile 0 may pick the K-sliced / K-grouped kernels, whose summation order over K differs from the tiled kernels'
 };
 
@@ -258,6 +260,9 @@ struct ScatterArgs {
 // how many other rows the call has; 4 and 5 are picked by tile 0 only when a.k_parallel is set (few tiles, where they
 // are faster).
 hipError_t launch_gemm(GemmArgs a, int in_dt, int out_dt, int tile, hipStream_t st);
+// True when launch_gemm (tile 0) would take the K-sliced path for these arguments, whose second pass can apply the
+// LayerNorm that follows the GEMM (GemmArgs::ln_*); launch_gemm rejects ln_out otherwise.
+bool gemm_folds_layernorm(const GemmArgs& a, int in_dt);
 hipError_t launch_layernorm(const LayerNormArgs& a, hipStream_t st);
 hipError_t launch_embed(const EmbedArgs& a, hipStream_t st);
 hipError_t launch_token_embed(const TokenEmbedArgs& a, hipStream_t st);

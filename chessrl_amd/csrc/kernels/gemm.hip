@@ -262,6 +262,51 @@ __global__ void __launch_bounds__(Cfg::NT_ALL, Cfg::MIN_WAVES) gemm_kernel(const
 // partial [ks, M, ldp] holds the raw fp32 sums of the slices. One thread per output row and group of four columns
 // adds them in slice order (so the result does not depend on which workgroup finished first) and applies the
 // epilogue of the one-pass kernels: C = res + alpha*act(descale*sum + bias), amax, the fp8 output scale, the C/C2 split.
+// The four columns n..n+3 of row m: slices added in order, epilogue applied, result stored; v receives the values
+// (as stored: rounded to the output type) and the return value their largest magnitude.
+template <int OUT_DT>
+__device__ __forceinline__ float reduce_columns4(const GemmArgs& a, const float* partial, int ks, long ldp, int m, int n, float (&v)[4]) {
+  f32x4_t acc = {0.f, 0.f, 0.f, 0.f};
+  const float* pp = partial + (long)m * ldp + n;
+#pragma unroll 8
+  for (int s = 0; s < ks; ++s) acc += *reinterpret_cast<const f32x4_t*>(pp + (long)s * a.M * ldp);   // ldp is a multiple of 4 and >= N rounded up
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const float b = (a.bias && n + i < a.N) ? a.bias[n + i] : 0.f;
+    v[i] = apply_act(fmaf(acc[i], a.descale, b), a.act);
+  }
+  if (a.res) {
+    const long ro = (long)(a.res_rows > 0 ? m % a.res_rows : m) * a.ldr + n;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      float rv = 0.f;
+      if (n + i < a.N) {
+        if (a.res_dtype == DT_F32) rv = reinterpret_cast<const float*>(a.res)[ro + i];
+        else {
+          const uint16_t h = reinterpret_cast<const uint16_t*>(a.res)[ro + i];
+          rv = a.res_dtype == DT_F16 ? f16_bits_to_f32(h) : bf16_bits_to_f32(h);
+        }
+      }
+      v[i] = fmaf(v[i], a.alpha, rv);
+    }
+  } else {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) v[i] *= a.alpha;
+  }
+  float amax = 0.f;
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    if (n + i >= a.N) { v[i] = 0.f; continue; }
+    amax = fmaxf(amax, fabsf(v[i]));
+    const float o = OUT_DT == DT_FP8 ? v[i] * a.out_scale : v[i];
+    if (n + i < a.nsplit) store1<OUT_DT>(a.C, (long)m * a.ldc + n + i, o);
+    else store1<OUT_DT>(a.C2, (long)m * a.ldc2 + (n + i - a.nsplit), o);
+    if constexpr (OUT_DT == DT_BF16) v[i] = bf16_bits_to_f32(f32_to_bf16_bits(v[i]));
+    else if constexpr (OUT_DT == DT_F16) v[i] = f16_bits_to_f32(f32_to_f16_bits(v[i]));
+  }
+  return amax;
+}
+
 template <int OUT_DT>
 __global__ void __launch_bounds__(256) splitk_reduce_kernel(const GemmArgs a, const float* partial, int ks, long ldp) {
   const int groups = (a.N + 3) / 4;
@@ -269,46 +314,68 @@ __global__ void __launch_bounds__(256) splitk_reduce_kernel(const GemmArgs a, co
   const int m = (int)(idx / groups), n = (int)(idx - (long)m * groups) * 4;
   float local_amax = 0.f;
   if (m < a.M) {
-    f32x4_t acc = {0.f, 0.f, 0.f, 0.f};
-    const float* pp = partial + (long)m * ldp + n;
-#pragma unroll 8
-    for (int s = 0; s < ks; ++s) acc += *reinterpret_cast<const f32x4_t*>(pp + (long)s * a.M * ldp);   // ldp is a multiple of 4 and >= N rounded up
     float v[4];
-#pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      const float b = (a.bias && n + i < a.N) ? a.bias[n + i] : 0.f;
-      v[i] = apply_act(fmaf(acc[i], a.descale, b), a.act);
-    }
-    if (a.res) {
-      const long ro = (long)(a.res_rows > 0 ? m % a.res_rows : m) * a.ldr + n;
-#pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        float rv = 0.f;
-        if (n + i < a.N) {
-          if (a.res_dtype == DT_F32) rv = reinterpret_cast<const float*>(a.res)[ro + i];
-          else {
-            const uint16_t h = reinterpret_cast<const uint16_t*>(a.res)[ro + i];
-            rv = a.res_dtype == DT_F16 ? f16_bits_to_f32(h) : bf16_bits_to_f32(h);
-          }
-        }
-        v[i] = fmaf(v[i], a.alpha, rv);
-      }
-    } else {
-#pragma unroll
-      for (int i = 0; i < 4; ++i) v[i] *= a.alpha;
-    }
-#pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      if (n + i >= a.N) continue;
-      local_amax = fmaxf(local_amax, fabsf(v[i]));
-      const float o = OUT_DT == DT_FP8 ? v[i] * a.out_scale : v[i];
-      if (n + i < a.nsplit) store1<OUT_DT>(a.C, (long)m * a.ldc + n + i, o);
-      else store1<OUT_DT>(a.C2, (long)m * a.ldc2 + (n + i - a.nsplit), o);
-    }
+    local_amax = reduce_columns4<OUT_DT>(a, partial, ks, ldp, m, n, v);
   }
   if (a.amax) {
     local_amax = wave_max(local_amax);
     if ((threadIdx.x & 63) == 0) atomic_amax(a.amax, local_amax);
+  }
+}
+
+// The same pass with the LayerNorm that follows the GEMM folded in (F.layer_norm over the N columns of the stored
+// result, model_bis.py:34): one workgroup per row, up to 4096 columns, wave sums added in wave order. It takes one
+// launch out of every such GEMM + norm pair of a token step, where a launch costs as much as the work.
+template <int OUT_DT>
+__global__ void __launch_bounds__(256) splitk_reduce_ln_kernel(const GemmArgs a, const float* partial, int ks, long ldp) {
+  __shared__ float s_red[2][4];
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int m = blockIdx.x;
+  float v[4][4];
+  float local_amax = 0.f, s = 0.f;
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const int n = (i * 256 + tid) * 4;
+    if (n < a.N) {
+      local_amax = fmaxf(local_amax, reduce_columns4<OUT_DT>(a, partial, ks, ldp, m, n, v[i]));
+      s += (v[i][0] + v[i][1]) + (v[i][2] + v[i][3]);
+    }
+  }
+  s = wave_sum(s);
+  if (lane == 0) s_red[0][wave] = s;
+  __syncthreads();
+  const float mean = (((s_red[0][0] + s_red[0][1]) + s_red[0][2]) + s_red[0][3]) / (float)a.N;
+  float q = 0.f;
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const int n = (i * 256 + tid) * 4;
+    if (n < a.N) {
+#pragma unroll
+      for (int e = 0; e < 4; ++e)
+        if (n + e < a.N) { const float d = v[i][e] - mean; q += d * d; }
+    }
+  }
+  q = wave_sum(q);
+  if (lane == 0) s_red[1][wave] = q;
+  __syncthreads();
+  const float rstd = rsqrtf((((s_red[1][0] + s_red[1][1]) + s_red[1][2]) + s_red[1][3]) / (float)a.N + a.ln_eps);
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const int n = (i * 256 + tid) * 4;
+    if (n < a.N) {
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        if (n + e >= a.N) continue;
+        const float y = (v[i][e] - mean) * rstd * a.ln_gamma[n + e] + (a.ln_beta ? a.ln_beta[n + e] : 0.f);
+        const long off = (long)m * a.ln_ldo + n + e;
+        if (a.ln_out_dtype == DT_F32) reinterpret_cast<float*>(a.ln_out)[off] = y;
+        else reinterpret_cast<uint16_t*>(a.ln_out)[off] = a.ln_out_dtype == DT_BF16 ? f32_to_bf16_bits(y) : f32_to_f16_bits(y);
+      }
+    }
+  }
+  if (a.amax) {
+    local_amax = wave_max(local_amax);
+    if (lane == 0) atomic_amax(a.amax, local_amax);
   }
 }
 
@@ -368,7 +435,8 @@ static hipError_t workspace_for(hipStream_t st, float** out) {
 static int splitk_plan(const GemmArgs& a, int esz, bool forced, int* slabs_per_slice) {
   const long tiles = (long)((a.M + 63) / 64) * ((a.N + 63) / 64);
   const int nslab = (int)(((long)a.K * esz + 127) >> 7);
-  if (!forced && (tiles > 64 || nslab < 16)) return 1;
+  // (a LayerNorm waiting to be folded into the second pass is worth the slices at half the K)
+  if (!forced && (tiles > 64 || nslab < (a.ln_out ? 8 : 16))) return 1;
   int ks = (int)std::min<long>(std::min(std::max(nslab / 4, 1), 16), (256 + tiles - 1) / tiles);
   if (forced) ks = std::max(ks, std::min(nslab, 2));
   const int per = (nslab + ks - 1) / ks;
@@ -396,6 +464,11 @@ static int splitk_plan_fixed(const GemmArgs& a, int esz, int* slabs_per_slice) {
   return ks;
 }
 
+bool gemm_folds_layernorm(const GemmArgs& a, int in_dt) {
+  int per = 0;
+  return a.k_parallel && a.N <= 4096 && (a.nsplit <= 0 || a.nsplit >= a.N || !a.C2) && splitk_plan(a, in_dt == DT_FP8 ? 1 : 2, false, &per) > 1;
+}
+
 template <typename Cfg, int IN_DT, int OUT_DT>
 static hipError_t launch_splitk(const GemmArgs& a, int ks, int per, hipStream_t st) {
   float* ws = a.splitk_ws;
@@ -419,6 +492,10 @@ static hipError_t launch_splitk(const GemmArgs& a, int ks, int per, hipStream_t 
   hipLaunchKernelGGL(kern, dim3(tiles * ks), dim3(Cfg::NT_ALL), Cfg::LDS_BYTES, st, b);
   e = hipGetLastError();
   if (e != hipSuccess) return e;
+  if (a.ln_out) {
+    hipLaunchKernelGGL((splitk_reduce_ln_kernel<OUT_DT>), dim3(a.M), dim3(256), 0, st, a, ws, ks, ldp);
+    return hipGetLastError();
+  }
   const long threads = (long)a.M * ((a.N + 3) / 4);
   hipLaunchKernelGGL((splitk_reduce_kernel<OUT_DT>), dim3((unsigned)((threads + 255) / 256)), dim3(256), 0, st, a, ws, ks, ldp);
   return hipGetLastError();
@@ -426,6 +503,7 @@ static hipError_t launch_splitk(const GemmArgs& a, int ks, int per, hipStream_t 
 
 template <int IN_DT, int OUT_DT>
 static hipError_t launch_in_out(const GemmArgs& a, int tile, hipStream_t st) {
+  if (a.ln_out && !gemm_folds_layernorm(a, IN_DT)) return hipErrorInvalidValue;   // only the K-sliced path has a whole row in one place
   if ((tile == 0 && a.k_parallel) || tile == 4) {
     int per = 0;
     const int ks = splitk_plan(a, IN_DT == DT_FP8 ? 1 : 2, tile == 4, &per);

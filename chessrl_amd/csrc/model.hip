@@ -394,6 +394,8 @@ struct GOpt {
   float* amax = nullptr;
   void* C2 = nullptr; long ldc2 = 0; int nsplit = 0;
   bool k_parallel = false;  // token steps of generation: few rows, so K is spread over more waves (different summation order)
+  // LayerNorm that follows this GEMM, to be folded into it where the GEMM kernel can (*ln_folded says whether it did).
+  const float* ln_g = nullptr; const float* ln_b = nullptr; void* ln_out = nullptr; int ln_dt = DT_BF16; bool* ln_folded = nullptr;
 };
 
 int Model::gemm(const Lin& L, const void* A, long lda, int in_dt, void* C, long ldc, int out_dt, int M, const GOpt& o, hipStream_t st) {
@@ -408,6 +410,13 @@ int Model::gemm(const Lin& L, const void* A, long lda, int in_dt, void* C, long 
   g.descale = in_dt == DT_FP8 ? 1.f / (o.a_scale * L.wscale) : 1.f;
   g.alpha = o.alpha; g.out_scale = o.out_scale; g.k_parallel = o.k_parallel ? 1 : 0;
   g.splitk_ws = ws.splitk; g.splitk_ws_bytes = Workspace::SPLITK_BYTES;
+  if (o.ln_out) {
+    g.nsplit = g.N;
+    g.ln_gamma = o.ln_g; g.ln_beta = o.ln_b; g.ln_out = o.ln_out; g.ln_ldo = L.N; g.ln_out_dtype = o.ln_dt; g.ln_eps = cfg.eps;
+    const bool fold = !profiling && gemm_folds_layernorm(g, in_dt == DT_FP8 ? DT_FP8 : L.dt);
+    if (o.ln_folded) *o.ln_folded = fold;
+    if (!fold) { g.ln_gamma = g.ln_beta = nullptr; g.ln_out = nullptr; }
+  }
   const int fam = in_dt == DT_FP8 ? 0 : 5;
   if (profiling) prof_flops[fam] += 2.0 * M * (double)L.N * L.K;
   prof_begin(fam, st);
@@ -724,9 +733,10 @@ int Model::generate(const float* planes, int B, int steps, float temperature, ui
     if (sample_only) return CRL_OK;
     const int pos = 64 + k;    // sequence position of token k
     STEP_HIP(launch_decode_embed(gen_tok, wte_f32, pe_f32, pos, dyn, ws.x, B, C, VOCAB_RL, xdt, s));
+    bool normed = false;   // ws.h (or, after the last layer, ws.hl) already holds the next LayerNorm's output
     for (int l = 0; l < L; ++l) {
       const Layer& ly = layers[l];
-      STEP_RUN(lnorm(ws.x, C, xdt, ly.ln1_g, ly.ln1_b, ws.h, ad, nullptr, 1.f, C, B, C, nullptr, s));
+      if (!normed) STEP_RUN(lnorm(ws.x, C, xdt, ly.ln1_g, ly.ln1_b, ws.h, ad, nullptr, 1.f, C, B, C, nullptr, s));
       if (dyn) {
         // q -> ws.qkv [B,C]; k|v -> staging, then to the row the counter names
         GOpt o; o.k_parallel = true; o.C2 = gen_kv_stage; o.ldc2 = 2 * C; o.nsplit = C;
@@ -738,12 +748,19 @@ int Model::generate(const float* planes, int B, int steps, float temperature, ui
         STEP_RUN(gemm(ly.qkv, ws.h, C, ad, ws.qkv, C, ad, B, o, s));
       }
       STEP_HIP(launch_decode_attention(ws.qkv, C, kv_layers[l], kv_Tmax, C, pos + 1, dyn, ws.ao, C, B, H, hs, ad, attn_scale, s));
-      { GOpt o; o.k_parallel = true; o.res = ws.x; o.ldr = C; o.res_dt = xdt; STEP_RUN(gemm(ly.proj, ws.ao, C, ad, ws.x, C, xdt, B, o, s)); }
-      STEP_RUN(lnorm(ws.x, C, xdt, ly.ln2_g, ly.ln2_b, ws.h, ad, nullptr, 1.f, C, B, C, nullptr, s));
+      bool normed2 = false;
+      { GOpt o; o.k_parallel = true; o.res = ws.x; o.ldr = C; o.res_dt = xdt;
+        o.ln_g = ly.ln2_g; o.ln_b = ly.ln2_b; o.ln_out = ws.h; o.ln_dt = ad; o.ln_folded = &normed2;
+        STEP_RUN(gemm(ly.proj, ws.ao, C, ad, ws.x, C, xdt, B, o, s)); }
+      if (!normed2) STEP_RUN(lnorm(ws.x, C, xdt, ly.ln2_g, ly.ln2_b, ws.h, ad, nullptr, 1.f, C, B, C, nullptr, s));
       { GOpt o; o.k_parallel = true; o.act = ACT_GELU; STEP_RUN(gemm(ly.ff1, ws.h, C, ad, ws.f, F, ad, B, o, s)); }
-      { GOpt o; o.k_parallel = true; o.res = ws.x; o.ldr = C; o.res_dt = xdt; STEP_RUN(gemm(ly.ff2, ws.f, F, ad, ws.x, C, xdt, B, o, s)); }
+      { // the norm that reads this GEMM's result (the next layer's ln_1, or ln_f) rides on its second pass where it is K-sliced
+        GOpt o; o.k_parallel = true; o.res = ws.x; o.ldr = C; o.res_dt = xdt; o.ln_folded = &normed;
+        if (l + 1 < L) { o.ln_g = layers[l + 1].ln1_g; o.ln_b = layers[l + 1].ln1_b; o.ln_out = ws.h; o.ln_dt = ad; }
+        else { o.ln_g = lnf_g; o.ln_b = lnf_b; o.ln_out = ws.hl; o.ln_dt = hd; }
+        STEP_RUN(gemm(ly.ff2, ws.f, F, ad, ws.x, C, xdt, B, o, s)); }
     }
-    STEP_RUN(lnorm(ws.x, C, xdt, lnf_g, lnf_b, ws.hl, hd, nullptr, 1.f, C, B, C, nullptr, s));
+    if (!normed) STEP_RUN(lnorm(ws.x, C, xdt, lnf_g, lnf_b, ws.hl, hd, nullptr, 1.f, C, B, C, nullptr, s));
     { GOpt o; o.k_parallel = true; STEP_RUN(gemm(lm_head, ws.hl, C, hd, gen_logits, VOCAB_RL, DT_F32, B, o, s)); }
     if (dyn) STEP_HIP(launch_add_int(gen_k, 1, s));
     return CRL_OK;

@@ -417,6 +417,30 @@ def test_generate_replayed_graph_equals_plain_launches(cuda):
     m._engine.set_decode_graph(False)
 
 
+def test_generate_folded_layernorm_equals_separate_kernels(cuda):
+    """The token step folds the LayerNorm after the out-projection and after FFN-2 into the second pass of those
+    K-sliced GEMMs; the profiling mode keeps the separate LayerNorm launches. Same step logits up to summation order."""
+    B, steps = 4, 40
+    oracle = om.test_init_(om.GPTOracle(3, 8, 256), seed=11)
+    planes, _ = positions(B, seed=12)
+    m = models.GPT(models.GPTConfig(block_size=256, vocab_size=1929, n_layer=3, n_head=8, n_embd=256))
+    m.load_state_dict(oracle.state_dict())
+    x = planes.to(cuda)
+    seq_a, log_a = m._engine.generate(x, steps, T=0.0, rules=False, want_step_out=True, out_logits=True)
+    m._engine.set_profiling(True)
+    seq_b, log_b = m._engine.generate(x, steps, T=0.0, rules=False, want_step_out=True, out_logits=True)
+    prof = m._engine.get_profile()
+    m._engine.set_profiling(False)
+    assert prof["layernorm"]["launches"] > (2 * 3 + 1) * (steps - 1)     # every norm of every step ran as its own launch
+    # greedy decoding can part ways after a near-tie, so compare the steps up to the first differing token
+    same = (seq_a == seq_b).all(0).cpu().tolist()
+    upto = same.index(False) if False in same else steps + 1
+    assert upto >= 10
+    err = rel_rms(log_a[:, :upto - 1].cpu(), log_b[:, :upto - 1].cpu())
+    print("folded vs separate LayerNorm: %d common steps, logits rel-rms %.2e" % (upto - 1, err))
+    assert err < 2e-3
+
+
 def test_generate_forced_tokens(cuda):
     """generate_sequence's bookkeeping (model_bis.py:252-259) on a model rigged to prefer end_variation: the sequences
     equal the rule application of the oracle to the arg-max of the recorded step logits."""
