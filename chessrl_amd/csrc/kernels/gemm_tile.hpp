@@ -266,7 +266,7 @@ __device__ __forceinline__ void gemm_epilogue(const GemmArgs& a, f32x16_t (&acc)
             v[it][e] = fmaf(v[it][e], alpha, __uint_as_float((e & 1) ? (w[e >> 1] & 0xffff0000u) : (w[e >> 1] << 16)));
         }
       }
-    } else {
+    } else if (alpha != 1.f) {
 #pragma unroll
       for (int it = 0; it < ITERS; ++it)
 #pragma unroll
