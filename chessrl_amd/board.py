@@ -61,7 +61,8 @@ def legal_moves(fen):
     """UCI strings of the legal moves (the library's generation order)."""
     buf = C.create_string_buffer(6 * 256)
     n = check(lib().crl_legal_moves(fen.encode(), buf, 256), "crl_legal_moves")
-    return [buf.raw[i * 6:(i + 1) * 6].split(b"\0")[0].decode() for i in range(n)]
+    raw = buf.raw
+    return [raw[i * 6:(i + 1) * 6].split(b"\0")[0].decode() for i in range(n)]
 
 
 def child_fens(fen):
@@ -69,8 +70,9 @@ def child_fens(fen):
     fb = C.create_string_buffer(96 * 256)
     mb = C.create_string_buffer(6 * 256)
     n = check(lib().crl_child_fens(fen.encode(), fb, mb, 256), "crl_child_fens")
-    moves = [mb.raw[i * 6:(i + 1) * 6].split(b"\0")[0].decode() for i in range(n)]
-    fens = [fb.raw[i * 96:(i + 1) * 96].split(b"\0")[0].decode() for i in range(n)]
+    mraw, fraw = mb.raw, fb.raw
+    moves = [mraw[i * 6:(i + 1) * 6].split(b"\0")[0].decode() for i in range(n)]
+    fens = [fraw[i * 96:(i + 1) * 96].split(b"\0")[0].decode() for i in range(n)]
     return moves, fens
 
 
@@ -105,5 +107,6 @@ def random_positions(seed, n, max_plies=80, late_fraction=0.0, late_max_pieces=1
     if masks_leela:
         out["masks_leela"] = ml
     if fens:
-        out["fens"] = [fb.raw[i * 96:(i + 1) * 96].split(b"\0")[0].decode() for i in range(n)]
+        fraw = fb.raw
+        out["fens"] = [fraw[i * 96:(i + 1) * 96].split(b"\0")[0].decode() for i in range(n)]
     return out

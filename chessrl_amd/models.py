@@ -301,13 +301,15 @@ class _Engine:
         vals = torch.empty((max(cap, 1),), dtype=torch.float32) if want_values else None
         check(lib().crl_model_search_1ply(self.handle, arr, n, int(chunk), float(T), int(seed) & (2 ** 64 - 1), best, counts,
                                           mv, _ptr(vals), cap, int(threads)), "crl_model_search_1ply")
-        moves = [best.raw[6 * i:6 * i + 6].split(b"\0")[0].decode() for i in range(n)]
+        braw = best.raw                       # .raw copies the whole buffer: take it once
+        moves = [braw[6 * i:6 * i + 6].split(b"\0")[0].decode() for i in range(n)]
         if not want_values:
             return moves
+        mraw = mv.raw
         per_root, o = [], 0
         for i in range(n):
             k = counts[i]
-            per_root.append(([mv.raw[6 * (o + c):6 * (o + c) + 6].split(b"\0")[0].decode() for c in range(k)], vals[o:o + k].clone()))
+            per_root.append(([mraw[6 * (o + c):6 * (o + c) + 6].split(b"\0")[0].decode() for c in range(k)], vals[o:o + k].clone()))
             o += k
         return moves, per_root
 
