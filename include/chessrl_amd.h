@@ -102,7 +102,10 @@ int crl_random_positions(uint64_t seed, int n, int max_plies, double late_fracti
  * crl_model_generate use them): 4 = 64x64 tiles with K cut into slices, one workgroup per (tile, slice) leaving raw
  * fp32 sums in a workspace of 64 MB that the library keeps per stream, and a second kernel that adds them in slice
  * order and applies the epilogue; 5 = 64x64 tiles whose K slabs four groups of four waves take in turn and add up in
- * LDS. Both are deterministic from launch to launch but differ from 1-3 in summation order. */
+ * LDS. Both are deterministic from launch to launch but differ from 1-3 in summation order. With tile 0, outputs of at
+ * most 256 columns whose K is 4 KB or more per row are always K-sliced the same way (a function of N and K alone), so
+ * the row-count independence holds for them too. The first K-sliced launch on a stream allocates that stream's
+ * workspace: issue it once outside any graph capture. */
 int crl_gemm(const void* A, int64_t lda, const void* W, int64_t ldw, void* C, int64_t ldc,
              int M, int N, int K, int in_dtype, int out_dtype,
              const float* bias, int act, float descale, float alpha,
