@@ -20,9 +20,13 @@ What each class follows (reference file:line):
                  scaling of input and weight, high-precision accumulate. Restated as
                  quantise->dequantise->F.linear. PARITY UNPINNED against transformer_engine.
 
-Pins: library routines (F.layer_norm, F.gelu, F.scaled_dot_product_attention) are used
-directly; the relative shift is pinned in tests/test_oracle.py against the pad/reshape
-formulation and a brute-force definition; the move lists are pinned by SHA-256.
+Pins: GPTOracle (64-token forward, token forward, loss), BT4Oracle (policy and value) and
+relative_attention are checked in tests/test_golden.py against outputs of the reference's own
+module code on the same weights and inputs (tests/golden/reference_vectors.npz, written by
+tests/golden/make_vectors.py). Library routines (F.layer_norm, F.gelu,
+F.scaled_dot_product_attention) are used directly; the relative shift is also pinned in
+tests/test_oracle.py against the pad/reshape formulation and a brute-force definition; the move
+lists are pinned by SHA-256. BT4ClassOracle and the fp8 emulation have no such vectors.
 """
 import math
 
@@ -271,6 +275,22 @@ class _ValueHead(nn.Module):
         return self.dense3(act(self.dense2(x)))
 
 
+def relative_attention(at, x, pe, H):
+    """RelativeMultiHeadAttention2.forward (new_paradigm/attn.py:491-523) on x [B,T,C] with the position table
+    pe [T,C] (the same for every batch row, so it is projected once)."""
+    B, T, C = x.shape
+    hs = C // H
+    q = at.query_proj(x).view(B, T, H, hs)
+    k = at.key_proj(x).view(B, T, H, hs).permute(0, 2, 1, 3)
+    v = at.value_proj(x).view(B, T, H, hs).permute(0, 2, 1, 3)
+    p = at.pos_proj(pe).view(T, H, hs)
+    content = torch.matmul((q + at.u_bias).transpose(1, 2), k.transpose(2, 3))
+    pos = torch.matmul((q + at.v_bias).transpose(1, 2), p.permute(1, 2, 0))
+    score = (content + rel_shift(pos)) / math.sqrt(C)
+    ctx = torch.matmul(F.softmax(score, -1), v).transpose(1, 2).reshape(B, T, C)
+    return at.out_proj(ctx)
+
+
 class BT4Oracle(nn.Module):
     def __init__(self, num_layers=10, d_model=512, d_ff=736, num_heads=8):
         super().__init__()
@@ -293,19 +313,9 @@ class BT4Oracle(nn.Module):
         x = self.ma_gating(self.layernorm1(F.gelu(self.linear1(x))))
         B, T, C = x.shape
         H = self.num_heads
-        hs = C // H
         pe = self.pe
         for ly in self.layers:
-            at = ly.attention
-            q = at.query_proj(x).view(B, T, H, hs)
-            k = at.key_proj(x).view(B, T, H, hs).permute(0, 2, 1, 3)
-            v = at.value_proj(x).view(B, T, H, hs).permute(0, 2, 1, 3)
-            p = at.pos_proj(pe).view(T, H, hs)
-            content = torch.matmul((q + at.u_bias).transpose(1, 2), k.transpose(2, 3))
-            pos = torch.matmul((q + at.v_bias).transpose(1, 2), p.permute(1, 2, 0))
-            score = (content + rel_shift(pos)) / math.sqrt(C)
-            ctx = torch.matmul(F.softmax(score, -1), v).transpose(1, 2).reshape(B, T, C)
-            x = ly.norm1(at.out_proj(ctx) + x)
+            x = ly.norm1(relative_attention(ly.attention, x, pe, H) + x)
             y = F.gelu(ly.ff2(ly.ff1(x)))
             x = ly.norm2(y + x)
         wdl = self.value_head(x, F.gelu)

@@ -1,0 +1,39 @@
+"""Deterministic tensor contents shared by the script that writes the golden vectors and the tests that read them.
+
+Values come from integer hashing only (no library random generator, no transcendental function), so the same
+name and shape give bit-identical float32 data on any machine and the fixtures need to hold outputs only."""
+import zlib
+
+import numpy as np
+
+
+def det_fill(name, shape, lo, hi):
+    """float32 array of `shape`, values in [lo, hi), a pure function of (name, shape, lo, hi)."""
+    n = int(np.prod(shape)) if len(shape) else 1
+    x = np.arange(n, dtype=np.uint64) + np.uint64(zlib.crc32(name.encode()) << 20)
+    with np.errstate(over="ignore"):
+        x = (x ^ (x >> np.uint64(30))) * np.uint64(0xBF58476D1CE4E5B9)
+        x = (x ^ (x >> np.uint64(27))) * np.uint64(0x94D049BB133111EB)
+        x = x ^ (x >> np.uint64(31))
+    u = (x >> np.uint64(40)).astype(np.float64) / float(1 << 24)  # 24 bits -> [0, 1)
+    return (lo + (hi - lo) * u).astype(np.float32).reshape(shape)
+
+
+def fill_state_dict(shapes):
+    """{key: shape} -> {key: float32 array}. Linear and embedding weights are uniform with unit-order outputs,
+    LayerNorm weights and the gating offsets sit around one, everything else (biases, gating exponents, the
+    attention's u/v offsets) around zero, so that no term of a forward pass is negligible."""
+    out = {}
+    for k, shp in shapes.items():
+        leaf = k.split(".")[-1]
+        is_norm = any(s in k for s in ("ln_", "norm", "layernorm"))
+        if leaf == "weight" and len(shp) == 2:
+            a = (3.0 / shp[1]) ** 0.5
+            out[k] = det_fill(k, shp, -a, a)
+        elif (leaf == "weight" and is_norm) or leaf == "b":
+            out[k] = det_fill(k, shp, 0.8, 1.2)
+        elif leaf in ("u_bias", "v_bias"):
+            out[k] = det_fill(k, shp, -0.5, 0.5)
+        else:
+            out[k] = det_fill(k, shp, -0.2, 0.2)
+    return out
