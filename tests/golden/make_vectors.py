@@ -19,8 +19,13 @@ What is written (all float32):
   gpt_last      GPT.forward((planes, idx[:, :0]))[0]                    model_bis.py:171-199   [B,1,1929]
   gpt_tok_last  GPT.forward((planes, idx))[0]                           same                    [B,1,1929]
   gpt_tok_rows, gpt_tok_loss  GPT.forward((planes, idx), compute_loss=True): logits[:, TOK_ROWS] and the loss
+  gpt_generated GPT.generate_sequence(planes, T=0)[0] on rigged weights  model_bis.py:213-268   [B,block_size-64]
   attn_out      RelativeMultiHeadAttention2(x, x, x, pe)                new_paradigm/attn.py:491-533
   bt4_policy, bt4_value  BT4.forward(inp, compute_loss=True)[:2]        new_paradigm/value.py:155-212
+  grpo_loss_kl_legal_logpdiff  ChessGRPOTrainer.compute_loss_bis(...): loss, mean KL, legal probability, avg_logp_diff
+                                                                       grpo_refactored.py:322-372
+  leela_mapping_black, leela_to_rl_*  the mirror table and map_leela_to_rl(policies, first_is_white)
+                                                                       Leela/compare_policy.py:469-523
 """
 import ast
 import importlib.util
@@ -36,7 +41,7 @@ import torch.nn.functional as F
 
 HERE = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, HERE)
-from fill import det_fill, fill_state_dict  # noqa: E402
+from fill import det_fill, fill_state_dict, rig_end_variation  # noqa: E402
 
 # sizes of the fixture models (small, head size 32 so that the GPU library accepts them too)
 GPT_CFG = dict(block_size=96, vocab_size=1929, n_layer=2, n_head=4, n_embd=128, dropout=0.0, bias=True)
@@ -45,6 +50,7 @@ TOK_ROWS = [0, 31, 63, 64, 70]   # rows of the all-token logits kept (the loss c
 BT4_CFG = dict(num_layers=2, d_model=128, d_ff=192, num_heads=4)
 BT4_B, BT4_S = 2, 2
 ATTN_B = 3
+GRPO_G, GRPO_B, GRPO_BETA, GRPO_LEGAL_W = 2, 2, 0.04, 0.1
 
 
 def planes_input(name, shape):
@@ -80,6 +86,52 @@ def classes_of(path, names, namespace, redirect_cuda=False):
     return namespace
 
 
+def functions_of(path, class_name, names, namespace, redirect_cuda=False):
+    """The named methods of one class, compiled as plain functions (first argument: whatever stands in for self)."""
+    lines = open(path).read().split("\n")
+    # Only the class is parsed: the script part of grpo_refactored.py uses an f-string form that needs Python 3.12.
+    start = [i for i, l in enumerate(lines) if l.startswith("class " + class_name)][0]
+    stop = [i for i in range(start + 1, len(lines)) if lines[i] and not lines[i][0].isspace() and not lines[i].startswith("#")]
+    tree = ast.parse("\n" * start + "\n".join(lines[start:stop[0] if stop else len(lines)]), filename=path)
+    cls = tree.body[0]
+    mod = ast.Module(body=[n for n in cls.body if isinstance(n, ast.FunctionDef) and n.name in names], type_ignores=[])
+    if redirect_cuda:
+        mod = _Redirect().visit(mod)
+    exec(compile(ast.fix_missing_locations(mod), path, "exec"), namespace)
+    return namespace
+
+
+def statements_of(path, names, namespace):
+    """Module-level functions, assignments to the named variables, and loops that fill one of them."""
+    tree = ast.parse(open(path).read(), filename=path)
+    keep = []
+    for node in tree.body:
+        if isinstance(node, ast.FunctionDef) and node.name in names:
+            keep.append(node)
+        elif isinstance(node, ast.Assign) and all(isinstance(t, ast.Name) and t.id in names for t in node.targets):
+            keep.append(node)
+        elif isinstance(node, ast.For) and any(isinstance(n, ast.Subscript) and isinstance(n.value, ast.Name) and
+                                               n.value.id in names and isinstance(n.ctx, ast.Store) for n in ast.walk(node)):
+            keep.append(node)
+    exec(compile(ast.fix_missing_locations(ast.Module(body=keep, type_ignores=[])), path, "exec"), namespace)
+    return namespace
+
+
+def grpo_inputs():
+    """new_logits, ref_logits [G,B,256,1929], advantages [G,B], sampled sequences [G,B,192] (an `end` token at a
+    different place in each, none in one of them), legal masks [G,B,1929]."""
+    G, B = GRPO_G, GRPO_B
+    new_logits = det_fill("grpo.new", (G, B, 256, 1929), -3.0, 3.0)
+    ref_logits = (new_logits + det_fill("grpo.delta", (G, B, 256, 1929), -1.0, 1.0)).astype(np.float32)
+    adv = det_fill("grpo.adv", (G, B), -1.5, 1.5)
+    seqs = token_input("grpo.seq", (G, B, 192))
+    for i, at in enumerate([5, 191, None, 60][: G * B]):
+        if at is not None:
+            seqs.reshape(-1, 192)[i, at] = 1927
+    legal = (det_fill("grpo.legal", (G, B, 1929), 0.0, 1.0) < 0.02).astype(np.float32)
+    return new_logits, ref_logits, adv, seqs, legal
+
+
 def load_filled(module):
     sd = module.state_dict()
     filled = fill_state_dict({k: tuple(v.shape) for k, v in sd.items() if k != "pe"})
@@ -102,6 +154,13 @@ def main(ref):
         out["gpt_tok_last"] = gpt((planes, idx))[0].numpy()
         logits, loss, _ = gpt((planes, idx), compute_loss=True)
         out["gpt_tok_rows"], out["gpt_tok_loss"] = logits[:, TOK_ROWS].numpy(), loss.numpy()
+        # greedy generation with the forced-token rules, on a model rigged to prefer end_variation
+        ns.update(start_think_index=1924, end_think_index=1925, end_variation_index=1926, end_index=1927)
+        arrays = rig_end_variation(fill_state_dict({k: tuple(v.shape) for k, v in gpt.state_dict().items() if k != "pe"}))
+        gpt.load_state_dict({k: torch.from_numpy(v) for k, v in arrays.items()}, strict=False)
+        seq, probs = gpt.generate_sequence(planes, T=0)
+        assert probs is None
+        out["gpt_generated"] = seq.numpy()
 
         # ---- relative attention (new_paradigm/attn.py), imported whole
         spec = importlib.util.spec_from_file_location("ref_attn", os.path.join(ref, "new_paradigm", "attn.py"))
@@ -127,6 +186,24 @@ def main(ref):
         res = bt4([planes, targets, None, values], compute_loss=True)
         out["bt4_policy"], out["bt4_value"] = res[0].numpy(), res[1].numpy()
         assert torch.equal(bt4([planes]), res[0])
+
+        # ---- GRPO scoring terms (grpo_refactored.py:322-372), the method run with a stand-in for `self`
+        import types
+        ns = functions_of(os.path.join(ref, "grpo_refactored.py"), "ChessGRPOTrainer", ["compute_loss_bis"],
+                          dict(base, end_index=1927, print=lambda *a, **k: None), redirect_cuda=True)
+        me = types.SimpleNamespace(beta=GRPO_BETA, config={"legal_loss_weight": GRPO_LEGAL_W})
+        new_logits, ref_logits, adv, seqs, legal = (torch.from_numpy(a) for a in grpo_inputs())
+        loss, mean_kl, legal_prob = ns["compute_loss_bis"](me, new_logits, ref_logits, adv, seqs, legal)
+        out["grpo_loss_kl_legal_logpdiff"] = np.array([loss.item(), mean_kl.item(), legal_prob.item(), me.avg_logp_diff.item()])
+
+    # ---- the 1858 -> 1929 move remap tables (Leela/compare_policy.py:469-523)
+    ns = statements_of(os.path.join(ref, "Leela", "compare_policy.py"),
+                       ["policy_index_leela", "policy_index", "policy_index_leela_size", "policy_index_size",
+                        "mirror_uci_string", "policy_dict", "mapping_black", "mapping_white", "map_leela_to_rl"], dict(base))
+    out["leela_mapping_black"] = ns["mapping_black"].astype(np.float32)
+    pol = det_fill("leela.policies", (4, 1858), 0.0, 1.0)
+    out["leela_to_rl_white_first"] = ns["map_leela_to_rl"](pol, True)
+    out["leela_to_rl_black_first"] = ns["map_leela_to_rl"](pol, False)
 
     path = os.path.join(HERE, "reference_vectors.npz")
     np.savez_compressed(path, **{k: np.asarray(v, dtype=np.float32) for k, v in out.items()})

@@ -10,7 +10,7 @@ import torch
 HERE = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, os.path.join(HERE, "golden"))
 import make_vectors as mv  # noqa: E402  (sizes and input recipes only; nothing of the reference is read here)
-from fill import det_fill, fill_state_dict  # noqa: E402
+from fill import det_fill, fill_state_dict, rig_end_variation  # noqa: E402
 
 from oracle import models as om  # noqa: E402
 
@@ -78,6 +78,27 @@ def test_gpt_vectors_would_catch_a_swapped_split():
     assert np.abs(g.forward_last(planes)[:, None, :].numpy() - GOLD["gpt_last"]).max() > 1e-3
 
 
+def test_greedy_generation_with_forced_tokens_matches_reference_vectors():
+    """GPT.generate_sequence(T=0) of model_bis.py:213-268: arg-max of the oracle's last-token logits, fed back through
+    the oracle's rule bookkeeping, step by step."""
+    planes, _ = gpt_inputs()
+    g = gpt_oracle()
+    arrays = rig_end_variation(fill_state_dict({k: tuple(v.shape) for k, v in g.state_dict().items() if k != "pe"}))
+    g.load_state_dict({k: torch.from_numpy(v) for k, v in arrays.items()}, strict=False)
+    want = GOLD["gpt_generated"].astype(np.int64)
+    steps = want.shape[1] - 1
+    assert steps == mv.GPT_CFG["block_size"] - 65
+    raw = torch.zeros(mv.GPT_B, 0, dtype=torch.int64)
+    seq = om.apply_generation_rules(raw)
+    for _ in range(steps):
+        nxt = g.forward_tokens(planes, seq)[0][:, 0].argmax(-1, keepdim=True)
+        raw = torch.cat((raw, nxt), dim=1)
+        seq = om.apply_generation_rules(raw)
+    assert seq.tolist() == want.tolist()
+    rows = want.tolist()
+    assert any(1925 in r and 1927 in r for r in rows) and any(1925 not in r for r in rows)
+
+
 def test_bt4_forward_matches_reference_vectors():
     c = mv.BT4_CFG
     m = filled(om.BT4Oracle(c["num_layers"], c["d_model"], c["d_ff"], c["num_heads"]))
@@ -99,3 +120,18 @@ def test_relative_attention_matches_reference_vectors():
     pe = torch.from_numpy(det_fill("attn.pe", (1, 64, C), -1.0, 1.0))[0]
     with torch.no_grad():
         close(om.relative_attention(at, x, pe, H), GOLD["attn_out"])
+
+
+def test_leela_mirror_table_matches_reference_vectors():
+    """mapping_black of Leela/compare_policy.py:469-487, all 1858 entries, against the library's host table."""
+    from chessrl_amd import vocab
+    w, b = vocab.leela_to_rl_maps()
+    assert np.array_equal(b.astype(np.int64), GOLD["leela_mapping_black"].astype(np.int64))
+    assert np.array_equal(w, np.arange(1858))
+    # map_leela_to_rl on four rows, white first and black first: a scatter through those tables
+    pol = det_fill("leela.policies", (4, 1858), 0.0, 1.0)
+    for first_white, key in ((True, "leela_to_rl_white_first"), (False, "leela_to_rl_black_first")):
+        res = np.zeros((4, 1929), dtype=np.float32)
+        for r in range(4):
+            res[r, w if (r % 2 == 0) == first_white else b] = pol[r]
+        assert np.array_equal(res, GOLD[key])

@@ -11,7 +11,7 @@ import torch
 HERE = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, os.path.join(HERE, "golden"))
 import make_vectors as mv  # noqa: E402
-from fill import fill_state_dict  # noqa: E402
+from fill import det_fill, fill_state_dict  # noqa: E402
 
 from chessrl_amd import models  # noqa: E402
 
@@ -64,3 +64,41 @@ def test_bt4_against_reference_vectors(cuda, act):
     print("bt4 %s vs reference vectors: policy rel-rms %.2e, wdl max-abs %.2e" % (act, e, w))
     assert e < (2e-2 if act == "bf16" else 4e-3)
     assert w <= (1e-2 if act == "bf16" else 2e-3)
+
+
+def test_leela_to_rl_kernel_against_reference_vectors(cuda):
+    import ctypes as C
+    from chessrl_amd._lib import check, lib
+    pol = torch.from_numpy(det_fill("leela.policies", (4, 1858), 0.0, 1.0)).to(cuda)
+    st = C.c_void_p(torch.cuda.current_stream().cuda_stream)
+    for first_white, key in ((True, "leela_to_rl_white_first"), (False, "leela_to_rl_black_first")):
+        wtm = torch.tensor([(r % 2 == 0) == first_white for r in range(4)], dtype=torch.uint8, device=cuda)
+        dst = torch.full((4, 1929), 7.0, device=cuda)
+        check(lib().crl_leela_to_rl(C.c_void_p(pol.data_ptr()), 1858, C.c_void_p(dst.data_ptr()), 1929,
+                                    C.c_void_p(wtm.data_ptr()), 4, st), "crl_leela_to_rl")
+        assert np.array_equal(dst.cpu().numpy(), GOLD[key])
+
+
+def test_grpo_terms_against_reference_vectors(cuda):
+    """crl_token_scores' three outputs, assembled the way ChessGRPOTrainer.compute_loss_bis (grpo_refactored.py:322-372)
+    assembles its own: mean of the masked per-token KL, and the signed mean log-probability difference."""
+    G, B = mv.GRPO_G, mv.GRPO_B
+    new_logits, ref_logits, adv, seqs, _ = (torch.from_numpy(a).to(cuda) for a in mv.grpo_inputs())
+    new_l = new_logits[:, :, 63:-1].reshape(-1, 1929).contiguous()
+    ref_l = ref_logits[:, :, 63:-1].reshape(-1, 1929).contiguous()
+    logp, rlogp, kl = models.token_scores(new_l, seqs.reshape(-1), ref_l, want_kl=True)
+    logp, rlogp, kl = (t.view(G, B, 192) for t in (logp, rlogp, kl))
+    pos = torch.arange(192, device=cuda)
+    first = torch.where(seqs == 1927, pos.expand_as(seqs), 192).min(-1).values
+    mask = (pos.view(1, 1, -1) <= first.unsqueeze(-1)).float()
+    mean_kl = ((kl * mask).sum(-1) / mask.sum(-1)).mean().item()
+    a = adv.view(G, B, 1)
+    diff = ((a > 0) * (logp - rlogp) + (a < 0) * (rlogp - logp)).mean().item()
+    per_token = -(a - mv.GRPO_BETA * kl)     # exp(new - new.detach()) is one
+    loss_without_legal_term = ((per_token * mask).sum(-1) / mask.sum(-1)).mean().item()
+    want_loss, want_kl, _, want_diff = GOLD["grpo_loss_kl_legal_logpdiff"].tolist()
+    print("grpo terms: mean kl %.6f vs %.6f, logp diff %.6f vs %.6f" % (mean_kl, want_kl, diff, want_diff))
+    assert abs(mean_kl - want_kl) < 1e-5 * max(1.0, abs(want_kl))
+    assert abs(diff - want_diff) < 1e-5
+    # the remaining term of the loss (KL of the played move's distribution to the legal mask) is the caller's
+    assert loss_without_legal_term < want_loss + 1e-4
