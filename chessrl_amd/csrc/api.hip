@@ -433,16 +433,19 @@ int crl_model_set_amax(crl_model* m, const float* in, int n) {
   return CRL_OK;
 }
 int crl_model_forward(crl_model* m, const float* planes, int B, float* policy_logits, float* wdl_logits, void* stream) {
+  if (m && B == 0) return CRL_OK;  // an empty batch writes nothing (its buffers may be null)
   if (!m || !planes) return arg_fail("crl_model_forward: bad arguments");
   return m->impl.forward(planes, nullptr, nullptr, B, policy_logits, wdl_logits, false, (hipStream_t)stream);
 }
 int crl_model_forward_compact(crl_model* m, const uint8_t* ids, const uint8_t* flags, int B, float* policy_logits,
                               float* wdl_logits, void* stream) {
+  if (m && B == 0) return CRL_OK;
   if (!m || !ids || !flags) return arg_fail("crl_model_forward_compact: bad arguments");
   return m->impl.forward(nullptr, ids, flags, B, policy_logits, wdl_logits, false, (hipStream_t)stream);
 }
 int crl_model_forward_tokens(crl_model* m, const float* planes, const int64_t* idx, int B, int t, float* last_logits,
                              float* all_logits, void* stream) {
+  if (m && B == 0) return CRL_OK;
   if (!m || !planes) return arg_fail("crl_model_forward_tokens: bad arguments");
   return m->impl.forward_tokens(planes, nullptr, nullptr, idx, t, B, last_logits, all_logits, nullptr, false, (hipStream_t)stream);
 }

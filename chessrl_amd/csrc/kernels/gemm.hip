@@ -22,6 +22,7 @@
 //  * Workgroup ids are remapped so each XCD (ids round-robin over 8 XCDs) walks a
 //    contiguous range of tiles, N fastest: the weight matrix stays in that XCD's L2
 //    and every activation slab is fetched from HBM by one XCD only.
+#include <atomic>
 #include <mutex>
 #include <unordered_map>
 
@@ -394,7 +395,7 @@ typedef GemmCfg<64, 64, 2, 2, 2, 0, 2, 4> CfgSmallK4;   // the same tile walked 
 
 template <typename Cfg, int IN_DT, int OUT_DT>
 static hipError_t launch_cfg(const GemmArgs& a, hipStream_t st) {
-  static bool attr_set[16] = {};
+  static std::atomic<bool> attr_set[16] = {};
   int dev = 0;
   (void)hipGetDevice(&dev);
   auto kern = gemm_kernel<Cfg, IN_DT, OUT_DT>;
@@ -479,7 +480,7 @@ static hipError_t launch_splitk(const GemmArgs& a, int ks, int per, hipStream_t 
   b.C = b.C2 = ws; b.ldc = b.ldc2 = ldp; b.nsplit = a.N;
   b.bias = nullptr; b.res = nullptr; b.amax = nullptr; b.act = ACT_NONE; b.descale = 1.f; b.alpha = 1.f; b.out_scale = 1.f;
   b.vec_ok = 1; b.stream_out = 0; b.k_slices = ks; b.slabs_per_slice = per; b.splitk_ws = nullptr;
-  static bool attr_set[16] = {};
+  static std::atomic<bool> attr_set[16] = {};
   int dev = 0;
   (void)hipGetDevice(&dev);
   auto kern = gemm_kernel<Cfg, IN_DT, DT_F32>;

@@ -2,6 +2,9 @@
 // of a 4096-position forward). The call sites, operand layout and epilogue are those described in gemm.hip.
 #include "gemm_tile.hpp"
 
+#include <atomic>
+#include <mutex>
+
 namespace crl {
 
 // ---- 256x256 tile fed by direct global->LDS loads ------------------------------------------
@@ -154,6 +157,10 @@ __global__ void __launch_bounds__(Cfg::NT, 2) gemm_dma_kernel(const GemmArgs a, 
     }
   };
 
+  // A wave whose 128x64 part lies wholly outside C (the last tile column of N = 3104 holds 32 columns) still takes its
+  // share of the loads and every barrier, but reads no fragments and issues no MFMAs.
+  const bool wave_active = (m0 + wm * Cfg::WM < a.M) && (n0 + wn * Cfg::WN < a.N);
+
 #pragma unroll
   for (int s0 = 0; s0 < NSTAGE - 1; ++s0)
     if (s0 < nslab) issue(s0);
@@ -167,6 +174,7 @@ __global__ void __launch_bounds__(Cfg::NT, 2) gemm_dma_kernel(const GemmArgs a, 
     __syncthreads();
     if (slab + NSTAGE - 1 < nslab) issue(slab + NSTAGE - 1);
     const uint8_t* st = smem + (slab % NSTAGE) * Cfg::STAGE_BYTES;
+    if (!wave_active) continue;
 #pragma unroll
     for (int ks = 0; ks < KSTEPS; ++ks) {
       Frag<IN_DT> wf[TN], xf[TM];
@@ -187,6 +195,8 @@ __global__ void __launch_bounds__(Cfg::NT, 2) gemm_dma_kernel(const GemmArgs a, 
 // One 256-byte block of zeros per device: the source of K-tail chunks for the direct-to-LDS loads.
 static const uint8_t* device_zeros(hipError_t* err) {
   static uint8_t* z[16] = {};
+  static std::mutex mu;   // first calls on one device may come from several host threads
+  std::lock_guard<std::mutex> lock(mu);
   int dev = 0;
   *err = hipGetDevice(&dev);
   if (*err != hipSuccess || dev < 0 || dev >= 16) { if (*err == hipSuccess) *err = hipErrorInvalidDevice; return nullptr; }
@@ -203,7 +213,7 @@ static const uint8_t* device_zeros(hipError_t* err) {
 
 template <typename DCfg, int IN_DT, int OUT_DT>
 static hipError_t launch_dma(const GemmArgs& a, hipStream_t st) {
-  static bool attr_set[16] = {};
+  static std::atomic<bool> attr_set[16] = {};
   hipError_t e = hipSuccess;
   const uint8_t* zeros = device_zeros(&e);
   if (!zeros) return e;

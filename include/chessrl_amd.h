@@ -174,7 +174,8 @@ int crl_model_set_amax(crl_model* m, const float* in, int n);
 /* The forward pass. planes: device f32 [B,64,19] (GPT.forward batch[0] / BT4.forward inp[0]).
  * policy_logits: device f32 [B, vocab] with vocab = 1929 (GPT64: logits of token 63,
  * model_bis.py:370; BT4: value.py:187) or 1858 (BT4-class). wdl_logits: device f32 [B,3]
- * in the order [black win, draw, white win] (value.py:248), NULL for GPT64 or to skip. */
+ * in the order [black win, draw, white win] (value.py:248), NULL for GPT64 or to skip.
+ * B = 0 is accepted by this and the two entry points below: nothing is launched or written. */
 int crl_model_forward(crl_model* m, const float* planes, int B, float* policy_logits, float* wdl_logits, void* stream);
 /* Same from the compact board form (device uint8[B,64] ids + uint8[B,4] flags). */
 int crl_model_forward_compact(crl_model* m, const uint8_t* ids, const uint8_t* flags, int B,

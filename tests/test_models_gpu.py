@@ -460,3 +460,14 @@ def test_generate_forced_tokens(cuda):
     assert row.count(1926) >= 5 and 1925 in row
     i = row.index(1925)
     assert row[1:i].count(1926) == 5 and row[i + 2] == 1927
+
+
+def test_empty_batch(cuda):
+    """B = 0 gives empty outputs (what the reference's torch modules do), for the board forward and the token forward."""
+    m = models.BT4Class(2, 256, 384, 8)
+    pol, wdl = m(torch.zeros(0, 8, 8, 19, device=cuda))
+    assert pol.shape == (0, 1858) and wdl.shape == (0, 3)
+    g = models.GPT(models.GPTConfig(block_size=256, vocab_size=1929, n_layer=2, n_head=8, n_embd=256))
+    logits, loss, _ = g.forward((torch.zeros(0, 8, 8, 19, device=cuda), torch.zeros(0, 3, dtype=torch.int64, device=cuda)))
+    assert logits.shape == (0, 1, 1929) and loss is None
+    assert m.evaluate_fens([], T=1.0)[0].shape == (0, 1858)
