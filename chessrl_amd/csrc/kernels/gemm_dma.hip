@@ -29,7 +29,8 @@ struct DmaCfgT {
   static constexpr int LOADS = 64 / ROWS_PER_INSTR;   // wave-instructions per wave and stage (64 rows each)
   static constexpr int STAGE_BYTES = (BM + BN) * ROWB;
   static constexpr int EPI_BYTES = NW * 32 * WN * 4;
-  static constexpr int LDS_BYTES = NSTAGE * STAGE_BYTES > EPI_BYTES ? NSTAGE * STAGE_BYTES : EPI_BYTES;
+  static constexpr int RING_BYTES = NSTAGE * STAGE_BYTES > EPI_BYTES ? NSTAGE * STAGE_BYTES : EPI_BYTES;
+  static constexpr int LDS_BYTES = RING_BYTES + 256;   // + the landing strip of the L2 prefetch loads
 };
 typedef DmaCfgT<128, 2> DmaCfg2;     // 128-byte rows, 2 stages (one in flight), half as many barriers
 
@@ -44,7 +45,7 @@ __device__ __forceinline__ void wait_vmcnt() {
 }
 
 template <typename Cfg, int IN_DT, int OUT_DT>
-__global__ void __launch_bounds__(Cfg::NT, 2) gemm_dma_kernel(const GemmArgs a, const uint8_t* zeros) {
+__global__ void __launch_bounds__(Cfg::NT, 2) gemm_dma_kernel(const GemmArgs a, const uint8_t* zeros, const int pf) {
   constexpr int BM = Cfg::BM, BN = Cfg::BN, TM = Cfg::TM, TN = Cfg::TN, NSTAGE = Cfg::NSTAGE, LOADS = Cfg::LOADS;
   constexpr int ESZ = (IN_DT == DT_FP8) ? 1 : 2;
   constexpr int KSTEPS = Cfg::ROWB / ((IN_DT == DT_FP8) ? 64 : 32);  // MFMA k-steps per stage
@@ -61,17 +62,25 @@ __global__ void __launch_bounds__(Cfg::NT, 2) gemm_dma_kernel(const GemmArgs a, 
     const int per = nblk >> 3;
     if (pid < (per << 3)) pid = (pid & 7) * per + (pid >> 3);
   }
-  // Inside an XCD's range the tiles are walked in groups of 8 x 4 (M x N), so the 32 workgroups resident on the
-  // XCD share 8 activation tiles and 4 weight tiles (3 MB of operands at K = 1024 bytes, inside its 4 MB L2).
+  // Inside an XCD's range the tiles are walked in groups of 8 x w (M x N), w = 4 where the tile columns divide by
+  // four and 3 or 4 otherwise (13 columns: 4+3+3+3), so the 32 workgroups resident on the XCD share 8 activation
+  // tiles and about 4 weight tiles (3 MB of operands at K = 1024 bytes, inside its 4 MB L2). Eight tile rows are
+  // walked column group by column group before the next eight rows.
   int tile_m = pid / tiles_n, tile_n = pid - tile_m * tiles_n;
+  int grp_w = 4, grp_q = tile_n & 3;   // width of this tile's column group and its place in it
   {
-    constexpr int GM = 8, GN = 4;
+    constexpr int GM = 8;
     const int tiles_m = (a.M + BM - 1) / BM;
-    if (tiles_m % GM == 0 && tiles_n % GN == 0) {
+    if (tiles_m % GM == 0) {
+      const int ngrp = (tiles_n + 3) >> 2, wb = tiles_n / ngrp, extra = tiles_n - wb * ngrp;
       const int sr = pid / (GM * tiles_n), rem = pid - sr * (GM * tiles_n);
-      const int ng = rem / (GM * GN), r2 = rem - ng * (GM * GN);
-      tile_m = sr * GM + r2 / GN;
-      tile_n = ng * GN + r2 % GN;
+      const int big = GM * (wb + 1) * extra;   // tiles of the `extra` groups that are one column wider
+      int gi, r2;
+      if (rem < big) { grp_w = wb + 1; gi = rem / (GM * grp_w); r2 = rem - gi * GM * grp_w; }
+      else { grp_w = wb; const int rem2 = rem - big; gi = rem2 / (GM * wb); r2 = rem2 - gi * GM * wb; gi += extra; }
+      grp_q = r2 % grp_w;
+      tile_m = sr * GM + r2 / grp_w;
+      tile_n = gi * wb + (gi < extra ? gi : extra) + grp_q;
     }
   }
   const int m0 = tile_m * BM, n0 = tile_n * BN;
@@ -109,6 +118,39 @@ __global__ void __launch_bounds__(Cfg::NT, 2) gemm_dma_kernel(const GemmArgs a, 
       const uint8_t* src = (kb + kchunk[j] <= kmax) ? gptr[j] + kb : zeros;
       __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)src,
                                        (__attribute__((address_space(3))) void*)(st + j * 1024), 16, 0, 0);
+    }
+  };
+
+  // L2 prefetch. The workgroups resident on an XCD walk K in step, so the 4-8 readers of an operand line ask for it
+  // at the same moment and all of them wait out the one fetch from memory. Each reader therefore touches its share of
+  // the lines of a slab `pf` slabs before any of them loads it: one dword per 128-byte line, landed in an LDS strip
+  // nobody reads. Wave 0 takes 64 of the 256 activation rows (the quarter chosen by the tile's column), wave 1 32 of
+  // the 256 weight rows (the eighth chosen by the tile's row; its upper lanes touch the second half-line).
+  const uint8_t* pf_ptr = nullptr;
+  int pf_n = 0, pf_step = 0;   // wave-instructions per slab and the byte distance between their rows
+  if (pf > 0 && wave < 2) {
+    if (wave == 0) {
+      pf_n = (4 + grp_w - 1) / grp_w;
+      int gm = m0 + ((grp_q * pf_n) & 3) * 64 + lane;
+      gm = gm < a.M ? gm : a.M - 1;
+      pf_ptr = reinterpret_cast<const uint8_t*>(a.A) + (long)gm * a.lda * ESZ;
+      pf_step = (m0 + 256 <= a.M) ? 64 * a.lda * ESZ : 0;
+    } else {
+      pf_n = 1;
+      int gn = n0 + (tile_m & 7) * 32 + (lane & 31);
+      gn = gn < a.N ? gn : a.N - 1;
+      pf_ptr = reinterpret_cast<const uint8_t*>(a.W) + (long)gn * a.ldw * ESZ + (lane >> 5) * 64;
+    }
+  }
+  auto prefetch = [&](int slab) {
+    if (pf_ptr && slab < nslab) {
+      const long kb = (long)slab * Cfg::ROWB;
+      const bool inside = kb + 64 + 4 <= kbytes;
+      for (int i = 0; i < pf_n; ++i) {
+        const uint8_t* src = inside ? pf_ptr + kb + (long)i * pf_step : zeros;
+        __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)src,
+                                         (__attribute__((address_space(3))) void*)(smem + Cfg::RING_BYTES), 4, 0, 0);
+      }
     }
   };
 
@@ -164,6 +206,7 @@ __global__ void __launch_bounds__(Cfg::NT, 2) gemm_dma_kernel(const GemmArgs a, 
 #pragma unroll
   for (int s0 = 0; s0 < NSTAGE - 1; ++s0)
     if (s0 < nslab) issue(s0);
+  for (int s0 = NSTAGE - 1; s0 < NSTAGE - 1 + pf; ++s0) prefetch(s0);
 
   for (int slab = 0; slab < nslab; ++slab) {
     // Loads still allowed in flight behind this slab's: LOADS per later slab already issued.
@@ -173,6 +216,7 @@ __global__ void __launch_bounds__(Cfg::NT, 2) gemm_dma_kernel(const GemmArgs a, 
     else wait_vmcnt<0>();
     __syncthreads();
     if (slab + NSTAGE - 1 < nslab) issue(slab + NSTAGE - 1);
+    prefetch(slab + NSTAGE - 1 + pf);
     const uint8_t* st = smem + (slab % NSTAGE) * Cfg::STAGE_BYTES;
     if (!wave_active) continue;
 #pragma unroll
@@ -226,7 +270,12 @@ static hipError_t launch_dma(const GemmArgs& a, hipStream_t st) {
     attr_set[dev] = true;
   }
   const int tiles = ((a.M + DCfg::BM - 1) / DCfg::BM) * ((a.N + DCfg::BN - 1) / DCfg::BN);
-  hipLaunchKernelGGL(kern, dim3(tiles), dim3(DCfg::NT), DCfg::LDS_BYTES, st, a, zeros);
+  // The L2 prefetch pays where the column groups are exactly four tiles wide and K is long enough to run ahead of
+  // (measured: 3-4 % at N = 1024, K = 1024 and 1536 bytes; nothing or a small loss at 6 and 13 tile columns and at K = 256).
+  const int tiles_n = (a.N + DCfg::BN - 1) / DCfg::BN;
+  const long kbytes = (long)a.K * (IN_DT == DT_FP8 ? 1 : 2);
+  const int pf = (tiles_n % 4 == 0 && kbytes >= 8 * DCfg::ROWB) ? 2 : 0;
+  hipLaunchKernelGGL(kern, dim3(tiles), dim3(DCfg::NT), DCfg::LDS_BYTES, st, a, zeros, pf);
   return hipGetLastError();
 }
 
