@@ -471,3 +471,34 @@ def test_empty_batch(cuda):
     logits, loss, _ = g.forward((torch.zeros(0, 8, 8, 19, device=cuda), torch.zeros(0, 3, dtype=torch.int64, device=cuda)))
     assert logits.shape == (0, 1, 1929) and loss is None
     assert m.evaluate_fens([], T=1.0)[0].shape == (0, 1858)
+
+
+def test_gpt_fp8_vs_emulation(cuda):
+    """The reference's own fp8 model is the GPT of model_fp8.py (te.Linear at :43,45,90,92, high-precision LayerNorm,
+    attention and residual stream): the HIP fp8 path against the quantise->dequantise oracle with the same static scales."""
+    L, H, Cm = 3, 8, 256
+    oracle = om.test_init_(om.GPTOracle(L, H, Cm), seed=11)
+    calib, _ = positions(64, seed=5)
+    planes, mask = positions(64, seed=6)
+    plan = om.Fp8Plan(L)
+    plan.recording = True
+    oracle.forward_last(calib, plan)
+    plan.recording = False
+    ref8 = oracle.forward_last(planes, plan)
+    ref32 = oracle.forward_last(planes)
+    m = models.GPT(models.GPTConfig(block_size=256, vocab_size=1929, n_layer=L, n_head=H, n_embd=Cm), fp8=True)
+    m.load_state_dict(oracle.state_dict())
+    m.calibrate(calib.to(cuda))
+    own = m._engine.get_amax()[:, :4]
+    want = plan.amax.numpy()[:, :4]
+    print("gpt amax rel diff (own calibration vs oracle fp32):", np.abs(own / want - 1).max())
+    assert np.abs(own / want - 1).max() < 0.05
+    full = m._engine.get_amax()
+    full[:, :4] = want
+    m._engine.set_amax(full)
+    pol = m.forward((planes.to(cuda), None))[0][:, 0].cpu()
+    report("gpt fp8 vs fp8-emulation", pol, ref8, mask)
+    report("gpt fp8 vs fp32", pol, ref32, mask)
+    report("fp8-emulation vs fp32 (oracle only)", ref8, ref32, mask)
+    assert rel_rms(pol, ref8) < 5e-2
+    assert rel_rms(pol, ref32) < 2 * rel_rms(ref8, ref32) + 1e-2
