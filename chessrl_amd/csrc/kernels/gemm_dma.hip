@@ -110,6 +110,13 @@ __global__ void __launch_bounds__(Cfg::NT, 2) gemm_dma_kernel(const GemmArgs a, 
     }
   }
   const int lds_row0 = (loads_a ? BN : 0) + rbase;  // first stage row this wave fills
+  auto issue_one = [&](int slab, int j) {
+    uint8_t* st = smem + (slab % NSTAGE) * Cfg::STAGE_BYTES + lds_row0 * Cfg::ROWB;
+    const long kb = (long)slab * Cfg::ROWB;
+    const uint8_t* src = (kb + kchunk[j] <= kmax) ? gptr[j] + kb : zeros;
+    __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)src,
+                                     (__attribute__((address_space(3))) void*)(st + j * 1024), 16, 0, 0);
+  };
   auto issue = [&](int slab) {
     uint8_t* st = smem + (slab % NSTAGE) * Cfg::STAGE_BYTES + lds_row0 * Cfg::ROWB;
     const long kb = (long)slab * Cfg::ROWB;
@@ -215,10 +222,13 @@ __global__ void __launch_bounds__(Cfg::NT, 2) gemm_dma_kernel(const GemmArgs a, 
     else if (NSTAGE >= 3 && ahead == 1) wait_vmcnt<LOADS>();
     else wait_vmcnt<0>();
     __syncthreads();
-    if (slab + NSTAGE - 1 < nslab) issue(slab + NSTAGE - 1);
+    const bool more = slab + NSTAGE - 1 < nslab;
     prefetch(slab + NSTAGE - 1 + pf);
     const uint8_t* st = smem + (slab % NSTAGE) * Cfg::STAGE_BYTES;
-    if (!wave_active) continue;
+    if (!wave_active) {   // no MFMAs to put the loads between
+      if (more) issue(slab + NSTAGE - 1);
+      continue;
+    }
 #pragma unroll
     for (int ks = 0; ks < KSTEPS; ++ks) {
       Frag<IN_DT> wf[TN], xf[TM];
@@ -226,7 +236,22 @@ __global__ void __launch_bounds__(Cfg::NT, 2) gemm_dma_kernel(const GemmArgs a, 
 #pragma unroll
       for (int tn = 0; tn < TN; ++tn)
 #pragma unroll
-        for (int tm = 0; tm < TM; ++tm) acc[tn][tm] = mfma_frag<IN_DT>(wf[tn], xf[tm], acc[tn][tm]);
+        for (int tm = 0; tm < TM; ++tm) {
+          acc[tn][tm] = mfma_frag<IN_DT>(wf[tn], xf[tm], acc[tn][tm]);
+          // The next slab's loads go out one at a time between the MFMAs (every second MFMA for fp8, every fourth for
+          // 16-bit elements), held in place by scheduling barriers, instead of eight in a row behind the barrier: a
+          // wave stalls at a load until the memory pipeline takes it, and spread out those stalls fall under MFMAs that
+          // are already executing (measured 1-4 % per GEMM; the loads and the MFMAs still add up rather than overlap,
+          // as they do when either is halved: the launch is bound by the energy both spend, not by a pipeline).
+          const int i = tn * TM + tm;
+          constexpr int PER = (TN * TM * KSTEPS) / LOADS >= 1 ? (TN * TM * KSTEPS) / LOADS : 1;
+          if ((i % PER) == PER - 1) {
+            const int j = (ks * TN * TM + i) / PER;
+            __builtin_amdgcn_sched_barrier(0);
+            if (more && j < LOADS) issue_one(slab + NSTAGE - 1, j);
+            __builtin_amdgcn_sched_barrier(0);
+          }
+        }
     }
   }
 
