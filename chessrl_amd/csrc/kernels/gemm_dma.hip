@@ -241,8 +241,7 @@ __global__ void __launch_bounds__(Cfg::NT, 2) gemm_dma_kernel(const GemmArgs a, 
           // The next slab's loads go out one at a time between the MFMAs (every second MFMA for fp8, every fourth for
           // 16-bit elements), held in place by scheduling barriers, instead of eight in a row behind the barrier: a
           // wave stalls at a load until the memory pipeline takes it, and spread out those stalls fall under MFMAs that
-          // are already executing (measured 1-4 % per GEMM; the loads and the MFMAs still add up rather than overlap,
-          // as they do when either is halved: the launch is bound by the energy both spend, not by a pipeline).
+          // are already executing (measured 1-4 % per GEMM).
           const int i = tn * TM + tm;
           constexpr int PER = (TN * TM * KSTEPS) / LOADS >= 1 ? (TN * TM * KSTEPS) / LOADS : 1;
           if ((i % PER) == PER - 1) {
