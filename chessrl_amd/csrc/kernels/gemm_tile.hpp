@@ -74,6 +74,13 @@ __device__ __forceinline__ void wave_lds_fence() {
   __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
 }
 
+// 16 bytes read once (a residual row segment): loaded with the non-temporal hint so that it does not displace the
+// operand tiles the workgroups of an XCD share in L2.
+__device__ __forceinline__ uint4 nt_load16(const char* p) {
+  const i32x4_t v = __builtin_nontemporal_load(reinterpret_cast<const i32x4_t*>(p));
+  return make_uint4((uint32_t)v[0], (uint32_t)v[1], (uint32_t)v[2], (uint32_t)v[3]);
+}
+
 // NT: store with the non-temporal hint, so a streamed output does not evict the operands from L2.
 template <int OUT_DT, int NT = 0>
 __device__ __forceinline__ void store8(void* base, long off, const float v[8]) {
@@ -166,7 +173,7 @@ __device__ __forceinline__ void gemm_epilogue(const GemmArgs& a, f32x16_t (&acc)
         const long ro = rrow * a.ldr + n;
         if (res32) {
           const float* rp = reinterpret_cast<const float*>(a.res) + ro + 4 * half;
-          if (__builtin_expect(full, 1)) val = *reinterpret_cast<const uint4*>(res_base + rrow * res_stride + 16 * half);
+          if (__builtin_expect(full, 1)) val = nt_load16(res_base + rrow * res_stride + 16 * half);
           else {
             uint32_t w[4];
 #pragma unroll
@@ -175,7 +182,7 @@ __device__ __forceinline__ void gemm_epilogue(const GemmArgs& a, f32x16_t (&acc)
           }
         } else {
           const uint16_t* rp = reinterpret_cast<const uint16_t*>(a.res) + ro;
-          if (__builtin_expect(full, 1)) val = *reinterpret_cast<const uint4*>(res_base + rrow * res_stride);
+          if (__builtin_expect(full, 1)) val = nt_load16(res_base + rrow * res_stride);
           else {
             uint32_t h[8];
 #pragma unroll
