@@ -132,6 +132,10 @@ struct GemmArgs {
   // Optional LayerNorm over the N columns of the result, written to ln_out (only where gemm_folds_layernorm says so).
   const float* ln_gamma; const float* ln_beta; void* ln_out; long ln_ldo; int ln_out_dtype; float ln_eps;
   int k_parallel;     // 1: tile 0 may pick the K-sliced / K-grouped kernels, whose summation order over K differs from the tiled kernels'
+  // Optional: the residual is LayerNorm(res) rather than res, normalised on the fly from the row statistics
+  // res_stats [M,2] = (1/std, -mean/std) a LayerNorm launch left behind and that norm's gain and offset [N]
+  // (256x256 tile with a 16-bit residual only; see gemm_takes_res_norm).
+  const float* res_stats; const float* res_gamma; const float* res_beta;
 };
 
 struct LayerNormArgs {
@@ -145,6 +149,7 @@ struct LayerNormArgs {
   int rows, C;
   int in_dtype, out_dtype;
   float eps, fp8_scale;
+  float* stats;         // optional [rows, 2]: 1/std and -mean/std of every row
 };
 
 struct EmbedArgs {

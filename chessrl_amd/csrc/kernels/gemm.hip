@@ -51,7 +51,7 @@ struct GemmCfg {
   static_assert(WN >= 32 && WM >= 32, "wave tile too small");
 };
 
-template <typename Cfg, int IN_DT, int OUT_DT>
+template <typename Cfg, int IN_DT, int OUT_DT, int RES_NORM = 0>
 __global__ void __launch_bounds__(Cfg::NT_ALL, Cfg::MIN_WAVES) gemm_kernel(const GemmArgs a) {
   constexpr int BM = Cfg::BM, BN = Cfg::BN, TM = Cfg::TM, TN = Cfg::TN, KG = Cfg::KG;
   constexpr int ESZ = (IN_DT == DT_FP8) ? 1 : 2;
@@ -255,8 +255,9 @@ __global__ void __launch_bounds__(Cfg::NT_ALL, Cfg::MIN_WAVES) gemm_kernel(const
                                              m0 + wm * Cfg::WM, n0 + wn * Cfg::WN, lane);
     return;
   }
-  gemm_epilogue<Cfg::WM, Cfg::WN, OUT_DT>(a, acc, reinterpret_cast<float*>(smem) + wave * (32 * Cfg::WN),
-                                           m0 + wm * Cfg::WM, n0 + wn * Cfg::WN, lane);
+  gemm_epilogue<Cfg::WM, Cfg::WN, OUT_DT, RES_NORM>(a, acc, reinterpret_cast<float*>(smem) + wave * (32 * Cfg::WN),
+                                                     m0 + wm * Cfg::WM, n0 + wn * Cfg::WN, lane,
+                                                     reinterpret_cast<float*>(smem + Cfg::EPI_BYTES) + wave * (2 * Cfg::WM));
 }
 
 // ---- second pass of a K-sliced GEMM -------------------------------------------------------------
@@ -393,12 +394,26 @@ typedef GemmCfg<128, 128, 2, 2, 2, 0, 2> CfgMid;    // 4 waves, 64x64 per wave, 
 typedef GemmCfg<64, 64, 2, 2, 2, 0, 2> CfgSmall;    // 4 waves, 32x32 per wave
 typedef GemmCfg<64, 64, 2, 2, 2, 0, 2, 4> CfgSmallK4;   // the same tile walked by 4 groups of 4 waves, K slabs in turn
 
-template <typename Cfg, int IN_DT, int OUT_DT>
+template <typename Cfg, int IN_DT, int OUT_DT, int RES_NORM = 0>
 static hipError_t launch_cfg(const GemmArgs& a, hipStream_t st) {
+  if constexpr (!RES_NORM) {
+    if (a.res_stats) {
+      // The residual-normalising epilogue exists for the case that uses it (e4m3 operands, bf16 output and residual),
+      // on every tile size, so that a row's result does not depend on the tile its batch size selects.
+      if constexpr (IN_DT == DT_FP8 && OUT_DT == DT_BF16 && Cfg::KG == 1) {
+        if (!a.res || a.res_dtype != DT_BF16 || !a.res_gamma || a.res_rows > 0 || a.alpha == 0.f) return hipErrorInvalidValue;
+        return launch_cfg<Cfg, IN_DT, OUT_DT, 1>(a, st);
+      } else {
+        return hipErrorInvalidValue;
+      }
+    }
+  } else {
+    static_assert(Cfg::EPI_BYTES + Cfg::NW * 2 * Cfg::WM * 4 <= Cfg::LDS_BYTES, "row statistics need room behind the epilogue patches");
+  }
   static std::atomic<bool> attr_set[16] = {};
   int dev = 0;
   (void)hipGetDevice(&dev);
-  auto kern = gemm_kernel<Cfg, IN_DT, OUT_DT>;
+  auto kern = gemm_kernel<Cfg, IN_DT, OUT_DT, RES_NORM>;
   if (dev >= 0 && dev < 16 && !attr_set[dev]) {
     hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, Cfg::LDS_BYTES);
     if (e != hipSuccess) return e;
@@ -530,6 +545,7 @@ static hipError_t launch_in_out(const GemmArgs& a, int tile, hipStream_t st) {
       if (ks > 1) return launch_splitk<CfgSmallK4, IN_DT, OUT_DT>(a, ks, per, st);
     }
   }
+  if (a.res_stats && tile == 5) return hipErrorInvalidValue;   // the K-grouped tile has no residual-normalising form
   if (tile == 3) return launch_gemm_dma(a, IN_DT, OUT_DT, st);
   if (tile == 2) return launch_cfg<CfgMid, IN_DT, OUT_DT>(a, st);
   if (tile == 5) return launch_cfg<CfgSmallK4, IN_DT, OUT_DT>(a, st);

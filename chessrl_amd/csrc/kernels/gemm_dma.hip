@@ -30,7 +30,8 @@ struct DmaCfgT {
   static constexpr int STAGE_BYTES = (BM + BN) * ROWB;
   static constexpr int EPI_BYTES = NW * 32 * WN * 4;
   static constexpr int RING_BYTES = NSTAGE * STAGE_BYTES > EPI_BYTES ? NSTAGE * STAGE_BYTES : EPI_BYTES;
-  static constexpr int LDS_BYTES = RING_BYTES + 256;   // + the landing strip of the L2 prefetch loads
+  static constexpr int STATS_OFF = RING_BYTES + 256;   // behind the landing strip of the L2 prefetch loads
+  static constexpr int LDS_BYTES = STATS_OFF + NW * 2 * WM * 4;   // + row statistics of a residual normalised on the fly
 };
 typedef DmaCfgT<128, 2> DmaCfg2;     // 128-byte rows, 2 stages (one in flight), half as many barriers
 
@@ -44,7 +45,7 @@ __device__ __forceinline__ void wait_vmcnt() {
   __builtin_amdgcn_s_waitcnt((N & 0xF) | ((N >> 4) << 14) | (0x7 << 4) | (0xF << 8));
 }
 
-template <typename Cfg, int IN_DT, int OUT_DT>
+template <typename Cfg, int IN_DT, int OUT_DT, int RES_NORM = 0>
 __global__ void __launch_bounds__(Cfg::NT, 2) gemm_dma_kernel(const GemmArgs a, const uint8_t* zeros, const int pf) {
   constexpr int BM = Cfg::BM, BN = Cfg::BN, TM = Cfg::TM, TN = Cfg::TN, NSTAGE = Cfg::NSTAGE, LOADS = Cfg::LOADS;
   constexpr int ESZ = (IN_DT == DT_FP8) ? 1 : 2;
@@ -88,6 +89,16 @@ __global__ void __launch_bounds__(Cfg::NT, 2) gemm_dma_kernel(const GemmArgs a, 
   const long kbytes = (long)a.K * ESZ;
   const int nslab = (int)((kbytes + Cfg::ROWB - 1) / Cfg::ROWB);
   const long kmax = kbytes - 16;
+
+  if constexpr (RES_NORM != 0) {
+    // Statistics of this wave's 128 rows (two rows = 16 bytes per lane), requested before anything else and landed
+    // outside the ring: they are in LDS long before the epilogue asks for them.
+    static_assert(Cfg::WM == 128, "one 16-byte load per lane covers the wave's rows");
+    int m = m0 + wm * Cfg::WM + 2 * lane;
+    m = m + 1 < a.M ? m : 0;
+    __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(a.res_stats + 2 * (long)m),
+                                     (__attribute__((address_space(3))) void*)(smem + Cfg::STATS_OFF + wave * (2 * Cfg::WM * 4)), 16, 0, 0);
+  }
 
   // Loader role of this wave.
   const bool loads_a = wave >= 4;
@@ -256,8 +267,9 @@ __global__ void __launch_bounds__(Cfg::NT, 2) gemm_dma_kernel(const GemmArgs a, 
 
   __syncthreads();  // every wave is done with the ring before it becomes epilogue scratch
 
-  gemm_epilogue<Cfg::WM, Cfg::WN, OUT_DT>(a, acc, reinterpret_cast<float*>(smem) + wave * (32 * Cfg::WN),
-                                           m0 + wm * Cfg::WM, n0 + wn * Cfg::WN, lane);
+  gemm_epilogue<Cfg::WM, Cfg::WN, OUT_DT, RES_NORM>(a, acc, reinterpret_cast<float*>(smem) + wave * (32 * Cfg::WN),
+                                                     m0 + wm * Cfg::WM, n0 + wn * Cfg::WN, lane,
+                                                     reinterpret_cast<float*>(smem + Cfg::STATS_OFF) + wave * (2 * Cfg::WM));
 }
 
 // One 256-byte block of zeros per device: the source of K-tail chunks for the direct-to-LDS loads.
@@ -279,7 +291,7 @@ static const uint8_t* device_zeros(hipError_t* err) {
   return z[dev];
 }
 
-template <typename DCfg, int IN_DT, int OUT_DT>
+template <typename DCfg, int IN_DT, int OUT_DT, int RES_NORM = 0>
 static hipError_t launch_dma(const GemmArgs& a, hipStream_t st) {
   static std::atomic<bool> attr_set[16] = {};
   hipError_t e = hipSuccess;
@@ -287,7 +299,7 @@ static hipError_t launch_dma(const GemmArgs& a, hipStream_t st) {
   if (!zeros) return e;
   int dev = 0;
   (void)hipGetDevice(&dev);
-  auto kern = gemm_dma_kernel<DCfg, IN_DT, OUT_DT>;
+  auto kern = gemm_dma_kernel<DCfg, IN_DT, OUT_DT, RES_NORM>;
   if (!attr_set[dev]) {
     e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, DCfg::LDS_BYTES);
     if (e != hipSuccess) return e;
@@ -304,6 +316,12 @@ static hipError_t launch_dma(const GemmArgs& a, hipStream_t st) {
 }
 
 hipError_t launch_gemm_dma(const GemmArgs& a, int in_dt, int out_dt, hipStream_t st) {
+  if (a.res_stats) {
+    // The residual-normalising epilogue exists for the case that uses it: e4m3 operands, bf16 output and residual.
+    if (in_dt != DT_FP8 || out_dt != DT_BF16 || !a.res || a.res_dtype != DT_BF16 || !a.res_gamma || a.res_rows > 0 || a.alpha == 0.f || (a.M & 1))
+      return hipErrorInvalidValue;
+    return launch_dma<DmaCfg2, DT_FP8, DT_BF16, 2>(a, st);
+  }
 #define DMA_OUT(IN)                                                        \
   switch (out_dt) {                                                        \
     case DT_F32: return launch_dma<DmaCfg2, IN, DT_F32>(a, st);            \

@@ -128,8 +128,13 @@ __device__ __forceinline__ void store8(void* base, long off, const float v[8]) {
 // on where the code object happened to place them (instruction-cache misses at the jump targets), and 5 % slower than
 // this form at best. (A second, compile-time variant of the epilogue for tiles entirely inside C was tried on top:
 // two inlined copies push the 256x256 kernel into register spills.)
-template <int WM, int WN, int OUT_DT>
-__device__ __forceinline__ void gemm_epilogue(const GemmArgs& a, f32x16_t (&acc)[WN / 32][WM / 32], float* sC, int mw0, int nw0, int lane) {
+// RES_NORM: the 16-bit residual is normalised on the fly, LayerNorm(res) = (res * s0_m + s1_m) * gain_n + offset_n with
+// s0 = 1/std and s1 = -mean/std of row m, from the row statistics a.res_stats and the norm's gain and offset (the normalised tensor then never travels
+// through memory). sStats: 2*WM floats of LDS of this wave's own for its rows' statistics, filled here (RES_NORM 1)
+// or by the kernel before its main loop (RES_NORM 2).
+template <int WM, int WN, int OUT_DT, int RES_NORM = 0>
+__device__ __forceinline__ void gemm_epilogue(const GemmArgs& a, f32x16_t (&acc)[WN / 32][WM / 32], float* sC, int mw0, int nw0, int lane,
+                                              float* sStats = nullptr) {
   constexpr int TM = WM / 32, TN = WN / 32, CH4 = WN / 4, CP = WN / 8, RSTEP = 64 / CP, ITERS = 32 / RSTEP;
   const int lr = lane & 31, g = lane >> 5;
   const int ec = lane % CP, er = lane / CP;
@@ -148,6 +153,26 @@ __device__ __forceinline__ void gemm_epilogue(const GemmArgs& a, f32x16_t (&acc)
   const int res_dt = a.res_dtype;
   const float descale = a.descale, alpha = a.alpha;
   float local_amax = 0.f;
+  float gain8[8];
+  if constexpr (RES_NORM) {
+    // offset_n joins the bias (which is multiplied by alpha below); the statistics of this wave's rows go to LDS.
+    const float inv_alpha = 1.0f / alpha;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+      const bool ok = n + e < a.N;
+      gain8[e] = ok ? a.res_gamma[n + e] : 0.f;
+      if (a.res_beta && ok) bias8[e] += a.res_beta[n + e] * inv_alpha;
+    }
+    if constexpr (RES_NORM == 1) {   // (2: the kernel has staged them before its main loop)
+#pragma unroll
+      for (int r = lane; r < WM; r += 64) {
+        const int m = mw0 + r;
+        const float2 st = m < a.M ? *reinterpret_cast<const float2*>(a.res_stats + 2 * (long)m) : make_float2(0.f, 0.f);
+        *reinterpret_cast<float2*>(sStats + 2 * r) = st;
+      }
+      wave_lds_fence();
+    }
+  }
   // A lane keeps its 8 columns for every row, so which output (C or C2), the column inside it and the row stride are
   // fixed per lane: the vector paths address row m as base + m * stride.
   constexpr int OUT_SZ = OUT_DT == DT_F32 ? 4 : OUT_DT == DT_FP8 ? 1 : 2;
@@ -262,6 +287,18 @@ __device__ __forceinline__ void gemm_epilogue(const GemmArgs& a, f32x16_t (&acc)
 #pragma unroll
           for (int e = 0; e < 8; ++e)
             v[it][e] = fmaf(v[it][e], alpha, f16_bits_to_f32((uint16_t)((e & 1) ? (w[e >> 1] >> 16) : (w[e >> 1] & 0xffff))));
+        }
+      } else if constexpr (RES_NORM) {
+#pragma unroll
+        for (int it = 0; it < ITERS; ++it) {
+          const uint4 q = rraw[tm & 1][it];
+          const uint32_t w[4] = {q.x, q.y, q.z, q.w};
+          const float2 st = *reinterpret_cast<const float2*>(sStats + 2 * (tm * 32 + er + it * RSTEP));
+#pragma unroll
+          for (int e = 0; e < 8; ++e) {
+            const float r = __uint_as_float((e & 1) ? (w[e >> 1] & 0xffff0000u) : (w[e >> 1] << 16));
+            v[it][e] = fmaf(v[it][e], alpha, fmaf(r, st.x, st.y) * gain8[e]);
+          }
         }
       } else {
 #pragma unroll

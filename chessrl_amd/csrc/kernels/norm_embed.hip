@@ -64,7 +64,7 @@ __device__ __forceinline__ void store8_fp8(uint8_t* base, long off, const float 
 // Normalise the VPL*8 values a lane holds (columns col0(i) = (i*64+lane)*8) and write them.
 template <int VPL>
 __device__ __forceinline__ void ln_finish(float (&x)[VPL][8], int lane, int C, const float* gamma, const float* beta,
-                                           float eps, float (&y)[VPL][8]) {
+                                           float eps, float (&y)[VPL][8], float* stats = nullptr) {
   float s = 0.f;
 #pragma unroll
   for (int i = 0; i < VPL; ++i) {
@@ -83,6 +83,7 @@ __device__ __forceinline__ void ln_finish(float (&x)[VPL][8], int lane, int C, c
     }
   }
   const float rstd = rsqrtf(wave_sum(q) / (float)C + eps);
+  if (stats && lane == 0) *reinterpret_cast<float2*>(stats) = make_float2(rstd, -mean * rstd);   // (x - mean) * rstd = x * s0 + s1
 #pragma unroll
   for (int i = 0; i < VPL; ++i) {
     const int col = (i * 64 + lane) * 8;
@@ -107,7 +108,7 @@ __global__ void __launch_bounds__(256) layernorm_kernel(const LayerNormArgs a) {
     const int col = (i * 64 + lane) * 8;
     if (col < a.C) load8<IN_DT>(a.x, (long)row * a.ldx + col, x[i]);
   }
-  ln_finish<VPL>(x, lane, a.C, a.gamma, a.beta, a.eps, y);
+  ln_finish<VPL>(x, lane, a.C, a.gamma, a.beta, a.eps, y, a.stats ? a.stats + 2 * (long)row : nullptr);
   float am = 0.f;
 #pragma unroll
   for (int i = 0; i < VPL; ++i) {
@@ -203,6 +204,7 @@ static hipError_t launch_ln_dt(const LayerNormArgs& a, hipStream_t st) {
 hipError_t launch_layernorm(const LayerNormArgs& a, hipStream_t st) {
   if (a.rows <= 0) return hipSuccess;
   if (a.C % 8 || a.ldx % 8 || a.ldo % 8 || a.C > 8192) return hipErrorInvalidValue;
+  if (a.stats && a.C > 2048) return hipErrorInvalidValue;   // the four-waves-per-row kernel does not write them
   switch (a.in_dtype) {
     case DT_F32: return launch_ln_dt<DT_F32>(a, st);
     case DT_BF16: return launch_ln_dt<DT_BF16>(a, st);

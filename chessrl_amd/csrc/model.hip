@@ -330,6 +330,8 @@ int Model::ensure_ws(int mb) {
   WS(ws.f, M * F * 2);
   WS(ws.f8, M * F);
   WS(ws.stm, (size_t)mb);
+  WS(ws.st1, M * 2 * sizeof(float));
+  WS(ws.st2, M * 2 * sizeof(float));
   WS(ws.splitk, (size_t)Workspace::SPLITK_BYTES);
   if (cfg.arch == CRL_ARCH_BT4CLASS) {
     WS(ws.comp, M * cfg.smolgen_compress * 2);
@@ -396,6 +398,8 @@ struct GOpt {
   bool k_parallel = false;  // token steps of generation: few rows, so K is spread over more waves (different summation order)
   // LayerNorm that follows this GEMM, to be folded into it where the GEMM kernel can (*ln_folded says whether it did).
   const float* ln_g = nullptr; const float* ln_b = nullptr; void* ln_out = nullptr; int ln_dt = DT_BF16; bool* ln_folded = nullptr;
+  // The residual is LayerNorm(res), normalised in the epilogue from these row statistics, gain and offset.
+  const float* res_stats = nullptr; const float* res_g = nullptr; const float* res_b = nullptr;
 };
 
 int Model::gemm(const Lin& L, const void* A, long lda, int in_dt, void* C, long ldc, int out_dt, int M, const GOpt& o, hipStream_t st) {
@@ -407,6 +411,7 @@ int Model::gemm(const Lin& L, const void* A, long lda, int in_dt, void* C, long 
   g.C = C; g.ldc = ldc; g.C2 = o.C2; g.ldc2 = o.ldc2; g.nsplit = o.nsplit > 0 ? o.nsplit : L.N;
   g.bias = L.b; g.res = o.res; g.ldr = o.ldr; g.res_dtype = o.res_dt; g.res_rows = o.res_rows;
   g.amax = o.amax; g.M = M; g.N = L.N; g.K = L.K; g.act = o.act;
+  g.res_stats = o.res_stats; g.res_gamma = o.res_g; g.res_beta = o.res_b;
   g.descale = in_dt == DT_FP8 ? 1.f / (o.a_scale * L.wscale) : 1.f;
   g.alpha = o.alpha; g.out_scale = o.out_scale; g.k_parallel = o.k_parallel ? 1 : 0;
   g.splitk_ws = ws.splitk; g.splitk_ws_bytes = Workspace::SPLITK_BYTES;
@@ -427,11 +432,11 @@ int Model::gemm(const Lin& L, const void* A, long lda, int in_dt, void* C, long 
 }
 
 int Model::lnorm(const void* x, long ldx, int in_dt, const float* g, const float* b, void* out, int out_dt, uint8_t* out8,
-                 float scale8, long ldo, int rows, int C, float* amax, hipStream_t st) {
+                 float scale8, long ldo, int rows, int C, float* amax, hipStream_t st, float* stats) {
   LayerNormArgs a;
   std::memset(&a, 0, sizeof(a));
   a.x = x; a.ldx = ldx; a.in_dtype = in_dt; a.gamma = g; a.beta = b; a.out = out; a.out_dtype = out_dt;
-  a.out_fp8 = out8; a.fp8_scale = scale8; a.ldo = ldo; a.rows = rows; a.C = C; a.eps = cfg.eps; a.amax = amax;
+  a.out_fp8 = out8; a.fp8_scale = scale8; a.ldo = ldo; a.rows = rows; a.C = C; a.eps = cfg.eps; a.amax = amax; a.stats = stats;
   prof_begin(2, st);
   hipError_t e = launch_layernorm(a, st);
   prof_end(st);
@@ -517,6 +522,9 @@ int Model::forward_chunk(const float* planes, const uint8_t* ids, const uint8_t*
     HIPCHK(launch_extract_stm(planes, flags, ws.stm, mb, st));
   }
 
+  // BT4-class in e4m3 with bf16 activations: the normalised activations are not written in 16 bits at all (every
+  // tile size has the residual-normalising epilogue, so this does not depend on the batch).
+  const bool fold = ln_fold && f8 && cfg.arch == CRL_ARCH_BT4CLASS && ad == DT_BF16;
   const float attn_scale = cfg.arch == CRL_ARCH_BT4 ? 1.0f / std::sqrt((float)C) : 1.0f / std::sqrt((float)hs);
   const float alpha = cfg.arch == CRL_ARCH_BT4CLASS ? std::pow(2.0f * (float)L, -0.25f) : 1.0f;
 
@@ -581,10 +589,14 @@ int Model::forward_chunk(const float* planes, const uint8_t* ids, const uint8_t*
       { GOpt o; o.res = ws.x; o.ldr = C; o.res_dt = xdt; o.a_scale = f8 ? act_scale(l, 3) : 1.f;
         RUN(gemm(ly.ff2, f8 ? (const void*)ws.f8 : (const void*)ws.f, F, ao_dt, ws.x, C, xdt, M, o, st)); }
     } else {
-      // t = x + alpha*proj(ao);  h = LN1(t)
+      // t = x + alpha*proj(ao);  h = LN1(t). With `fold` the normalised tensors x and h exist only as e4m3 copies
+      // (the products' operands): the LayerNorm launches leave their row statistics behind, and the product that
+      // takes x or h as its residual re-normalises the un-normalised tensor t in its epilogue, writing in place.
       { GOpt o; o.res = ws.x; o.ldr = C; o.res_dt = ad; o.alpha = alpha; o.a_scale = f8 ? act_scale(l, 1) : 1.f;
+        if (fold && l > 0) { o.res = ws.t; o.res_stats = ws.st2; o.res_g = layers[l - 1].ln2_g; o.res_b = layers[l - 1].ln2_b; }
         RUN(gemm(ly.proj, ao_in, C, ao_dt, ws.t, C, ad, M, o, st)); }
-      RUN(lnorm(ws.t, C, ad, ly.ln1_g, ly.ln1_b, ws.h, ad, f8 ? ws.h8 : nullptr, f8 ? act_scale(l, 2) : 1.f, C, M, C, am(l, 2), st));
+      RUN(lnorm(ws.t, C, ad, ly.ln1_g, ly.ln1_b, fold ? nullptr : ws.h, ad, f8 ? ws.h8 : nullptr, f8 ? act_scale(l, 2) : 1.f, C, M, C, am(l, 2), st,
+                fold ? ws.st1 : nullptr));
       const void* h_in = f8 ? (const void*)ws.h8 : (const void*)ws.h;
       if (cfg.arch == CRL_ARCH_BT4) {
         // y = ff2(ff1(h)) with no activation in between; t = gelu(y) + h (new_paradigm/value.py:65-70)
@@ -596,11 +608,12 @@ int Model::forward_chunk(const float* planes, const uint8_t* ids, const uint8_t*
         { GOpt o; o.act = ACT_MISH; o.a_scale = f8 ? act_scale(l, 2) : 1.f; o.out_scale = f8 ? act_scale(l, 3) : 1.f; o.amax = am(l, 3);
           RUN(gemm(ly.ff1, h_in, C, ao_dt, f8 ? (void*)ws.f8 : (void*)ws.f, F, ao_dt, M, o, st)); }
         { GOpt o; o.res = ws.h; o.ldr = C; o.res_dt = ad; o.alpha = alpha; o.a_scale = f8 ? act_scale(l, 3) : 1.f;
+          if (fold) { o.res = ws.t; o.res_stats = ws.st1; o.res_g = ly.ln1_g; o.res_b = ly.ln1_b; }
           RUN(gemm(ly.ff2, f8 ? (const void*)ws.f8 : (const void*)ws.f, F, ao_dt, ws.t, C, ad, M, o, st)); }
       }
       // x = LN2(t); the last layer's output feeds only the heads.
-      RUN(lnorm(ws.t, C, ad, ly.ln2_g, ly.ln2_b, ws.x, last ? hd : ad, (f8 && !last) ? ws.x8 : nullptr,
-                (f8 && !last) ? act_scale(l + 1, 0) : 1.f, C, M, C, last ? nullptr : am(l + 1, 0), st));
+      RUN(lnorm(ws.t, C, ad, ly.ln2_g, ly.ln2_b, (fold && !last) ? nullptr : ws.x, last ? hd : ad, (f8 && !last) ? ws.x8 : nullptr,
+                (f8 && !last) ? act_scale(l + 1, 0) : 1.f, C, M, C, last ? nullptr : am(l + 1, 0), st, (fold && !last) ? ws.st2 : nullptr));
     }
   }
 

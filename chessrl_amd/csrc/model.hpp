@@ -35,6 +35,7 @@ struct Layer {
 struct Workspace {
   void *x = nullptr, *t = nullptr, *h = nullptr, *qkv = nullptr, *ao = nullptr, *f = nullptr;
   uint8_t *x8 = nullptr, *h8 = nullptr, *ao8 = nullptr, *f8 = nullptr, *stm = nullptr;
+  float *st1 = nullptr, *st2 = nullptr;   // row statistics (mean, 1/std) of a layer's two LayerNorms
   void *comp = nullptr, *sh1 = nullptr, *sh2 = nullptr, *sg1 = nullptr, *sg2 = nullptr, *bias = nullptr;
   uint8_t* sg2_8 = nullptr;
   void *hl = nullptr, *tok = nullptr, *pqk = nullptr, *v1 = nullptr, *v2 = nullptr, *dense = nullptr;
@@ -80,6 +81,7 @@ struct Model {
   bool decode_graph = false;
   bool kv_capture = false;     // forward_chunk copies every layer's keys|values into the cache
   bool force_16bit = false;    // forward_chunk ignores cfg.fp8
+  bool ln_fold = true;         // e4m3 BT4-class: normalised activations exist only as e4m3 copies (forward_chunk)
 
   struct ProfEvent { hipEvent_t a, b; int fam; };
   bool profiling = false;
@@ -116,7 +118,7 @@ struct Model {
                     float* all_logits, float* wdl, bool calibrate, hipStream_t st);
   int gemm(const Lin& L, const void* A, long lda, int in_dt, void* C, long ldc, int out_dt, int M, const GOpt& o, hipStream_t st);
   int lnorm(const void* x, long ldx, int in_dt, const float* g, const float* b, void* out, int out_dt, uint8_t* out8, float scale8,
-            long ldo, int rows, int C, float* amax, hipStream_t st);
+            long ldo, int rows, int C, float* amax, hipStream_t st, float* stats = nullptr);
   float act_scale(int layer, int slot) const;
   void prof_begin(int fam, hipStream_t st);
   void prof_end(hipStream_t st);
