@@ -17,6 +17,7 @@ SOURCES = [
     "host/chess.cpp",
     "kernels/gemm.hip",
     "kernels/gemm_dma.hip",
+    "kernels/gemm_dma_resnorm.hip",
     "kernels/norm_embed.hip",
     "kernels/attention.hip",
     "kernels/heads.hip",

@@ -74,8 +74,9 @@ __device__ __forceinline__ void wave_lds_fence() {
   __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
 }
 
-// 16 bytes read once (a residual row segment): loaded with the non-temporal hint so that it does not displace the
-// operand tiles the workgroups of an XCD share in L2.
+// 16 bytes read once (a 16-bit residual row segment): loaded with the non-temporal hint so that it does not displace
+// the operand tiles the workgroups of an XCD share in L2 (an fp32 residual stream measured 2 % slower with the hint
+// and keeps plain loads).
 __device__ __forceinline__ uint4 nt_load16(const char* p) {
   const i32x4_t v = __builtin_nontemporal_load(reinterpret_cast<const i32x4_t*>(p));
   return make_uint4((uint32_t)v[0], (uint32_t)v[1], (uint32_t)v[2], (uint32_t)v[3]);
@@ -198,7 +199,7 @@ __device__ __forceinline__ void gemm_epilogue(const GemmArgs& a, f32x16_t (&acc)
         const long ro = rrow * a.ldr + n;
         if (res32) {
           const float* rp = reinterpret_cast<const float*>(a.res) + ro + 4 * half;
-          if (__builtin_expect(full, 1)) val = nt_load16(res_base + rrow * res_stride + 16 * half);
+          if (__builtin_expect(full, 1)) val = *reinterpret_cast<const uint4*>(res_base + rrow * res_stride + 16 * half);
           else {
             uint32_t w[4];
 #pragma unroll
@@ -359,5 +360,6 @@ __device__ __forceinline__ void gemm_epilogue(const GemmArgs& a, f32x16_t (&acc)
 // own: its speed depends measurably on where its code lands (identical instructions ran 3-8 % slower after unrelated
 // kernels were added to the same code object), and alone it stays where it was measured.
 hipError_t launch_gemm_dma(const GemmArgs& a, int in_dt, int out_dt, hipStream_t st);
+hipError_t launch_gemm_dma_resnorm(const GemmArgs& a, hipStream_t st);   // gemm_dma_resnorm.hip
 
 }  // namespace crl
