@@ -165,7 +165,9 @@ def test_gemm_f16_inputs_and_broadcast_residual(cuda):
     assert torch.allclose(out.float(), ref, rtol=2 ** -10, atol=2 ** -8)
 
 
-@pytest.mark.parametrize("M,N,K,tile", [(256, 256, 256, 3), (512, 1536, 1024, 0), (200, 1024, 1536, 2), (64, 3104, 1024, 1), (64, 3104, 1024, 5), (200, 1024, 1072, 5), (4096, 1024, 1024, 3), (4096, 1536, 1024, 3), (1000, 3104, 1072, 3), (8192, 1536, 1024, 3), (20000, 1024, 1536, 3)])
+@pytest.mark.parametrize("M,N,K,tile", [(256, 256, 256, 3), (512, 1536, 1024, 0), (200, 1024, 1536, 2), (64, 3104, 1024, 1), (64, 3104, 1024, 5), (200, 1024, 1072, 5), (4096, 1024, 1024, 3), (4096, 1536, 1024, 3), (1000, 3104, 1072, 3), (8192, 1536, 1024, 3), (20000, 1024, 1536, 3),
+    # eight tile rows (the grouped tile order) with 13, 1, 6 and 7 tile columns, the last with a K tail
+    (2048, 3104, 1024, 3), (2048, 200, 512, 3), (4096, 1300, 640, 3), (2048, 1700, 1040, 3)])
 def test_gemm_fp8(cuda, M, N, K, tile):
     torch.manual_seed(N)
     x = torch.randn(M, K, device=cuda)
