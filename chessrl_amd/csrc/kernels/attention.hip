@@ -319,20 +319,40 @@ __global__ void __launch_bounds__(64 * AttnWaves<MODE>::N, (AttnMinWaves<HS, MOD
 #pragma unroll
     for (int dt = 0; dt < DT_TILES; ++dt)
 #pragma unroll
-      for (int rq = 0; rq < 4; ++rq) {
-        const int d = 32 * dt + 8 * rq + 4 * g;
-        float v[4];
+      for (int rp = 0; rp < 2; ++rp) {
+        // A lane holds dims 8rq + 4g .. +3 of its row for rq = 0..3; the lane 32 away holds the other four of each
+        // group of eight. The two swap one half per pair of groups, so each stores 8 consecutive dims of the row
+        // (8 bytes of e4m3 or 16 bytes of 16-bit elements) and a row receives 16 or 32 contiguous bytes per instruction.
+        uint32_t pk[2][2];   // [rq - 2rp][word]: e4m3 uses word 0 only
 #pragma unroll
-        for (int e = 0; e < 4; ++e) {
-          v[e] = o[dt][it][4 * rq + e] * inv_l[it];
-          am = fmaxf(am, fabsf(v[e]));
+        for (int q2 = 0; q2 < 2; ++q2) {
+          const int rq = 2 * rp + q2;
+          float v[4];
+#pragma unroll
+          for (int e = 0; e < 4; ++e) {
+            v[e] = o[dt][it][4 * rq + e] * inv_l[it];
+            am = fmaxf(am, fabsf(v[e]));
+          }
+          if constexpr (OUT_FP8) {
+            pk[q2][0] = pack_fp8x4(v[0] * a.out_scale, v[1] * a.out_scale, v[2] * a.out_scale, v[3] * a.out_scale);
+            pk[q2][1] = 0;
+          } else {
+            pk[q2][0] = H16::pack2(v[0], v[1]);
+            pk[q2][1] = H16::pack2(v[2], v[3]);
+          }
         }
+        // g = 0 keeps group 2rp and receives the partner's half of it; g = 1 keeps group 2rp+1.
+        const int keep = g, give = 1 - g;
+        const uint32_t r0 = __shfl_xor(pk[give][0], 32, 64);
+        const int d = 32 * dt + 16 * rp + 8 * g;
         const long off = row * a.ldo + h * HS + d;
         if constexpr (OUT_FP8) {
-          *reinterpret_cast<uint32_t*>(reinterpret_cast<uint8_t*>(a.out) + off) =
-              pack_fp8x4(v[0] * a.out_scale, v[1] * a.out_scale, v[2] * a.out_scale, v[3] * a.out_scale);
+          const uint2 w = g ? make_uint2(r0, pk[keep][0]) : make_uint2(pk[keep][0], r0);
+          *reinterpret_cast<uint2*>(reinterpret_cast<uint8_t*>(a.out) + off) = w;
         } else {
-          *reinterpret_cast<uint2*>(reinterpret_cast<uint16_t*>(a.out) + off) = make_uint2(H16::pack2(v[0], v[1]), H16::pack2(v[2], v[3]));
+          const uint32_t r1 = __shfl_xor(pk[give][1], 32, 64);
+          const uint4 w = g ? make_uint4(r0, r1, pk[keep][0], pk[keep][1]) : make_uint4(pk[keep][0], pk[keep][1], r0, r1);
+          *reinterpret_cast<uint4*>(reinterpret_cast<uint16_t*>(a.out) + off) = w;
         }
       }
   }
