@@ -20,7 +20,7 @@ class ModelConfig(C.Structure):
         ("arch", C.c_int32), ("n_layer", C.c_int32), ("d_model", C.c_int32), ("n_head", C.c_int32),
         ("d_ff", C.c_int32), ("fp8", C.c_int32), ("micro_batch", C.c_int32), ("stream_f32", C.c_int32),
         ("head_dtype", C.c_int32), ("smolgen_compress", C.c_int32), ("smolgen_hidden", C.c_int32),
-        ("smolgen_gen", C.c_int32), ("eps", C.c_float), ("act_dtype", C.c_int32), ("reserved", C.c_int32 * 3),
+        ("smolgen_gen", C.c_int32), ("eps", C.c_float), ("act_dtype", C.c_int32), ("ln_fold", C.c_int32), ("norm_rms", C.c_int32), ("fp8_lm_head", C.c_int32),
     ]
 
 
@@ -51,7 +51,9 @@ SIGNATURES = {
     "crl_perft": (C.c_uint64, [_cp, _i]),
     "crl_random_positions": (_i, [C.c_uint64, _i, _i, C.c_double, _i, _vp, _vp, _vp, _vp]),
     "crl_gemm": (_i, [_vp, _i64, _vp, _i64, _vp, _i64, _i, _i, _i, _i, _i, _vp, _i, _f, _f, _vp, _i64, _i, _f, _vp, _i, _vp]),
+    "crl_shutdown": (None, []),
     "crl_layernorm": (_i, [_vp, _i64, _i, _vp, _vp, _vp, _i, _vp, _f, _i64, _i, _i, _f, _vp, _vp]),
+    "crl_rmsnorm": (_i, [_vp, _i64, _i, _vp, _vp, _i, _vp, _f, _i64, _i, _i, _f, _vp, _vp]),
     "crl_attention": (_i, [_vp, _i64, _vp, _i64, _vp, _i64, _i, _vp, _i64, _i, _f, _i, _i, _i, _i, _f, _vp, _vp, _vp, _vp, _vp, _vp]),
     "crl_attn_bias_slot": (_i, [_i, _i]),
     "crl_masked_softmax": (_i, [_vp, _i64, _vp, _i64, _vp, _i64, _vp, _i, _i, _f, _vp]),

@@ -52,6 +52,9 @@ int parse(const char* fen, Board& b) {
   return 0;
 }
 
+// Inverse move maps of crl_leela_to_rl on the device, one copy per device; crl_shutdown frees them.
+int32_t* g_inv_dev[16] = {};
+
 void put_str(char* dst, size_t cap, const std::string& s) {
   std::memset(dst, 0, cap);
   std::memcpy(dst, s.data(), std::min(cap - 1, s.size()));
@@ -62,7 +65,20 @@ void put_str(char* dst, size_t cap, const std::string& s) {
 extern "C" {
 
 const char* crl_last_error(void) { return get_error(); }
-const char* crl_version(void) { return "chessrl_amd 0.1 (gfx950)"; }
+const char* crl_version(void) { return "chessrl_amd 0.2 (gfx950)"; }
+
+void crl_shutdown(void) {
+  release_gemm_globals();
+  int cur = 0;
+  const bool have_dev = hipGetDevice(&cur) == hipSuccess;
+  for (int d = 0; d < 16; ++d)
+    if (g_inv_dev[d]) {
+      if (have_dev) (void)hipSetDevice(d);
+      (void)hipFree(g_inv_dev[d]);
+      g_inv_dev[d] = nullptr;
+    }
+  if (have_dev) (void)hipSetDevice(cur);
+}
 
 const char* crl_policy_index(int i) {
   const auto& v = policy_index();
@@ -219,6 +235,18 @@ int crl_layernorm(const void* x, int64_t ldx, int in_dtype, const float* gamma, 
   return e == hipSuccess ? CRL_OK : hip_fail("crl_layernorm", e);
 }
 
+int crl_rmsnorm(const void* x, int64_t ldx, int in_dtype, const float* gamma, void* out, int out_dtype, uint8_t* out_fp8, float fp8_scale,
+                int64_t ldo, int rows, int C, float eps, float* amax, void* stream) {
+  if (!x || !gamma || (!out && !out_fp8) || rows < 0) return arg_fail("crl_rmsnorm: bad arguments");
+  LayerNormArgs a;
+  std::memset(&a, 0, sizeof(a));
+  a.x = x; a.ldx = ldx; a.in_dtype = in_dtype; a.gamma = gamma; a.out = out; a.out_dtype = out_dtype;
+  a.out_fp8 = out_fp8; a.fp8_scale = fp8_scale; a.ldo = ldo; a.rows = rows; a.C = C; a.eps = eps; a.amax = amax; a.rms = 1;
+  hipError_t e = launch_layernorm(a, (hipStream_t)stream);
+  if (e == hipErrorInvalidValue) return arg_fail("crl_rmsnorm: C and strides must be multiples of 8 and C <= 8192");
+  return e == hipSuccess ? CRL_OK : hip_fail("crl_rmsnorm", e);
+}
+
 int crl_attention(const void* q, int64_t ldq, const void* k, int64_t ldk, const void* v, int64_t ldv, int in_dtype, void* out, int64_t ldo,
                   int out_dtype, float out_scale, int B, int H, int head_dim, int mode, float scale, const void* bias,
                   const void* pos, const float* u_bias, const float* v_bias, float* amax, void* stream) {
@@ -253,7 +281,7 @@ int crl_masked_softmax(const float* logits, int64_t ldl, const uint8_t* mask, in
 int crl_leela_to_rl(const float* src, int64_t lds, float* dst, int64_t ldd, const uint8_t* white_to_move, int B, void* stream) {
   if (!src || !dst || !white_to_move || B < 0) return arg_fail("crl_leela_to_rl: bad arguments");
   // Inverse maps live on the device for the lifetime of the process, one copy per device.
-  static int32_t* inv_dev[16] = {};
+  int32_t** inv_dev = g_inv_dev;
   int dev = 0;
   hipError_t e = hipGetDevice(&dev);
   if (e != hipSuccess) return hip_fail("hipGetDevice", e);
@@ -423,12 +451,16 @@ int crl_model_calibrate(crl_model* m, const float* planes, int B, void* stream) 
   return m->impl.calibrate(planes, B, (hipStream_t)stream);
 }
 int crl_model_get_amax(crl_model* m, float* out, int n) {
-  if (!m || !out || n != (int)m->impl.amax_host.size()) return arg_fail("crl_model_get_amax: n must be n_layer*5");
+  if (!m) return arg_fail("crl_model_get_amax: null model");
+  const int full = (int)m->impl.amax_host.size();   // (n_layer + 1) * 5
+  if (!m || !out || (n != full && n != full - Model::AMAX_SLOTS)) return arg_fail("crl_model_get_amax: n must be n_layer*5 or (n_layer+1)*5");
   std::memcpy(out, m->impl.amax_host.data(), sizeof(float) * n);
   return CRL_OK;
 }
 int crl_model_set_amax(crl_model* m, const float* in, int n) {
-  if (!m || !in || n != (int)m->impl.amax_host.size()) return arg_fail("crl_model_set_amax: n must be n_layer*5");
+  if (!m) return arg_fail("crl_model_set_amax: null model");
+  const int full = (int)m->impl.amax_host.size();
+  if (!m || !in || (n != full && n != full - Model::AMAX_SLOTS)) return arg_fail("crl_model_set_amax: n must be n_layer*5 or (n_layer+1)*5");
   std::memcpy(m->impl.amax_host.data(), in, sizeof(float) * n);
   return CRL_OK;
 }
@@ -468,7 +500,13 @@ static int evaluate_boards(crl_model* m, int n, int chunk, float temperature, fl
   if (n == 0) return CRL_OK;
   if (chunk > n) chunk = n;
   FenPipeline& P = m->pipe;
-  hipError_t e = P.ensure(chunk, V);
+  // The pipeline runs on streams of its own and shares the model's workspace with every other entry point: work a
+  // caller has queued on this model through crl_model_forward (on any stream) must have finished before the first
+  // chunk starts, and the workspace may be re-allocated below. Nothing here knows the caller's streams, so wait for
+  // the device.
+  hipError_t e = hipDeviceSynchronize();
+  if (e != hipSuccess) return hip_fail("evaluate: waiting for earlier work on the device", e);
+  e = P.ensure(chunk, V);
   if (e != hipSuccess) return hip_fail("evaluate: staging buffers", e);
   // Results of a finished slot go from pinned staging to the caller's arrays.
   auto drain = [&](FenPipeline::Slot& s) -> hipError_t {

@@ -131,6 +131,7 @@ struct GemmArgs {
   long splitk_ws_bytes;
   // Optional LayerNorm over the N columns of the result, written to ln_out (only where gemm_folds_layernorm says so).
   const float* ln_gamma; const float* ln_beta; void* ln_out; long ln_ldo; int ln_out_dtype; float ln_eps;
+  int ln_rms;         // the folded norm is an RMSNorm (no mean subtraction, no offset)
   int k_parallel;     // 1: tile 0 may pick the K-sliced / K-grouped kernels, whose summation order over K differs from the tiled kernels'
   // Optional: the residual is LayerNorm(res) rather than res, normalised on the fly from the row statistics
   // res_stats [M,2] = (1/std, -mean/std) a LayerNorm launch left behind and that norm's gain and offset [N]
@@ -150,6 +151,9 @@ struct LayerNormArgs {
   int in_dtype, out_dtype;
   float eps, fp8_scale;
   float* stats;         // optional [rows, 2]: 1/std and -mean/std of every row
+  void* out_b;          // optional second copy [rows, C] in out_b_dtype (a 16-bit operand copy beside an fp32 residual copy)
+  int out_b_dtype;
+  int rms;              // 1: RMSNorm, y = x / sqrt(mean(x^2) + eps) * gamma (no mean subtraction, beta ignored)
 };
 
 struct EmbedArgs {
@@ -164,6 +168,8 @@ struct EmbedArgs {
   const float* pe;          // optional [64, C] added after gating
   void* out;            // [B*64, C] in out_dtype
   uint8_t* out_fp8;     // optional
+  void* out_b;          // optional second copy in out_b_dtype
+  int out_b_dtype;
   float* amax;
   int tokens, C, out_dtype, act;
   float eps, fp8_scale;
@@ -268,6 +274,8 @@ hipError_t launch_gemm(GemmArgs a, int in_dt, int out_dt, int tile, hipStream_t 
 // True when launch_gemm (tile 0) would take the K-sliced path for these arguments, whose second pass can apply the
 // LayerNorm that follows the GEMM (GemmArgs::ln_*); launch_gemm rejects ln_out otherwise.
 bool gemm_folds_layernorm(const GemmArgs& a, int in_dt);
+// Frees the device memory the GEMM launchers keep outside any model (per-stream K-slice workspaces, the zeros block).
+void release_gemm_globals();
 hipError_t launch_layernorm(const LayerNormArgs& a, hipStream_t st);
 hipError_t launch_embed(const EmbedArgs& a, hipStream_t st);
 hipError_t launch_token_embed(const TokenEmbedArgs& a, hipStream_t st);

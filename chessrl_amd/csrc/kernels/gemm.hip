@@ -346,7 +346,8 @@ __global__ void __launch_bounds__(256) splitk_reduce_ln_kernel(const GemmArgs a,
   s = wave_sum(s);
   if (lane == 0) s_red[0][wave] = s;
   __syncthreads();
-  const float mean = (((s_red[0][0] + s_red[0][1]) + s_red[0][2]) + s_red[0][3]) / (float)a.N;
+  const float mean = a.ln_rms ? 0.f : (((s_red[0][0] + s_red[0][1]) + s_red[0][2]) + s_red[0][3]) / (float)a.N;
+  const float* ln_beta = a.ln_rms ? nullptr : a.ln_beta;
   float q = 0.f;
 #pragma unroll
   for (int i = 0; i < 4; ++i) {
@@ -368,7 +369,7 @@ __global__ void __launch_bounds__(256) splitk_reduce_ln_kernel(const GemmArgs a,
 #pragma unroll
       for (int e = 0; e < 4; ++e) {
         if (n + e >= a.N) continue;
-        const float y = (v[i][e] - mean) * rstd * a.ln_gamma[n + e] + (a.ln_beta ? a.ln_beta[n + e] : 0.f);
+        const float y = (v[i][e] - mean) * rstd * a.ln_gamma[n + e] + (ln_beta ? ln_beta[n + e] : 0.f);
         const long off = (long)m * a.ln_ldo + n + e;
         if (a.ln_out_dtype == DT_F32) reinterpret_cast<float*>(a.ln_out)[off] = y;
         else reinterpret_cast<uint16_t*>(a.ln_out)[off] = a.ln_out_dtype == DT_BF16 ? f32_to_bf16_bits(y) : f32_to_f16_bits(y);
@@ -424,11 +425,13 @@ static hipError_t launch_cfg(const GemmArgs& a, hipStream_t st) {
   return hipGetLastError();
 }
 
-// Workspace of the K-sliced GEMMs: one per (device, stream a launch is issued or recorded on), so launches that may
-// run at the same time never share one. Lives until the process ends.
+// Device memory the GEMM launchers keep outside any model: the block of zeros of the 256x256 kernel (one per device) and
+// the workspaces of the K-sliced GEMMs issued through crl_gemm, one per (device, stream a launch is issued or recorded
+// on) so that launches that may run at the same time never share one. release_gemm_globals() (crl_shutdown) frees them.
 constexpr size_t SPLITK_WS_BYTES = 64u << 20;
 static std::mutex g_ws_mutex;
 static std::unordered_map<uint64_t, float*> g_ws;
+static uint8_t* g_zeros[16] = {};
 static hipError_t workspace_for(hipStream_t st, float** out) {
   int dev = 0;
   hipError_t e = hipGetDevice(&dev);
@@ -443,6 +446,40 @@ static hipError_t workspace_for(hipStream_t st, float** out) {
   g_ws.emplace(key, p);
   *out = p;
   return hipSuccess;
+}
+
+const uint8_t* device_zeros(hipError_t* err) {
+  std::lock_guard<std::mutex> lock(g_ws_mutex);   // first calls on one device may come from several host threads
+  int dev = 0;
+  *err = hipGetDevice(&dev);
+  if (*err != hipSuccess || dev < 0 || dev >= 16) { if (*err == hipSuccess) *err = hipErrorInvalidDevice; return nullptr; }
+  if (!g_zeros[dev]) {
+    uint8_t* p = nullptr;
+    *err = hipMalloc((void**)&p, 256);
+    if (*err != hipSuccess) return nullptr;
+    *err = hipMemset(p, 0, 256);
+    if (*err != hipSuccess) { (void)hipFree(p); return nullptr; }
+    g_zeros[dev] = p;
+  }
+  return g_zeros[dev];
+}
+
+void release_gemm_globals() {
+  std::lock_guard<std::mutex> lock(g_ws_mutex);
+  int cur = 0;
+  const bool have_dev = hipGetDevice(&cur) == hipSuccess;
+  for (auto& kv : g_ws) {
+    if (have_dev) (void)hipSetDevice((int)(kv.first & 15));
+    (void)hipFree(kv.second);
+  }
+  g_ws.clear();
+  for (int d = 0; d < 16; ++d)
+    if (g_zeros[d]) {
+      if (have_dev) (void)hipSetDevice(d);
+      (void)hipFree(g_zeros[d]);
+      g_zeros[d] = nullptr;
+    }
+  if (have_dev) (void)hipSetDevice(cur);
 }
 
 // Few output tiles and a long K leave most CUs idle while a few walk K alone (M=128, N=768, K=3072: 24 workgroups
@@ -487,6 +524,7 @@ bool gemm_folds_layernorm(const GemmArgs& a, int in_dt) {
 
 template <typename Cfg, int IN_DT, int OUT_DT>
 static hipError_t launch_splitk(const GemmArgs& a, int ks, int per, hipStream_t st) {
+  if (a.res_stats) return hipErrorInvalidValue;   // the second pass adds the residual as stored: it has no normalising form
   float* ws = a.splitk_ws;
   hipError_t e = ws ? hipSuccess : workspace_for(st, &ws);
   if (e != hipSuccess) return e;
@@ -520,6 +558,7 @@ static hipError_t launch_splitk(const GemmArgs& a, int ks, int per, hipStream_t 
 template <int IN_DT, int OUT_DT>
 static hipError_t launch_in_out(const GemmArgs& a, int tile, hipStream_t st) {
   if (a.ln_out && !gemm_folds_layernorm(a, IN_DT)) return hipErrorInvalidValue;   // only the K-sliced path has a whole row in one place
+  if (a.res_stats && (a.k_parallel || tile >= 4)) return hipErrorInvalidValue;   // tiles 1-3 only
   if ((tile == 0 && a.k_parallel) || tile == 4) {
     int per = 0;
     const int ks = splitk_plan(a, IN_DT == DT_FP8 ? 1 : 2, tile == 4, &per);
@@ -539,13 +578,13 @@ static hipError_t launch_in_out(const GemmArgs& a, int tile, hipStream_t st) {
     const long small = (long)((a.M + 63) / 64) * ((a.N + 63) / 64);
     const long nslab = ((long)a.K * (IN_DT == DT_FP8 ? 1 : 2) + 127) >> 7;
     if (tile == 1 && a.k_parallel && small <= 512 && nslab >= 8) tile = 5;
-    if (tile == 1 && !a.k_parallel) {
+    // (a residual that is normalised on the fly needs the tiled kernels' epilogue: no K slices for it)
+    if (tile == 1 && !a.k_parallel && !a.res_stats) {
       int per = 0;
       const int ks = splitk_plan_fixed(a, IN_DT == DT_FP8 ? 1 : 2, &per);
       if (ks > 1) return launch_splitk<CfgSmallK4, IN_DT, OUT_DT>(a, ks, per, st);
     }
   }
-  if (a.res_stats && tile == 5) return hipErrorInvalidValue;   // the K-grouped tile has no residual-normalising form
   if (tile == 3) return launch_gemm_dma(a, IN_DT, OUT_DT, st);
   if (tile == 2) return launch_cfg<CfgMid, IN_DT, OUT_DT>(a, st);
   if (tile == 5) return launch_cfg<CfgSmallK4, IN_DT, OUT_DT>(a, st);

@@ -279,25 +279,6 @@ __global__ void __launch_bounds__(Cfg::NT, 2) gemm_dma_kernel(const GemmArgs a, 
                                                      reinterpret_cast<float*>(smem + Cfg::STATS_OFF) + wave * (2 * Cfg::WM));
 }
 
-// One 256-byte block of zeros per device: the source of K-tail chunks for the direct-to-LDS loads.
-inline const uint8_t* device_zeros(hipError_t* err) {
-  static uint8_t* z[16] = {};
-  static std::mutex mu;   // first calls on one device may come from several host threads
-  std::lock_guard<std::mutex> lock(mu);
-  int dev = 0;
-  *err = hipGetDevice(&dev);
-  if (*err != hipSuccess || dev < 0 || dev >= 16) { if (*err == hipSuccess) *err = hipErrorInvalidDevice; return nullptr; }
-  if (!z[dev]) {
-    uint8_t* p = nullptr;
-    *err = hipMalloc((void**)&p, 256);
-    if (*err != hipSuccess) return nullptr;
-    *err = hipMemset(p, 0, 256);
-    if (*err != hipSuccess) { (void)hipFree(p); return nullptr; }
-    z[dev] = p;
-  }
-  return z[dev];
-}
-
 template <typename DCfg, int IN_DT, int OUT_DT, int RES_NORM = 0>
 static hipError_t launch_dma(const GemmArgs& a, hipStream_t st) {
   static std::atomic<bool> attr_set[16] = {};

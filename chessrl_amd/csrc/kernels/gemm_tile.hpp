@@ -360,6 +360,8 @@ __device__ __forceinline__ void gemm_epilogue(const GemmArgs& a, f32x16_t (&acc)
 // own: its speed depends measurably on where its code lands (identical instructions ran 3-8 % slower after unrelated
 // kernels were added to the same code object), and alone it stays where it was measured.
 hipError_t launch_gemm_dma(const GemmArgs& a, int in_dt, int out_dt, hipStream_t st);
+// One 256-byte block of zeros per device (gemm.hip): the source of K-tail chunks for the direct-to-LDS loads.
+const uint8_t* device_zeros(hipError_t* err);
 hipError_t launch_gemm_dma_resnorm(const GemmArgs& a, hipStream_t st);   // gemm_dma_resnorm.hip
 
 }  // namespace crl

@@ -62,9 +62,10 @@ __device__ __forceinline__ void store8_fp8(uint8_t* base, long off, const float 
 }
 
 // Normalise the VPL*8 values a lane holds (columns col0(i) = (i*64+lane)*8) and write them.
+// rms: RMSNorm (mean taken as zero, no offset): y = x * rsqrt(mean(x^2) + eps) * gamma.
 template <int VPL>
 __device__ __forceinline__ void ln_finish(float (&x)[VPL][8], int lane, int C, const float* gamma, const float* beta,
-                                           float eps, float (&y)[VPL][8], float* stats = nullptr) {
+                                           float eps, float (&y)[VPL][8], float* stats = nullptr, bool rms = false) {
   float s = 0.f;
 #pragma unroll
   for (int i = 0; i < VPL; ++i) {
@@ -73,7 +74,8 @@ __device__ __forceinline__ void ln_finish(float (&x)[VPL][8], int lane, int C, c
       for (int e = 0; e < 8; ++e) s += x[i][e];
     }
   }
-  const float mean = wave_sum(s) / (float)C;
+  const float mean = rms ? 0.f : wave_sum(s) / (float)C;
+  if (rms) beta = nullptr;
   float q = 0.f;
 #pragma unroll
   for (int i = 0; i < VPL; ++i) {
@@ -108,13 +110,14 @@ __global__ void __launch_bounds__(256) layernorm_kernel(const LayerNormArgs a) {
     const int col = (i * 64 + lane) * 8;
     if (col < a.C) load8<IN_DT>(a.x, (long)row * a.ldx + col, x[i]);
   }
-  ln_finish<VPL>(x, lane, a.C, a.gamma, a.beta, a.eps, y, a.stats ? a.stats + 2 * (long)row : nullptr);
+  ln_finish<VPL>(x, lane, a.C, a.gamma, a.beta, a.eps, y, a.stats ? a.stats + 2 * (long)row : nullptr, a.rms != 0);
   float am = 0.f;
 #pragma unroll
   for (int i = 0; i < VPL; ++i) {
     const int col = (i * 64 + lane) * 8;
     if (col < a.C) {
       if (a.out) store8(a.out, (long)row * a.ldo + col, y[i], a.out_dtype);
+      if (a.out_b) store8(a.out_b, (long)row * a.ldo + col, y[i], a.out_b_dtype);
       if (a.out_fp8) store8_fp8(a.out_fp8, (long)row * a.ldo + col, y[i], a.fp8_scale);
       if (a.amax) {
 #pragma unroll
@@ -152,7 +155,9 @@ __global__ void __launch_bounds__(256) layernorm_wide_kernel(const LayerNormArgs
   s = wave_sum(s);
   if (lane == 0) s_red[0][wave] = s;
   __syncthreads();
-  const float mean = (((s_red[0][0] + s_red[0][1]) + s_red[0][2]) + s_red[0][3]) / (float)a.C;
+  const bool rms = a.rms != 0;
+  const float mean = rms ? 0.f : (((s_red[0][0] + s_red[0][1]) + s_red[0][2]) + s_red[0][3]) / (float)a.C;
+  const float* beta = rms ? nullptr : a.beta;
   float q = 0.f;
 #pragma unroll
   for (int i = 0; i < VPT; ++i) {
@@ -172,10 +177,11 @@ __global__ void __launch_bounds__(256) layernorm_wide_kernel(const LayerNormArgs
     if (col < a.C) {
       float gv[8], bv[8], y[8];
       load8<DT_F32>(a.gamma, col, gv);
-      if (a.beta) load8<DT_F32>(a.beta, col, bv);
+      if (beta) load8<DT_F32>(beta, col, bv);
 #pragma unroll
-      for (int e = 0; e < 8; ++e) y[e] = (x[i][e] - mean) * rstd * gv[e] + (a.beta ? bv[e] : 0.f);
+      for (int e = 0; e < 8; ++e) y[e] = (x[i][e] - mean) * rstd * gv[e] + (beta ? bv[e] : 0.f);
       if (a.out) store8(a.out, row * a.ldo + col, y, a.out_dtype);
+      if (a.out_b) store8(a.out_b, row * a.ldo + col, y, a.out_b_dtype);
       if (a.out_fp8) store8_fp8(a.out_fp8, row * a.ldo + col, y, a.fp8_scale);
       if (a.amax) {
 #pragma unroll
@@ -204,6 +210,7 @@ static hipError_t launch_ln_dt(const LayerNormArgs& a, hipStream_t st) {
 hipError_t launch_layernorm(const LayerNormArgs& a, hipStream_t st) {
   if (a.rows <= 0) return hipSuccess;
   if (a.C % 8 || a.ldx % 8 || a.ldo % 8 || a.C > 8192) return hipErrorInvalidValue;
+  if ((a.out && a.out_dtype == DT_FP8) || (a.out_b && a.out_b_dtype == DT_FP8)) return hipErrorInvalidValue;   // e4m3 goes through out_fp8
   if (a.stats && a.C > 2048) return hipErrorInvalidValue;   // the four-waves-per-row kernel does not write them
   switch (a.in_dtype) {
     case DT_F32: return launch_ln_dt<DT_F32>(a, st);
@@ -279,6 +286,7 @@ __global__ void __launch_bounds__(256) embed_kernel(const EmbedArgs a) {
         for (int e = 0; e < 8; ++e) y[i][e] += pe[e];
       }
       store8(a.out, orow * a.C + col, y[i], a.out_dtype);
+      if (a.out_b) store8(a.out_b, orow * a.C + col, y[i], a.out_b_dtype);
       if (a.out_fp8) store8_fp8(a.out_fp8, orow * a.C + col, y[i], a.fp8_scale);
       if (a.amax) {
 #pragma unroll

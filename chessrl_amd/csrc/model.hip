@@ -46,6 +46,11 @@ Model::Model(const crl_model_config& c) : cfg(c) {
   if (cfg.act_dtype != DT_F16) cfg.act_dtype = DT_BF16;
   if (cfg.head_dtype != DT_F16 && cfg.head_dtype != DT_BF16) cfg.head_dtype = cfg.act_dtype;
   if (cfg.micro_batch <= 0) cfg.micro_batch = 4096;
+  // tri-state switches: 0 picks the default
+  if (cfg.stream_f32 == 0) cfg.stream_f32 = cfg.arch == CRL_ARCH_GPT64 ? 1 : -1;
+  if (cfg.ln_fold == 0) cfg.ln_fold = 1;
+  if (cfg.fp8_lm_head == 0) cfg.fp8_lm_head = 1;
+  cfg.norm_rms = cfg.norm_rms ? 1 : 0;
   vocab = cfg.arch == CRL_ARCH_BT4CLASS ? VOCAB_LEELA : VOCAB_RL;
   const long C = cfg.d_model, F = cfg.d_ff, L = cfg.n_layer, H = cfg.n_head;
   auto add = [&](const std::string& k, long n) { expected.push_back({k, n}); };
@@ -92,7 +97,7 @@ Model::Model(const crl_model_config& c) : cfg(c) {
     }
     lin("value_head.dense1", 128, C); lin("value_head.dense2", 128, 128 * 64); lin("value_head.dense3", 3, 128);
   }
-  amax_host.assign((size_t)L * AMAX_SLOTS, 0.f);
+  amax_host.assign((size_t)(L + 1) * AMAX_SLOTS, 0.f);
 }
 
 Model::~Model() {
@@ -109,10 +114,13 @@ int Model::set_weight(const char* key, const float* data, long numel) {
   if (k == "transformer.wte.weight") return CRL_OK;  // tied to lm_head.weight (model_bis.py:148)
   for (auto& e : expected) {
     if (e.first != k) continue;
-    const bool ok = (k == "pe") ? numel >= e.second : numel == e.second;
+    // pe may carry more rows than the 64 board tokens; lm_head may carry padding rows behind the 1929 moves
+    // (pretrain_fp8.py:16 trains with vocab_size 1936 so that the fp8 GEMM's N is a multiple of 16).
+    const bool grows = k == "pe" || k == "lm_head.weight";
+    const bool ok = grows ? (numel >= e.second && numel % cfg.d_model == 0) : numel == e.second;
     if (!ok) { set_error("set_weight: " + k + " has " + std::to_string(numel) + " elements, expected " + std::to_string(e.second)); return CRL_ERR_ARG; }
     // The positional table may carry more rows than the 64 board tokens (block_size rows, model_bis.py:141-146).
-    const long keep = (k == "pe") ? numel - numel % cfg.d_model : e.second;
+    const long keep = grows ? numel : e.second;
     host[k].assign(data, data + keep);
     finalized = false;
     return CRL_OK;
@@ -145,12 +153,12 @@ int Model::upload(const std::vector<float>& v, int dt, float scale, void** out) 
 
 const std::vector<float>& Model::w(const std::string& k) { return host.at(k); }
 
-int Model::make_lin(Lin& L, const std::vector<float>& W, const std::vector<float>* bias, int N, int K, int dt16, bool fp8) {
+int Model::make_lin(Lin& L, const std::vector<float>& W, const std::vector<float>* bias, int N, int K, int dt16, bool fp8, float amax_all) {
   L.N = N; L.K = K; L.dt = dt16;
   int rc = upload(W, dt16, 1.f, &L.w);
   if (rc) return rc;
   if (fp8) {
-    float am = 0.f;
+    float am = amax_all > 0.f ? amax_all : 0.f;
     for (float x : W) am = std::fmax(am, std::fabs(x));
     L.wscale = am > 0.f ? 448.f / am : 1.f;
     rc = upload(W, DT_FP8, L.wscale, &L.w8);
@@ -199,7 +207,12 @@ int Model::finalize() {
   if (cfg.arch == CRL_ARCH_GPT64) {
     UP(w("pe"), DT_F32, pe_f32);
     pe_rows = (int)(w("pe").size() / (size_t)C);
-    UP(w("lm_head.weight"), DT_F32, wte_f32);   // token embedding, tied to the output head (model_bis.py:148)
+    // The first 1929 rows of lm_head are the moves; a checkpoint trained with a padded vocabulary has more. The e4m3
+    // scale is per tensor, so it is taken over every row the checkpoint holds.
+    std::vector<float> head_w(w("lm_head.weight").begin(), w("lm_head.weight").begin() + (size_t)VOCAB_RL * C);
+    float head_amax = 0.f;
+    for (float x : w("lm_head.weight")) head_amax = std::fmax(head_amax, std::fabs(x));
+    UP(head_w, DT_F32, wte_f32);   // token embedding, tied to the output head (model_bis.py:148)
     for (int i = 0; i < cfg.n_layer; ++i) {
       Layer& ly = layers[i];
       const std::string p = lkey("transformer.h.%d.", i);
@@ -211,7 +224,7 @@ int Model::finalize() {
       LIN(ly.ff2, w(p + "mlp.c_proj.weight"), &w(p + "mlp.c_proj.bias"), C, F, ad, f8);
     }
     UP(w("transformer.ln_f.weight"), DT_F32, lnf_g); UP(w("transformer.ln_f.bias"), DT_F32, lnf_b);
-    LIN(lm_head, w("lm_head.weight"), nullptr, VOCAB_RL, C, hd, false);
+    rc = make_lin(lm_head, head_w, nullptr, VOCAB_RL, C, hd, f8 && cfg.fp8_lm_head > 0, head_amax); if (rc) return rc;
   } else {
     // Absolute sinusoid table of new_paradigm/value.py:77-93.
     std::vector<float> pe((size_t)64 * C);
@@ -319,11 +332,13 @@ int Model::ensure_ws(int mb) {
   const size_t M = (size_t)mb * 64, C = cfg.d_model, F = cfg.d_ff, H = cfg.n_head;
   int rc;
 #define WS(ptr, bytes) do { rc = dev_alloc((void**)&(ptr), (bytes), true); if (rc) return rc; } while (0)
-  WS(ws.x, M * C * 4);        // residual stream (fp32 for GPT64 with stream_f32, else 16-bit)
+  const bool sf32_post = cfg.arch != CRL_ARCH_GPT64 && cfg.stream_f32 > 0;   // post-LN trunks keep x, t and h in the stream's type
+  WS(ws.x, M * C * 4);        // residual stream (fp32 with stream_f32, else 16-bit)
   WS(ws.x8, M * C);
-  WS(ws.t, M * C * 2);
-  WS(ws.h, M * C * 2);
+  WS(ws.t, M * C * (sf32_post ? 4 : 2));
+  WS(ws.h, M * C * (sf32_post ? 4 : 2));
   WS(ws.h8, M * C);
+  if (sf32_post) { WS(ws.x16, M * C * 2); WS(ws.h16, M * C * 2); }
   WS(ws.qkv, M * 3 * C * 2);
   WS(ws.ao, M * C * 2);
   WS(ws.ao8, M * C);
@@ -344,6 +359,7 @@ int Model::ensure_ws(int mb) {
   }
   if (cfg.arch == CRL_ARCH_GPT64) {
     WS(ws.hl, (size_t)mb * C * 2);
+    WS(ws.hl8, (size_t)mb * C);
   } else {
     WS(ws.tok, M * C * 2);
     WS(ws.pqk, M * 2 * C * 2);
@@ -411,13 +427,14 @@ int Model::gemm(const Lin& L, const void* A, long lda, int in_dt, void* C, long 
   g.C = C; g.ldc = ldc; g.C2 = o.C2; g.ldc2 = o.ldc2; g.nsplit = o.nsplit > 0 ? o.nsplit : L.N;
   g.bias = L.b; g.res = o.res; g.ldr = o.ldr; g.res_dtype = o.res_dt; g.res_rows = o.res_rows;
   g.amax = o.amax; g.M = M; g.N = L.N; g.K = L.K; g.act = o.act;
-  g.res_stats = o.res_stats; g.res_gamma = o.res_g; g.res_beta = o.res_b;
+  g.res_stats = o.res_stats; g.res_gamma = o.res_g; g.res_beta = cfg.norm_rms ? nullptr : o.res_b;
   g.descale = in_dt == DT_FP8 ? 1.f / (o.a_scale * L.wscale) : 1.f;
   g.alpha = o.alpha; g.out_scale = o.out_scale; g.k_parallel = o.k_parallel ? 1 : 0;
   g.splitk_ws = ws.splitk; g.splitk_ws_bytes = Workspace::SPLITK_BYTES;
   if (o.ln_out) {
     g.nsplit = g.N;
     g.ln_gamma = o.ln_g; g.ln_beta = o.ln_b; g.ln_out = o.ln_out; g.ln_ldo = L.N; g.ln_out_dtype = o.ln_dt; g.ln_eps = cfg.eps;
+    g.ln_rms = cfg.norm_rms;
     const bool fold = !profiling && gemm_folds_layernorm(g, in_dt == DT_FP8 ? DT_FP8 : L.dt);
     if (o.ln_folded) *o.ln_folded = fold;
     if (!fold) { g.ln_gamma = g.ln_beta = nullptr; g.ln_out = nullptr; }
@@ -431,12 +448,14 @@ int Model::gemm(const Lin& L, const void* A, long lda, int in_dt, void* C, long 
   return CRL_OK;
 }
 
+// trunk: one of the norms cfg.norm_rms turns into RMSNorm (the stem's and the bias generator's stay LayerNorm).
 int Model::lnorm(const void* x, long ldx, int in_dt, const float* g, const float* b, void* out, int out_dt, uint8_t* out8,
-                 float scale8, long ldo, int rows, int C, float* amax, hipStream_t st, float* stats) {
+                 float scale8, long ldo, int rows, int C, float* amax, hipStream_t st, float* stats, void* out_b, int out_b_dt, bool trunk) {
   LayerNormArgs a;
   std::memset(&a, 0, sizeof(a));
   a.x = x; a.ldx = ldx; a.in_dtype = in_dt; a.gamma = g; a.beta = b; a.out = out; a.out_dtype = out_dt;
   a.out_fp8 = out8; a.fp8_scale = scale8; a.ldo = ldo; a.rows = rows; a.C = C; a.eps = cfg.eps; a.amax = amax; a.stats = stats;
+  a.out_b = out_b; a.out_b_dtype = out_b_dt; a.rms = (trunk && cfg.norm_rms) ? 1 : 0;
   prof_begin(2, st);
   hipError_t e = launch_layernorm(a, st);
   prof_end(st);
@@ -488,7 +507,10 @@ int Model::forward_chunk(const float* planes, const uint8_t* ids, const uint8_t*
   const bool f8 = cfg.fp8 && !calibrate && !force_16bit;
   const int hd = cfg.head_dtype, ad = cfg.act_dtype;
   const bool gpt = cfg.arch == CRL_ARCH_GPT64;
-  const bool sf32 = gpt && cfg.stream_f32;
+  // fp32 residual stream: GPT64 keeps x in fp32; the post-LN trunks keep x, t and h in fp32 and hand the products a
+  // 16-bit (or e4m3) operand copy written by the same LayerNorm launch.
+  const bool sf32 = cfg.stream_f32 > 0 && (gpt || L > 0);
+  const bool sf32p = sf32 && !gpt;
   const int xdt = sf32 ? DT_F32 : ad;
   auto am = [&](int l, int slot) -> float* { return calibrate ? amax_dev + (size_t)l * AMAX_SLOTS + slot : nullptr; };
   int rc;
@@ -504,6 +526,7 @@ int Model::forward_chunk(const float* planes, const uint8_t* ids, const uint8_t*
     e.out = ws.x; e.out_dtype = (L == 0 && !gpt) ? hd : xdt; e.tokens = mb * 64; e.C = C; e.act = ACT_GELU; e.eps = cfg.eps;
     e.out_T = T;
     if (!gpt && L > 0) { e.out_fp8 = f8 ? ws.x8 : nullptr; e.fp8_scale = f8 ? act_scale(0, 0) : 1.f; e.amax = am(0, 0); }
+    if (sf32p && !f8) { e.out_b = ws.x16; e.out_b_dtype = ad; }
     prof_begin(3, st);
     hipError_t he = launch_embed(e, st);
     prof_end(st);
@@ -524,7 +547,10 @@ int Model::forward_chunk(const float* planes, const uint8_t* ids, const uint8_t*
 
   // BT4-class in e4m3 with bf16 activations: the normalised activations are not written in 16 bits at all (every
   // tile size has the residual-normalising epilogue, so this does not depend on the batch).
-  const bool fold = ln_fold && f8 && cfg.arch == CRL_ARCH_BT4CLASS && ad == DT_BF16;
+  const bool fold = cfg.ln_fold > 0 && f8 && cfg.arch == CRL_ARCH_BT4CLASS && ad == DT_BF16 && !sf32;
+  // 16-bit operand copies of x and h (the tensors themselves when the stream is 16-bit)
+  void* const x_op = sf32p ? ws.x16 : ws.x;
+  void* const h_op = sf32p ? ws.h16 : ws.h;
   const float attn_scale = cfg.arch == CRL_ARCH_BT4 ? 1.0f / std::sqrt((float)C) : 1.0f / std::sqrt((float)hs);
   const float alpha = cfg.arch == CRL_ARCH_BT4CLASS ? std::pow(2.0f * (float)L, -0.25f) : 1.0f;
 
@@ -537,7 +563,7 @@ int Model::forward_chunk(const float* planes, const uint8_t* ids, const uint8_t*
       RUN(lnorm(ws.x, C, xdt, ly.ln1_g, ly.ln1_b, f8 ? nullptr : ws.h, ad, f8 ? ws.h8 : nullptr, f8 ? act_scale(l, 0) : 1.f, C, M, C, am(l, 0), st));
       a_in = f8 ? (const void*)ws.h8 : (const void*)ws.h; a_dt = f8 ? DT_FP8 : ad; a_sc = f8 ? act_scale(l, 0) : 1.f;
     } else {
-      a_in = f8 ? (const void*)ws.x8 : (const void*)ws.x; a_dt = f8 ? DT_FP8 : ad; a_sc = f8 ? act_scale(l, 0) : 1.f;
+      a_in = f8 ? (const void*)ws.x8 : (const void*)x_op; a_dt = f8 ? DT_FP8 : ad; a_sc = f8 ? act_scale(l, 0) : 1.f;
     }
     // q|k|v (and the smolgen compression for BT4-class) in one GEMM
     {
@@ -551,12 +577,12 @@ int Model::forward_chunk(const float* planes, const uint8_t* ids, const uint8_t*
       const int sc = cfg.smolgen_compress, sh = cfg.smolgen_hidden, sg = cfg.smolgen_gen;
       GOpt o; o.act = ACT_SWISH;
       RUN(gemm(ly.sm_hidden, ws.comp, 64 * sc, ad, ws.sh1, sh, ad, mb, o, st));
-      RUN(lnorm(ws.sh1, sh, ad, ly.sm_ln1_g, ly.sm_ln1_b, ws.sh2, ad, nullptr, 1.f, sh, mb, sh, nullptr, st));
+      RUN(lnorm(ws.sh1, sh, ad, ly.sm_ln1_g, ly.sm_ln1_b, ws.sh2, ad, nullptr, 1.f, sh, mb, sh, nullptr, st, nullptr, nullptr, DT_BF16, false));
       RUN(gemm(ly.sm_gen, ws.sh2, sh, ad, ws.sg1, H * sg, ad, mb, o, st));
       // The shared 256 -> 4096 generator is the largest smolgen product (2*B*H*256*4096 per layer): in the fp8
       // configuration it takes e4m3 inputs like the trunk linears; the two small layers before it stay 16-bit.
       RUN(lnorm(ws.sg1, H * sg, ad, ly.sm_ln2_g, ly.sm_ln2_b, f8 ? nullptr : ws.sg2, ad, f8 ? ws.sg2_8 : nullptr, f8 ? act_scale(l, 4) : 1.f,
-                H * sg, mb, H * sg, am(l, 4), st));
+                H * sg, mb, H * sg, am(l, 4), st, nullptr, nullptr, DT_BF16, false));
       GOpt o2; o2.a_scale = f8 ? act_scale(l, 4) : 1.f;
       RUN(gemm(sm_weight_gen, f8 ? (const void*)ws.sg2_8 : (const void*)ws.sg2, sg, f8 ? DT_FP8 : ad, ws.bias, 4096, ad, mb * H, o2, st));
       bias_tile = ws.bias;
@@ -592,45 +618,51 @@ int Model::forward_chunk(const float* planes, const uint8_t* ids, const uint8_t*
       // t = x + alpha*proj(ao);  h = LN1(t). With `fold` the normalised tensors x and h exist only as e4m3 copies
       // (the products' operands): the LayerNorm launches leave their row statistics behind, and the product that
       // takes x or h as its residual re-normalises the un-normalised tensor t in its epilogue, writing in place.
-      { GOpt o; o.res = ws.x; o.ldr = C; o.res_dt = ad; o.alpha = alpha; o.a_scale = f8 ? act_scale(l, 1) : 1.f;
+      // With an fp32 stream x, t and h are fp32 and every norm also writes the 16-bit operand copy (x16, h16).
+      { GOpt o; o.res = ws.x; o.ldr = C; o.res_dt = xdt; o.alpha = alpha; o.a_scale = f8 ? act_scale(l, 1) : 1.f;
         if (fold && l > 0) { o.res = ws.t; o.res_stats = ws.st2; o.res_g = layers[l - 1].ln2_g; o.res_b = layers[l - 1].ln2_b; }
-        RUN(gemm(ly.proj, ao_in, C, ao_dt, ws.t, C, ad, M, o, st)); }
-      RUN(lnorm(ws.t, C, ad, ly.ln1_g, ly.ln1_b, fold ? nullptr : ws.h, ad, f8 ? ws.h8 : nullptr, f8 ? act_scale(l, 2) : 1.f, C, M, C, am(l, 2), st,
-                fold ? ws.st1 : nullptr));
-      const void* h_in = f8 ? (const void*)ws.h8 : (const void*)ws.h;
+        RUN(gemm(ly.proj, ao_in, C, ao_dt, ws.t, C, xdt, M, o, st)); }
+      RUN(lnorm(ws.t, C, xdt, ly.ln1_g, ly.ln1_b, fold ? nullptr : ws.h, xdt, f8 ? ws.h8 : nullptr, f8 ? act_scale(l, 2) : 1.f, C, M, C, am(l, 2), st,
+                fold ? ws.st1 : nullptr, (sf32p && !f8) ? ws.h16 : nullptr, ad));
+      const void* h_in = f8 ? (const void*)ws.h8 : (const void*)h_op;
       if (cfg.arch == CRL_ARCH_BT4) {
         // y = ff2(ff1(h)) with no activation in between; t = gelu(y) + h (new_paradigm/value.py:65-70)
         { GOpt o; o.a_scale = f8 ? act_scale(l, 2) : 1.f; o.out_scale = f8 ? act_scale(l, 3) : 1.f; o.amax = am(l, 3);
           RUN(gemm(ly.ff1, h_in, C, ao_dt, f8 ? (void*)ws.f8 : (void*)ws.f, F, ao_dt, M, o, st)); }
-        { GOpt o; o.act = ACT_GELU; o.res = ws.h; o.ldr = C; o.res_dt = ad; o.a_scale = f8 ? act_scale(l, 3) : 1.f;
-          RUN(gemm(ly.ff2, f8 ? (const void*)ws.f8 : (const void*)ws.f, F, ao_dt, ws.t, C, ad, M, o, st)); }
+        { GOpt o; o.act = ACT_GELU; o.res = ws.h; o.ldr = C; o.res_dt = xdt; o.a_scale = f8 ? act_scale(l, 3) : 1.f;
+          RUN(gemm(ly.ff2, f8 ? (const void*)ws.f8 : (const void*)ws.f, F, ao_dt, ws.t, C, xdt, M, o, st)); }
       } else {
         { GOpt o; o.act = ACT_MISH; o.a_scale = f8 ? act_scale(l, 2) : 1.f; o.out_scale = f8 ? act_scale(l, 3) : 1.f; o.amax = am(l, 3);
           RUN(gemm(ly.ff1, h_in, C, ao_dt, f8 ? (void*)ws.f8 : (void*)ws.f, F, ao_dt, M, o, st)); }
-        { GOpt o; o.res = ws.h; o.ldr = C; o.res_dt = ad; o.alpha = alpha; o.a_scale = f8 ? act_scale(l, 3) : 1.f;
+        { GOpt o; o.res = ws.h; o.ldr = C; o.res_dt = xdt; o.alpha = alpha; o.a_scale = f8 ? act_scale(l, 3) : 1.f;
           if (fold) { o.res = ws.t; o.res_stats = ws.st1; o.res_g = ly.ln1_g; o.res_b = ly.ln1_b; }
-          RUN(gemm(ly.ff2, f8 ? (const void*)ws.f8 : (const void*)ws.f, F, ao_dt, ws.t, C, ad, M, o, st)); }
+          RUN(gemm(ly.ff2, f8 ? (const void*)ws.f8 : (const void*)ws.f, F, ao_dt, ws.t, C, xdt, M, o, st)); }
       }
       // x = LN2(t); the last layer's output feeds only the heads.
-      RUN(lnorm(ws.t, C, ad, ly.ln2_g, ly.ln2_b, (fold && !last) ? nullptr : ws.x, last ? hd : ad, (f8 && !last) ? ws.x8 : nullptr,
-                (f8 && !last) ? act_scale(l + 1, 0) : 1.f, C, M, C, last ? nullptr : am(l + 1, 0), st, (fold && !last) ? ws.st2 : nullptr));
+      RUN(lnorm(ws.t, C, xdt, ly.ln2_g, ly.ln2_b, (fold && !last) ? nullptr : ws.x, last ? hd : xdt, (f8 && !last) ? ws.x8 : nullptr,
+                (f8 && !last) ? act_scale(l + 1, 0) : 1.f, C, M, C, last ? nullptr : am(l + 1, 0), st, (fold && !last) ? ws.st2 : nullptr,
+                (sf32p && !f8 && !last) ? ws.x16 : nullptr, ad));
     }
   }
 
   // ---- heads
   if (gpt) {
+    // lm_head takes e4m3 operands too in the fp8 model (model_fp8.py:140); its input scale is the first entry of the
+    // amax table's last row.
+    const bool f8h = f8 && lm_head.w8 != nullptr;
+    const float hsc = f8h ? act_scale(L, 0) : 1.f;
     if (all_logits) {
       // ln_f and lm_head on every token (model_bis.py:189-192, compute_loss=True).
-      RUN(lnorm(ws.x, C, xdt, lnf_g, lnf_b, ws.h, hd, nullptr, 1.f, C, M, C, nullptr, st));
-      GOpt o;
-      RUN(gemm(lm_head, ws.h, C, hd, all_logits, VOCAB_RL, DT_F32, M, o, st));
+      RUN(lnorm(ws.x, C, xdt, lnf_g, lnf_b, f8h ? nullptr : ws.h, hd, f8h ? ws.h8 : nullptr, hsc, C, M, C, policy ? nullptr : am(L, 0), st));
+      GOpt o; o.a_scale = hsc;
+      RUN(gemm(lm_head, f8h ? (const void*)ws.h8 : (const void*)ws.h, C, f8h ? DT_FP8 : hd, all_logits, VOCAB_RL, DT_F32, M, o, st));
     }
     if (policy) {
       // ln_f and lm_head on the last token only (model_bis.py:195-196, 369-370).
       const char* last_tok = reinterpret_cast<const char*>(ws.x) + (size_t)(T - 1) * C * dtype_size(xdt);
-      RUN(lnorm(last_tok, (long)T * C, xdt, lnf_g, lnf_b, ws.hl, hd, nullptr, 1.f, C, mb, C, nullptr, st));
-      GOpt o;
-      RUN(gemm(lm_head, ws.hl, C, hd, policy, VOCAB_RL, DT_F32, mb, o, st));
+      RUN(lnorm(last_tok, (long)T * C, xdt, lnf_g, lnf_b, f8h ? nullptr : ws.hl, hd, f8h ? ws.hl8 : nullptr, hsc, C, mb, C, am(L, 0), st));
+      GOpt o; o.a_scale = hsc;
+      RUN(gemm(lm_head, f8h ? (const void*)ws.hl8 : (const void*)ws.hl, C, f8h ? DT_FP8 : hd, policy, VOCAB_RL, DT_F32, mb, o, st));
     }
     return CRL_OK;
   }
@@ -709,7 +741,7 @@ int Model::generate(const float* planes, int B, int steps, float temperature, ui
     kv_B = B; kv_Tmax = Tmax;
   }
   const int hd = cfg.head_dtype, ad = cfg.act_dtype;
-  const int xdt = cfg.stream_f32 ? DT_F32 : ad;
+  const int xdt = cfg.stream_f32 > 0 ? DT_F32 : ad;
   const long START_THINK = 1924, END_THINK = 1925, END_VARIATION = 1926, END = 1927;
   // <thinking> opens every sequence (model_bis.py:221-224); gen_zeros doubles as the fill source via a tiny host copy.
   {

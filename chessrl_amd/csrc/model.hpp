@@ -34,6 +34,8 @@ struct Layer {
 
 struct Workspace {
   void *x = nullptr, *t = nullptr, *h = nullptr, *qkv = nullptr, *ao = nullptr, *f = nullptr;
+  void *x16 = nullptr, *h16 = nullptr;   // 16-bit operand copies of x and h beside an fp32 residual stream (BT4, BT4-class)
+  uint8_t* hl8 = nullptr;                // e4m3 input of lm_head
   uint8_t *x8 = nullptr, *h8 = nullptr, *ao8 = nullptr, *f8 = nullptr, *stm = nullptr;
   float *st1 = nullptr, *st2 = nullptr;   // row statistics (mean, 1/std) of a layer's two LayerNorms
   void *comp = nullptr, *sh1 = nullptr, *sh2 = nullptr, *sg1 = nullptr, *sg2 = nullptr, *bias = nullptr;
@@ -61,8 +63,8 @@ struct Model {
   Lin lm_head, pol_tok, pol_qk, pol_head, val1, val2, val3, sm_weight_gen;
   int16_t* gidx = nullptr;
   int8_t* gpromo = nullptr;
-  // Activation amax table [n_layer][AMAX_SLOTS]: input of q|k|v, attention output, input of FFN-1, input of FFN-2,
-  // input of the shared bias generator (BT4-class only).
+  // Activation amax table [n_layer + 1][AMAX_SLOTS]: input of q|k|v, attention output, input of FFN-1, input of FFN-2,
+  // input of the shared bias generator (BT4-class only); the first entry of the last row is the input of lm_head (GPT64).
   static constexpr int AMAX_SLOTS = 5;
   float* amax_dev = nullptr;
   std::vector<float> amax_host;
@@ -81,7 +83,6 @@ struct Model {
   bool decode_graph = false;
   bool kv_capture = false;     // forward_chunk copies every layer's keys|values into the cache
   bool force_16bit = false;    // forward_chunk ignores cfg.fp8
-  bool ln_fold = true;         // e4m3 BT4-class: normalised activations exist only as e4m3 copies (forward_chunk)
 
   struct ProfEvent { hipEvent_t a, b; int fam; };
   bool profiling = false;
@@ -112,13 +113,14 @@ struct Model {
   const std::vector<float>& w(const std::string& k);
   int dev_alloc(void** p, size_t bytes, bool ws);
   int upload(const std::vector<float>& v, int dt, float scale, void** out);
-  int make_lin(Lin& L, const std::vector<float>& W, const std::vector<float>* bias, int N, int K, int dt16, bool fp8);
+  int make_lin(Lin& L, const std::vector<float>& W, const std::vector<float>* bias, int N, int K, int dt16, bool fp8, float amax_all = -1.f);
   int ensure_ws(int mb);
   int forward_chunk(const float* planes, const uint8_t* ids, const uint8_t* flags, const int64_t* idx, int t, int mb, float* policy,
                     float* all_logits, float* wdl, bool calibrate, hipStream_t st);
   int gemm(const Lin& L, const void* A, long lda, int in_dt, void* C, long ldc, int out_dt, int M, const GOpt& o, hipStream_t st);
   int lnorm(const void* x, long ldx, int in_dt, const float* g, const float* b, void* out, int out_dt, uint8_t* out8, float scale8,
-            long ldo, int rows, int C, float* amax, hipStream_t st, float* stats = nullptr);
+            long ldo, int rows, int C, float* amax, hipStream_t st, float* stats = nullptr, void* out_b = nullptr, int out_b_dt = DT_BF16,
+            bool trunk = true);
   float act_scale(int layer, int slot) const;
   void prof_begin(int fam, hipStream_t st);
   void prof_end(hipStream_t st);

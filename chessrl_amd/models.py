@@ -158,13 +158,18 @@ def cross_entropy(logits, targets, ignore_index=-100):
 class _Engine:
     """Owns one crl_model handle."""
 
-    def __init__(self, arch, n_layer, d_model, n_head, d_ff, fp8=False, micro_batch=0, stream_f32=True,
-                 head_dtype=None, act_dtype="bf16", compress=32, hidden=256, gen=256):
+    def __init__(self, arch, n_layer, d_model, n_head, d_ff, fp8=False, micro_batch=0, stream_f32=None,
+                 head_dtype=None, act_dtype="bf16", compress=32, hidden=256, gen=256, ln_fold=None, norm_rms=False,
+                 fp8_lm_head=None):
         cfg = _lib.ModelConfig()
         cfg.arch, cfg.n_layer, cfg.d_model, cfg.n_head, cfg.d_ff = arch, n_layer, d_model, n_head, d_ff
         cfg.fp8 = 1 if fp8 else 0
         cfg.micro_batch = micro_batch
-        cfg.stream_f32 = 1 if stream_f32 else 0
+        tri = lambda v: 0 if v is None else 1 if v else -1     # None = the library's default
+        cfg.stream_f32 = tri(stream_f32)
+        cfg.ln_fold = tri(ln_fold)
+        cfg.fp8_lm_head = tri(fp8_lm_head)
+        cfg.norm_rms = 1 if norm_rms else 0
         cfg.act_dtype = _lib.F16 if act_dtype in ("f16", "fp16") else _lib.BF16
         cfg.head_dtype = cfg.act_dtype if head_dtype is None else _lib.F16 if head_dtype in ("f16", "fp16") else _lib.BF16
         cfg.smolgen_compress, cfg.smolgen_hidden, cfg.smolgen_gen = compress, hidden, gen
@@ -215,10 +220,13 @@ class _Engine:
         planes = _as_planes(planes)
         check(lib().crl_model_calibrate(self.handle, _ptr(planes), planes.shape[0], _stream_ptr()), "crl_model_calibrate")
 
-    def get_amax(self):
-        a = np.zeros(self.n_layer * 5, np.float32)
+    def get_amax(self, head=False):
+        """Activation amax table [n_layer, 5]; with head=True [n_layer + 1, 5], whose last row starts with the amax
+        of lm_head's input."""
+        rows = self.n_layer + (1 if head else 0)
+        a = np.zeros(rows * 5, np.float32)
         check(lib().crl_model_get_amax(self.handle, a.ctypes.data, a.size), "crl_model_get_amax")
-        return a.reshape(self.n_layer, 5)
+        return a.reshape(rows, 5)
 
     def set_amax(self, a):
         a = np.ascontiguousarray(np.asarray(a, np.float32).reshape(-1))
@@ -371,6 +379,9 @@ class _ModelBase:
         return OrderedDict((k, v.clone()) for k, v in self._sd.items())
 
     def load_state_dict(self, sd, strict=True):
+        # transformer_engine's Linear (model_fp8.py:43-45,90-92,140) stores its fp8 recipe state under '<module>._extra_state':
+        # not weights, skipped. (The scales used here come from calibrate().)
+        sd = OrderedDict((k, v) for k, v in sd.items() if not k.endswith("_extra_state"))
         missing = [k for k in self._shapes if k not in sd and k != "transformer.wte.weight"]
         unexpected = [k for k in sd if k not in self._shapes]
         if strict and (missing or unexpected):
@@ -378,7 +389,10 @@ class _ModelBase:
         for k, shp in self._shapes.items():
             if k in sd:
                 t = sd[k].detach().to("cpu", torch.float32)
-                if tuple(t.shape) != tuple(shp) and not (k == "pe" and t.shape[0] >= 64 and t.shape[1] == shp[1]):
+                # pe may have more rows than used; lm_head / wte may carry padding rows behind the 1929 moves
+                # (pretrain_fp8.py:16 trains with vocab_size 1936)
+                grows = (k == "pe" and t.shape[0] >= 64) or (k in ("lm_head.weight", "transformer.wte.weight") and t.shape[0] >= VOCAB_RL)
+                if tuple(t.shape) != tuple(shp) and not (grows and t.dim() == 2 and t.shape[1] == shp[1]):
                     raise RuntimeError("load_state_dict: %s has shape %s, expected %s" % (k, tuple(t.shape), tuple(shp)))
                 self._sd[k] = t.clone()
         if "lm_head.weight" in self._sd:
@@ -490,9 +504,12 @@ class GPTConfig:
 class GPT(_ModelBase):
     """model_bis.GPT for the 64 board tokens (model_bis.py:125-199, 358-398)."""
 
-    def __init__(self, config, fp8=False, micro_batch=0, stream_f32=True, head_dtype=None, act_dtype="bf16", seed=0):
-        if config.vocab_size != VOCAB_RL:
-            raise ValueError("vocab_size must be %d (utils/vocab.py)" % VOCAB_RL)
+    def __init__(self, config, fp8=False, micro_batch=0, stream_f32=True, head_dtype=None, act_dtype="bf16", seed=0,
+                 norm_rms=False, fp8_lm_head=None):
+        # vocab_size above 1929 (pretrain_fp8.py:16 pads to 1936 for the fp8 GEMM) adds rows to lm_head / wte that no
+        # move uses: they are kept in the state dict, count towards the e4m3 weight scale, and the logits stay 1929 wide.
+        if config.vocab_size < VOCAB_RL:
+            raise ValueError("vocab_size must be at least %d (utils/vocab.py)" % VOCAB_RL)
         if not config.bias:
             raise ValueError("bias=False is not supported")
         self.config = config
@@ -506,7 +523,8 @@ class GPT(_ModelBase):
         from_pe[:, 1::2] = torch.cos(pos * div)
         self._sd["pe"] = from_pe
         self._engine = _Engine(_lib.ARCH_GPT64, config.n_layer, config.n_embd, config.n_head, 4 * config.n_embd,
-                               fp8=fp8, micro_batch=micro_batch, stream_f32=stream_f32, head_dtype=head_dtype, act_dtype=act_dtype)
+                               fp8=fp8, micro_batch=micro_batch, stream_f32=stream_f32, head_dtype=head_dtype, act_dtype=act_dtype,
+                               norm_rms=norm_rms, fp8_lm_head=fp8_lm_head)
         self._engine.load(self._sd)
 
     def get_num_params(self, non_embedding=True):
@@ -579,37 +597,37 @@ class GPT(_ModelBase):
 class BT4(_ModelBase):
     """new_paradigm/value.py BT4 (value.py:121-400)."""
 
-    def __init__(self, num_layers=10, d_model=512, d_ff=736, num_heads=8, fp8=False, micro_batch=0, head_dtype=None, act_dtype="bf16", seed=0):
+    def __init__(self, num_layers=10, d_model=512, d_ff=736, num_heads=8, fp8=False, micro_batch=0, head_dtype=None, act_dtype="bf16", seed=0,
+                 stream_f32=None, norm_rms=False):
         self.num_layers, self.d_model = num_layers, d_model
         self._shapes = bt4_shapes(num_layers, d_model, d_ff, num_heads)
         self._sd = _default_init(self._shapes, seed)
-        self._engine = _Engine(_lib.ARCH_BT4, num_layers, d_model, num_heads, d_ff, fp8=fp8, micro_batch=micro_batch, head_dtype=head_dtype, act_dtype=act_dtype)
+        self._engine = _Engine(_lib.ARCH_BT4, num_layers, d_model, num_heads, d_ff, fp8=fp8, micro_batch=micro_batch, head_dtype=head_dtype,
+                               act_dtype=act_dtype, stream_f32=stream_f32, norm_rms=norm_rms)
         self._engine.load(self._sd)
 
     @torch.no_grad()
     def forward(self, inp, compute_loss=False):
-        """inp[0]: [b, seq_len, 8, 8, 19] -> policy [b, seq_len, 1929] (value.py:155-212)."""
-        if compute_loss:
-            raise NotImplementedError("losses are not part of the forward path")
+        """inp[0]: [b, seq_len, 8, 8, 19] -> policy [b, seq_len, 1929] (value.py:155-212). With compute_loss the
+        reference's 6-tuple (value.py:197-202): inp[1] = policy targets [b, seq_len] (ignore_index 1928), inp[3] = value
+        classes [b, seq_len, 1] (ignore_index 3) -> (policy, value logits [b, seq_len, 3], policy cross-entropy, value
+        cross-entropy, targets, true_values). Forward values only: the losses carry no autograd graph."""
         x = inp[0]
         b, s = x.shape[0], x.shape[1]
-        pol, _ = self._engine.forward(x, want_wdl=False)
-        return pol.view(b, s, VOCAB_RL)
+        pol, wdl = self._engine.forward(x, want_wdl=compute_loss)
+        policy = pol.view(b, s, VOCAB_RL)
+        if not compute_loss:
+            return policy
+        targets, true_values = inp[1], inp[3]
+        if true_values.shape[-1] != 1:
+            # value.py:203-211 flattens a [b, 3] float target into F.cross_entropy's class-index slot, which torch rejects
+            raise ValueError("value targets must be class indices of shape [..., 1] (the branch of value.py:200-202)")
+        value_h = wdl.view(b, s, 3)
+        loss_policy = cross_entropy(pol, targets.reshape(-1).to(pol.device), ignore_index=1928)
+        loss_value = cross_entropy(wdl, true_values.reshape(-1).to(pol.device), ignore_index=3)
+        return policy, value_h, loss_policy, loss_value, targets, true_values
 
     __call__ = forward
-
-    @torch.no_grad()
-    def generate_sequence(self, board, T=1, seed=0):
-        """model_bis.py:213-263: (sequences [B,192], probs [B,191,1929] or None for T == 0), with the forced
-        </thinking> and end tokens. Keys and values of the prefix are cached instead of recomputed per token."""
-        seq, probs = self._engine.generate(board, self.config.block_size - 65, T, seed, rules=True, want_step_out=T != 0)
-        return seq, probs
-
-    @torch.no_grad()
-    def generate_sequence_raw(self, board, T=1, return_logits=False, seed=0):
-        """model_bis.py:266-311: as generate_sequence without the forced tokens; the per-step output is the
-        probabilities or, with return_logits, the logits."""
-        return self._engine.generate(board, self.config.block_size - 65, T, seed, rules=False, want_step_out=T != 0, out_logits=return_logits)
 
     @torch.no_grad()
     def get_move_from_fen_no_thinking(self, fen, T=1, device="cuda", force_legal=True, return_probs=False):
@@ -660,12 +678,14 @@ class BT4Class(_ModelBase):
     attention policy gathered to the 1858 side-to-move-frame moves, WDL head."""
 
     def __init__(self, num_layers=15, d_model=1024, d_ff=1536, num_heads=32, fp8=False, micro_batch=0,
-                 head_dtype=None, act_dtype="bf16", compress=32, hidden=256, gen=256, seed=0):
+                 head_dtype=None, act_dtype="bf16", compress=32, hidden=256, gen=256, seed=0, stream_f32=None, ln_fold=None,
+                 norm_rms=False):
         self.num_layers, self.d_model = num_layers, d_model
         self._shapes = bt4_shapes(num_layers, d_model, d_ff, num_heads, True, compress, hidden, gen)
         self._sd = _default_init(self._shapes, seed)
         self._engine = _Engine(_lib.ARCH_BT4CLASS, num_layers, d_model, num_heads, d_ff, fp8=fp8, micro_batch=micro_batch,
-                               head_dtype=head_dtype, act_dtype=act_dtype, compress=compress, hidden=hidden, gen=gen)
+                               head_dtype=head_dtype, act_dtype=act_dtype, compress=compress, hidden=hidden, gen=gen,
+                               stream_f32=stream_f32, ln_fold=ln_fold, norm_rms=norm_rms)
         self._engine.load(self._sd)
 
     @torch.no_grad()
@@ -674,19 +694,6 @@ class BT4Class(_ModelBase):
         return self._engine.forward(board_tokens)
 
     __call__ = forward
-
-    @torch.no_grad()
-    def generate_sequence(self, board, T=1, seed=0):
-        """model_bis.py:213-263: (sequences [B,192], probs [B,191,1929] or None for T == 0), with the forced
-        </thinking> and end tokens. Keys and values of the prefix are cached instead of recomputed per token."""
-        seq, probs = self._engine.generate(board, self.config.block_size - 65, T, seed, rules=True, want_step_out=T != 0)
-        return seq, probs
-
-    @torch.no_grad()
-    def generate_sequence_raw(self, board, T=1, return_logits=False, seed=0):
-        """model_bis.py:266-311: as generate_sequence without the forced tokens; the per-step output is the
-        probabilities or, with return_logits, the logits."""
-        return self._engine.generate(board, self.config.block_size - 65, T, seed, rules=False, want_step_out=T != 0, out_logits=return_logits)
 
     @torch.no_grad()
     def get_move_from_fen_no_thinking(self, fen, T=1, device="cuda", force_legal=True, return_probs=False):

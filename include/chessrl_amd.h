@@ -53,6 +53,10 @@ extern "C" {
 
 const char* crl_last_error(void);
 const char* crl_version(void);
+/* Frees the device memory the library keeps outside any model handle: the 64 MB K-slice workspaces crl_gemm allocates per
+ * stream, a 256-byte block of zeros per device and the move maps of crl_leela_to_rl. Call it with no library work in
+ * flight; later calls allocate again on demand. Models are freed by crl_model_destroy. */
+void crl_shutdown(void);
 
 /* ------------------------------------------------------------------ host: vocabulary */
 /* utils/vocab.py:9-227 / :229-438 — i-th move string (static storage), NULL if out of range. */
@@ -116,6 +120,10 @@ int crl_gemm(const void* A, int64_t lda, const void* W, int64_t ldw, void* C, in
 int crl_layernorm(const void* x, int64_t ldx, int in_dtype, const float* gamma, const float* beta,
                   void* out, int out_dtype, uint8_t* out_fp8, float fp8_scale, int64_t ldo,
                   int rows, int C, float eps, float* amax, void* stream);
+/* RMSNorm, x / sqrt(mean(x^2) + eps) * gamma, with the same outputs as crl_layernorm. The reference's models use
+ * LayerNorm only (model_bis.py:25-34, new_paradigm/value.py:36-37); this is the norm crl_model_config.norm_rms selects. */
+int crl_rmsnorm(const void* x, int64_t ldx, int in_dtype, const float* gamma, void* out, int out_dtype, uint8_t* out_fp8,
+                float fp8_scale, int64_t ldo, int rows, int C, float eps, float* amax, void* stream);
 /* Attention over 64 tokens per position, q/k/v of in_dtype (bf16 or f16) with head h at columns [h*head_dim, ...).
  * mode CAUSAL: model_bis.py:71; RELSHIFT: new_paradigm/attn.py:507-521 with pos = pos_proj(PE)
  * (in_dtype [64,H*head_dim]) and u_bias/v_bias fp32[H*head_dim]; BIAS: bias of in_dtype [B,H,64,64] in the
@@ -145,12 +153,19 @@ typedef struct crl_model_config {
   int32_t d_ff;
   int32_t fp8;            /* 1: trunk linears (qkv, out-proj, ffn) run in e4m3 with static per-tensor scales */
   int32_t micro_batch;    /* positions per pass through the trunk; 0 = default */
-  int32_t stream_f32;     /* GPT64 only: keep the residual stream in fp32 (default 1) */
+  int32_t stream_f32;     /* residual stream (the tensors the residual additions and the norms read) in fp32 instead of
+                             the 16-bit type: 0 = default (fp32 for GPT64, 16-bit for BT4 and BT4-class), 1 = fp32,
+                             -1 = 16-bit. The GEMM operands stay 16-bit / e4m3 either way. */
   int32_t head_dtype;     /* CRL_BF16 or CRL_F16: element type of the policy/value head GEMM inputs; 0 = act_dtype */
   int32_t smolgen_compress, smolgen_hidden, smolgen_gen;  /* BT4-class; 0 = 32/256/256 */
   float eps;              /* LayerNorm epsilon; 0 = 1e-5 */
   int32_t act_dtype;      /* CRL_BF16 (default) or CRL_F16: 16-bit element type of activations and weights */
-  int32_t reserved[3];
+  int32_t ln_fold;        /* e4m3 BT4-class with a 16-bit bf16 stream: the trunk norms write only their e4m3 copy and row
+                             statistics, and the product that takes the normalised tensor as its residual normalises it
+                             in its epilogue. 0 = default (on), -1 = off (every norm writes its 16-bit output). */
+  int32_t norm_rms;       /* 1: the norms of the trunk (and GPT64's ln_f) are RMSNorm, x/sqrt(mean(x^2)+eps)*weight; their
+                             .bias entries are accepted and ignored. 0 = LayerNorm as in the reference. */
+  int32_t fp8_lm_head;    /* GPT64 with fp8: lm_head runs in e4m3 as well (model_fp8.py:140). 0 = default (on), -1 = 16-bit. */
 } crl_model_config;
 
 /* GPT(config) / BT4(...) constructors (model_bis.py:127-157, new_paradigm/value.py:122-152). */
@@ -168,7 +183,8 @@ int crl_model_finalize(crl_model* m);
  * is one calibration batch). Synchronises the stream. */
 int crl_model_calibrate(crl_model* m, const float* planes, int B, void* stream);
 /* Read / overwrite the activation amax table, float[n_layer*5]: per layer the input of q|k|v, the attention output,
- * the inputs of the two FFN linears and the input of the shared attention-bias generator (BT4-class only, else 0). */
+ * the inputs of the two FFN linears and the input of the shared attention-bias generator (BT4-class only, else 0).
+ * With n = (n_layer+1)*5 the table carries one more row whose first entry is the amax of lm_head's input (GPT64). */
 int crl_model_get_amax(crl_model* m, float* out, int n);
 int crl_model_set_amax(crl_model* m, const float* in, int n);
 /* The forward pass. planes: device f32 [B,64,19] (GPT.forward batch[0] / BT4.forward inp[0]).
@@ -212,7 +228,10 @@ int crl_model_set_decode_graph(crl_model* m, int on);
  * softmax((logits + (1-mask)*-999)/temperature) (one-hot at the arg-max for temperature 0), wdl [n,3] the value
  * logits, best [n] the index of the best legal move; each may be NULL. V and the move order are those of the model
  * (1929 / crl_policy_index, or 1858 side-to-move-frame / crl_policy_leela for CRL_ARCH_BT4CLASS). One call at a time
- * per model; the staging buffers (2 chunks, pinned + device) stay with the model until it is destroyed. */
+ * per model; the staging buffers (2 chunks, pinned + device) stay with the model until it is destroyed. The call runs
+ * on streams of its own: it first waits for everything queued on the device (hipDeviceSynchronize), so forwards issued
+ * earlier on any stream of this model are complete before it touches the model's workspace, and it returns with its own
+ * work finished. crl_model_search_1ply behaves the same way. */
 int crl_model_evaluate_fens(crl_model* m, const char* const* fens, int n, int chunk, float temperature, float* probs,
                             float* wdl, int32_t* best, int threads);
 /* Batched 1-ply value search: BT4.calculate_move_values / get_best_move_value (new_paradigm/value.py:319-400) for n root

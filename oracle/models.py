@@ -13,12 +13,15 @@ What each class follows (reference file:line):
                  :402-435 (value head); new_paradigm/attn.py:445-533 (relative attention).
   BT4ClassOracle the BT4-class configuration of the benchmark (15x1024x32h, mish FFN 1536,
                  generated attention bias, gathered 1858-move policy, WDL head). It is NOT in
-                 the reference repository; this module is its definition. PARITY UNPINNED:
-                 self-consistency only.
-  fp8 emulation  model_fp8.py:43,45,90,92,140 + pretrain_fp8.py:75-79 run the linears through
-                 transformer_engine (not vendored, not installable here): per-tensor e4m3
-                 scaling of input and weight, high-precision accumulate. Restated as
-                 quantise->dequantise->F.linear. PARITY UNPINNED against transformer_engine.
+                 the reference repository (the reference only names the external lczero-training
+                 package, not vendored, no pinned version); this module is its definition, so no
+                 vector of a reference implementation can exist for it.
+  fp8 emulation  model_fp8.py:43,45,90,92,140 + pretrain_fp8.py:75-79 run the linears (lm_head
+                 included) through transformer_engine (not vendored, not installable here):
+                 per-tensor e4m3 scaling of input and weight, high-precision accumulate.
+                 Restated as quantise->dequantise->F.linear. PARITY UNPINNED against
+                 transformer_engine itself; the arithmetic is pinned as listed below.
+  rms_norm       the RMSNorm alternative of the trunk norms (no reference model uses it).
 
 Pins: GPTOracle (64-token forward, token forward, loss), BT4Oracle (policy and value) and
 relative_attention are checked in tests/test_golden.py against outputs of the reference's own
@@ -26,7 +29,18 @@ module code on the same weights and inputs (tests/golden/reference_vectors.npz, 
 tests/golden/make_vectors.py). Library routines (F.layer_norm, F.gelu,
 F.scaled_dot_product_attention) are used directly; the relative shift is also pinned in
 tests/test_oracle.py against the pad/reshape formulation and a brute-force definition; the move
-lists are pinned by SHA-256. BT4ClassOracle and the fp8 emulation have no such vectors.
+lists are pinned by SHA-256.
+BT4ClassOracle is pinned in tests/test_oracle.py by what its definition fixes: the policy gather
+by an independent per-move-string loop over all 1858 moves for a white and a black row (squares,
+rank mirror, promotion pieces and their offsets); the attention by F.scaled_dot_product_attention
+when the generated bias is zero and by a head-by-head loop with a hand-built bias otherwise
+(a transposed bias tile is shown to fail); the residual scale (2L)^-1/4, norm placement and
+mish position by a two-layer composition from plain tensor operations; the value head's
+token-major flatten likewise.
+fp8_quant_dequant / Fp8Plan are pinned against a table of all 256 e4m3fn codes built from the
+format's definition with an explicit nearest-even search (ties, subnormals, saturation), and the
+plan's linear against quantise-dequantise-matmul written out with that table; rms_norm against
+torch.nn.functional.rms_norm.
 """
 import math
 
@@ -56,16 +70,28 @@ class Fp8Plan:
     shared attention-bias generator (BT4-class)."""
 
     def __init__(self, n_layer):
+        self.n_layer = n_layer
         self.amax = torch.zeros(n_layer, 5)
+        self.head_amax = torch.zeros(1)     # input of lm_head (model_fp8.py:140); addressed as layer == n_layer, slot 0
         self.recording = False
 
-    def lin(self, x, layer, slot, weight, bias):
+    def lin(self, x, layer, slot, weight, bias, weight_amax=None):
+        """weight_amax: amax of the whole weight tensor when `weight` is a slice of it (padded vocabulary rows)."""
+        cell = self.head_amax[0:1] if layer == self.n_layer else self.amax[layer, slot:slot + 1]
         if self.recording:
-            self.amax[layer, slot] = max(self.amax[layer, slot].item(), x.abs().max().item())
+            cell[0] = max(cell.item(), x.abs().max().item())
             return F.linear(x, weight, bias)
-        sx = amax_scale(self.amax[layer, slot].item())
-        sw = amax_scale(weight.abs().max().item())
+        sx = amax_scale(cell.item())
+        sw = amax_scale(weight.abs().max().item() if weight_amax is None else weight_amax)
         return F.linear(fp8_quant_dequant(x, sx), fp8_quant_dequant(weight, sw), bias)
+
+    def table(self, head=False):
+        """numpy [n_layer, 5], or [n_layer + 1, 5] with the lm_head row appended (the library's layout)."""
+        if not head:
+            return self.amax.numpy().copy()
+        last = torch.zeros(1, 5)
+        last[0, 0] = self.head_amax[0]
+        return torch.cat([self.amax, last]).numpy()
 
 
 def _lin(plan, x, layer, slot, mod):
@@ -75,6 +101,16 @@ def _lin(plan, x, layer, slot, mod):
 
 
 # ------------------------------------------------------------------ shared pieces
+def rms_norm(x, weight, eps=1e-5):
+    """RMSNorm: x / sqrt(mean(x^2) + eps) * weight (no mean subtraction, no offset). Not used by any reference model;
+    it is the alternative norm the benchmark text names. Pinned against torch.nn.functional.rms_norm in tests/test_oracle.py."""
+    return x * torch.rsqrt(x.pow(2).mean(-1, keepdim=True) + eps) * weight
+
+
+def _norm(mod, x, rms):
+    return rms_norm(x, mod.weight, 1e-5) if rms else mod(x)
+
+
 class MaGating(nn.Module):
     def __init__(self, d_model):
         super().__init__()
@@ -155,9 +191,9 @@ class _GPTBlock(nn.Module):
 
 
 class GPTOracle(nn.Module):
-    def __init__(self, n_layer=6, n_head=8, n_embd=256, block_size=256, vocab_size=VOCAB_RL):
+    def __init__(self, n_layer=6, n_head=8, n_embd=256, block_size=256, vocab_size=VOCAB_RL, rms=False):
         super().__init__()
-        self.n_layer, self.n_head, self.n_embd = n_layer, n_head, n_embd
+        self.n_layer, self.n_head, self.n_embd, self.rms = n_layer, n_head, n_embd, rms
         self.FenEncoder = Stem(n_embd)
         self.transformer = nn.ModuleDict(dict(
             wte=nn.Embedding(vocab_size, n_embd),
@@ -171,22 +207,30 @@ class GPTOracle(nn.Module):
         B, T, C = x.shape
         H = self.n_head
         for li, blk in enumerate(self.transformer.h):
-            h = blk.ln_1(x)
+            h = _norm(blk.ln_1, x, self.rms)
             q, k, v = _lin(plan, h, li, 0, blk.attn.c_attn).split(C, dim=2)
             q, k, v = (t.view(B, T, H, C // H).transpose(1, 2) for t in (q, k, v))
             y = F.scaled_dot_product_attention(q, k, v, is_causal=True)
             y = y.transpose(1, 2).reshape(B, T, C)
             x = x + _lin(plan, y, li, 1, blk.attn.c_proj)
-            h = blk.ln_2(x)
+            h = _norm(blk.ln_2, x, self.rms)
             f = F.gelu(_lin(plan, h, li, 2, blk.mlp.c_fc))
             x = x + _lin(plan, f, li, 3, blk.mlp.c_proj)
-        return self.transformer.ln_f(x)
+        return _norm(self.transformer.ln_f, x, self.rms)
+
+    def _head(self, x, plan=None):
+        """lm_head on the 1929 move rows; under the fp8 plan it is an e4m3 linear too (model_fp8.py:140) whose
+        per-tensor weight scale covers every row of the (possibly padded, pretrain_fp8.py:16) weight."""
+        w = self.lm_head.weight
+        if plan is None:
+            return F.linear(x, w[:VOCAB_RL])
+        return plan.lin(x, self.n_layer, 0, w[:VOCAB_RL], None, weight_amax=w.abs().max().item())
 
     @torch.no_grad()
     def forward_last(self, planes, plan=None):
         """planes [B,8,8,19] -> logits [B,1929] of token 63 (model_bis.py:360-370)."""
         x = self._trunk(self.FenEncoder(planes) + self.pe[:64], plan)
-        return self.lm_head(x[:, -1, :])
+        return self._head(x[:, -1, :], plan)
 
     @torch.no_grad()
     def forward_tokens(self, planes, idx, compute_loss=False):
@@ -292,9 +336,9 @@ def relative_attention(at, x, pe, H):
 
 
 class BT4Oracle(nn.Module):
-    def __init__(self, num_layers=10, d_model=512, d_ff=736, num_heads=8):
+    def __init__(self, num_layers=10, d_model=512, d_ff=736, num_heads=8, rms=False):
         super().__init__()
-        self.num_layers, self.d_model, self.num_heads = num_layers, d_model, num_heads
+        self.num_layers, self.d_model, self.num_heads, self.rms = num_layers, d_model, num_heads, rms
         self.layers = nn.ModuleList([_BT4Layer(d_model, d_ff, num_heads) for _ in range(num_layers)])
         self.linear1 = nn.Linear(19, d_model)
         self.layernorm1 = nn.LayerNorm(d_model)
@@ -315,9 +359,9 @@ class BT4Oracle(nn.Module):
         H = self.num_heads
         pe = self.pe
         for ly in self.layers:
-            x = ly.norm1(relative_attention(ly.attention, x, pe, H) + x)
+            x = _norm(ly.norm1, relative_attention(ly.attention, x, pe, H) + x, self.rms)
             y = F.gelu(ly.ff2(ly.ff1(x)))
-            x = ly.norm2(y + x)
+            x = _norm(ly.norm2, y + x, self.rms)
         wdl = self.value_head(x, F.gelu)
         pt = F.gelu(self.policy_tokens_lin(x)) + pe
         qk = torch.matmul(self.queries_pol(pt), self.keys_pol(pt).transpose(-2, -1)) / math.sqrt(C)
@@ -372,9 +416,9 @@ def leela_gather_tables(policy_leela):
 
 class BT4ClassOracle(nn.Module):
     def __init__(self, policy_leela, num_layers=15, d_model=1024, d_ff=1536, num_heads=32,
-                 compress=32, hidden=256, gen=256):
+                 compress=32, hidden=256, gen=256, rms=False):
         super().__init__()
-        self.num_layers, self.d_model, self.num_heads = num_layers, d_model, num_heads
+        self.num_layers, self.d_model, self.num_heads, self.rms = num_layers, d_model, num_heads, rms
         self.layers = nn.ModuleList([_BT4ClassLayer(d_model, d_ff, num_heads, compress, hidden, gen)
                                      for _ in range(num_layers)])
         self.smol_weight_gen = nn.Linear(gen, 64 * 64, bias=False)
@@ -397,7 +441,7 @@ class BT4ClassOracle(nn.Module):
         B, T, C = x.shape
         H = self.num_heads
         hs = C // H
-        alpha = (2.0 * self.num_layers) ** -0.25
+        alpha = (2.0 * self.num_layers) ** -0.25 if self.num_layers else 1.0
         for li, ly in enumerate(self.layers):
             at, sm = ly.attention, ly.smolgen
             if plan is None:
@@ -414,9 +458,9 @@ class BT4ClassOracle(nn.Module):
             q, k, v = (t.view(B, T, H, hs).transpose(1, 2) for t in (q, k, v))
             score = torch.matmul(q, k.transpose(-2, -1)) / math.sqrt(hs) + bias
             ctx = torch.matmul(F.softmax(score, -1), v).transpose(1, 2).reshape(B, T, C)
-            x = ly.norm1(x + alpha * _lin(plan, ctx, li, 1, at.out_proj))
+            x = _norm(ly.norm1, x + alpha * _lin(plan, ctx, li, 1, at.out_proj), self.rms)
             f = F.mish(_lin(plan, x, li, 2, ly.ff1))
-            x = ly.norm2(x + alpha * _lin(plan, f, li, 3, ly.ff2))
+            x = _norm(ly.norm2, x + alpha * _lin(plan, f, li, 3, ly.ff2), self.rms)
         wdl = self.value_head(x, F.mish)
         tok = F.mish(self.policy_tokens_lin(x))
         qp, kp = self.queries_pol(tok), self.keys_pol(tok)

@@ -176,3 +176,48 @@ def test_no_cpu_fallback():
     m = models.GPT(models.GPTConfig(block_size=256, vocab_size=1929, n_layer=1, n_head=8, n_embd=256))
     with pytest.raises(_lib.CrlError):
         m.forward((torch.zeros(1, 8, 8, 19), None))
+
+
+def test_late_game_positions_match_python_oracle():
+    """The rollout-scoring sweep draws 30 % of its positions from playouts continued until at most 10 pieces remain
+    (sparser legal masks): planes, both masks and the piece counts against the pure-Python rules."""
+    r = board.random_positions(1, 120, late_fraction=0.3, fens=True, masks_rl=True, masks_leela=True)
+    late = 0
+    for i, fen in enumerate(r["fens"]):
+        pieces = sum(ch.isalpha() for ch in fen.split()[0])
+        late += pieces <= 10
+        assert np.array_equal(r["planes"][i], np.array(chess_py.fen_to_planes(fen), np.float32)), fen
+        assert r["masks_rl"][i].tolist() == chess_py.legal_mask(fen, vocab.policy_index), fen
+        assert r["masks_leela"][i].tolist() == chess_py.legal_mask_leela(fen, vocab.policy_leela), fen
+    assert 20 <= late <= 55, late           # about 30 % of 120
+    # the same seed without the late-game share leaves the other positions untouched in kind: none forced to <= 10 pieces
+    base = board.random_positions(1, 120, fens=True)["fens"]
+    assert sum(sum(ch.isalpha() for ch in f.split()[0]) <= 10 for f in base) < late
+    # seeded: the same call gives the same positions
+    again = board.random_positions(1, 120, late_fraction=0.3, fens=True)["fens"]
+    assert again == r["fens"]
+
+
+def test_fp8_checkpoint_layout_loads():
+    """A checkpoint of the reference's fp8 model (model_fp8.py, trained by pretrain_fp8.py:12-17 with vocab_size 1936):
+    lm_head / wte carry 7 padding rows, and transformer_engine's Linear modules add '<module>._extra_state' entries.
+    Both load; the first 1929 rows are the moves."""
+    import torch
+    cfg = models.GPTConfig(block_size=256, vocab_size=1936, n_layer=1, n_head=8, n_embd=256)
+    m = models.GPT(cfg, fp8=True)
+    sd = m.state_dict()
+    assert sd["lm_head.weight"].shape == (1936, 256) and sd["transformer.wte.weight"].shape == (1936, 256)
+    g = torch.Generator().manual_seed(0)
+    sd["lm_head.weight"] = torch.randn(1936, 256, generator=g) * 0.02
+    sd["transformer.wte.weight"] = sd["lm_head.weight"]
+    for mod in ("transformer.h.0.attn.c_attn", "transformer.h.0.attn.c_proj", "transformer.h.0.mlp.c_fc", "transformer.h.0.mlp.c_proj", "lm_head"):
+        sd[mod + "._extra_state"] = torch.zeros(8, dtype=torch.uint8)
+    m.load_state_dict(sd)                                   # strict
+    assert torch.equal(m.state_dict()["lm_head.weight"], sd["lm_head.weight"])
+    with pytest.raises(RuntimeError):
+        m.load_state_dict({**sd, "something.else": torch.zeros(1)})
+    with pytest.raises(ValueError):
+        models.GPT(models.GPTConfig(block_size=256, vocab_size=1900, n_layer=1, n_head=8, n_embd=256))
+    # a 1929-row checkpoint still loads into a 1929-row model, and a padded one into it as well (rows beyond 1929 ignored by the logits)
+    m2 = models.GPT(models.GPTConfig(block_size=256, vocab_size=1929, n_layer=1, n_head=8, n_embd=256))
+    m2.load_state_dict(sd)

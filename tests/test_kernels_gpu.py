@@ -429,3 +429,55 @@ def test_sample_distribution_and_argmax(cuda):
     t0 = torch.empty(64, dtype=torch.int64, device=cuda)
     check(lib().crl_sample(p(x), 1929, 64, 1929, 0.0, 0, 0, p(t0), None, st))
     assert bool((t0 == 7).all())
+
+
+@pytest.mark.parametrize("C_,in_dt", [(256, _lib.F32), (1024, _lib.BF16), (8192, _lib.BF16), (1536, _lib.F16)])
+def test_rmsnorm(cuda, C_, in_dt):
+    """crl_rmsnorm against torch.nn.functional.rms_norm on the same (rounded) input."""
+    torch.manual_seed(C_ + 1)
+    rows = 53
+    x = (torch.randn(rows, C_, device=cuda) * 2 + 0.5).to(TORCH_DT[in_dt])
+    g = torch.randn(C_, device=cuda)
+    out = torch.zeros(rows, C_, dtype=torch.float32, device=cuda)
+    out8 = torch.zeros(rows, C_, dtype=torch.uint8, device=cuda)
+    amax = torch.zeros(1, device=cuda)
+    check(lib().crl_rmsnorm(p(x), C_, in_dt, p(g), p(out), _lib.F32, p(out8), 7.0, C_, rows, C_, 1e-5, p(amax), stream()), "rms")
+    torch.cuda.synchronize()
+    ref = F.rms_norm(x.float(), (C_,), g, 1e-5)
+    assert torch.allclose(out, ref, rtol=1e-5, atol=1e-5), (out - ref).abs().max()
+    assert abs(amax.item() - ref.abs().max().item()) < 1e-4 * ref.abs().max().item()
+    # the e4m3 copy is the fp32 output times the scale, rounded as torch rounds
+    assert torch.equal(out8, (out * 7.0).clamp(-448, 448).to(torch.float8_e4m3fn).view(torch.uint8))
+
+
+def test_fp8_conversion_matches_torch_bit_for_bit(cuda):
+    """The kernels' e4m3 conversion (saturating, round to nearest even) against torch.float8_e4m3fn on every finite bf16
+    value: through the GEMM epilogue (A = all 65280 finite bf16 patterns, W = identity, so the accumulator is the input
+    itself) and through the LayerNorm kernel's e4m3 output (fp32 output times scale)."""
+    bits = torch.arange(65536, dtype=torch.int32, device=cuda)
+    finite = bits[((bits >> 7) & 0xFF) != 0xFF]
+    pad = (-finite.numel()) % 128
+    finite = torch.cat([finite, finite[:pad]])
+    A = finite.to(torch.int16).view(torch.bfloat16).view(-1, 128).contiguous()
+    W = torch.eye(128, device=cuda, dtype=torch.bfloat16)
+    def canon(c):            # a sum that starts at +0 cannot end at -0: compare zeros without their sign
+        return torch.where(c == 0x80, torch.zeros_like(c), c)
+
+    for tile in (1, 2, 3):
+        q = run_gemm(A, W, _lib.FP8, tile=tile)
+        want = A.float().clamp(-448, 448).to(torch.float8_e4m3fn).view(torch.uint8)
+        assert torch.equal(canon(q), canon(want)), (tile, (canon(q) != canon(want)).sum().item())
+    # with an output scale (the multiply is fp32 in both)
+    q = run_gemm(A, W, _lib.FP8, out_scale=3.0, tile=3)
+    assert torch.equal(canon(q), canon((A.float() * 3.0).clamp(-448, 448).to(torch.float8_e4m3fn).view(torch.uint8)))
+    # LayerNorm kernel: its e4m3 copy equals its own fp32 output times the scale, converted by torch
+    torch.manual_seed(0)
+    x = torch.randn(300, 1024, device=cuda) * torch.logspace(-3, 3, 300, device=cuda).unsqueeze(1)
+    g = torch.randn(1024, device=cuda) * 30
+    b = torch.randn(1024, device=cuda)
+    out = torch.zeros(300, 1024, device=cuda)
+    out8 = torch.zeros(300, 1024, dtype=torch.uint8, device=cuda)
+    check(lib().crl_layernorm(p(x), 1024, _lib.F32, p(g), p(b), p(out), _lib.F32, p(out8), 5.0, 1024, 300, 1024, 1e-5, None, stream()), "ln")
+    torch.cuda.synchronize()
+    assert torch.equal(out8, (out * 5.0).clamp(-448, 448).to(torch.float8_e4m3fn).view(torch.uint8))
+    assert (out.abs() * 5.0 > 448).any()          # the sweep reaches the saturating range

@@ -17,6 +17,10 @@ def positions(n, seed=1, leela=False):
     return torch.from_numpy(r["planes"]), torch.from_numpy(r["masks_leela" if leela else "masks_rl"])
 
 
+def r_planes_cpu(r):
+    return torch.from_numpy(r["planes"])
+
+
 def rel_rms(a, b):
     return ((a - b).pow(2).mean().sqrt() / b.pow(2).mean().sqrt()).item()
 
@@ -89,6 +93,22 @@ def test_bt4_torch(cuda, cfg, act="bf16"):
     assert top1_agreement(pol, rpol, mask) >= 0.98
 
 
+def test_bt4_fp32_stream(cuda):
+    """BT4 with the residual stream kept in fp32 (16-bit GEMM operands): closer to the oracle than the 16-bit stream."""
+    oracle = om.test_init_(om.BT4Oracle(10, 512, 736, 8), seed=1)
+    planes, mask = positions(96, seed=2)
+    rpol, rwdl = oracle.forward_pv(planes)
+    errs = {}
+    for sf in (False, True):
+        m = models.BT4(10, 512, 736, 8, stream_f32=sf)
+        m.load_state_dict(oracle.state_dict())
+        pol, wdl = m._engine.forward(planes.to(cuda))
+        report("bt4 10x512 bf16 stream %s" % ("fp32" if sf else "bf16"), pol.cpu(), rpol, mask, wdl.cpu(), rwdl)
+        errs[sf] = rel_rms(pol.cpu(), rpol)
+        assert (wdl.cpu() - rwdl).abs().max() <= 1e-2
+    assert errs[True] < errs[False] and errs[True] < 1e-2
+
+
 def test_bt4_f16(cuda):
     """The reference trains and runs this model under fp16 autocast (new_paradigm/train_value.py:38)."""
     test_bt4_torch(cuda, (10, 512, 736, 8), "f16")
@@ -147,25 +167,39 @@ def test_bt4class_batch_invariance(cuda, fp8):
     assert torch.equal(p3.cpu(), pol.cpu()[perm]) and torch.equal(w3.cpu(), wdl.cpu()[perm])
 
 
-@pytest.mark.parametrize("act", ["bf16", "f16"])
-def test_bt4class_full_size(cuda, act):
-    """The benchmark model at its real size (15 layers, d=1024, 32 heads, FFN 1536) and its benchmark
-    initialisation (normal(0, 0.02), zero biases), 256 positions.
+_FULL = {}
 
-    WDL meets the 1e-2 bar in both element types. The top-1 bar (99.5 %) cannot be met by any 16-bit
-    pipeline on THIS initialisation: the reference's top-1/top-2 logit gap has a median near 1e-3 while
-    the logits' standard deviation is 0.07, so rounding noise of 8 (bf16) or 11 (f16) significant bits
-    per stored activation is larger than most gaps. What the test pins instead: the logit error itself,
-    and that every position whose reference gap exceeds twice the largest logit error picks the same move."""
+
+def full_size_reference():
+    """The benchmark model (15 layers, d=1024, 32 heads, FFN 1536) with its benchmark initialisation, 256 seeded
+    positions and the fp32 oracle's outputs on them; computed once per test session (seconds of CPU time)."""
+    if not _FULL:
+        L, Cm, Fm, H = 15, 1024, 1536, 32
+        oracle = om.spec_init_(om.BT4ClassOracle(policy_leela, L, Cm, Fm, H), seed=0)
+        planes, mask = positions(256, seed=1, leela=True)
+        rpol, rwdl = oracle.forward_pv(planes)
+        _FULL.update(oracle=oracle, planes=planes, mask=mask, rpol=rpol, rwdl=rwdl)
+    return _FULL
+
+
+@pytest.mark.parametrize("act,stream_f32", [("bf16", False), ("f16", False), ("bf16", True), ("f16", True)])
+def test_bt4class_full_size(cuda, act, stream_f32):
+    """The benchmark model at its real size (15 layers, d=1024, 32 heads, FFN 1536) and its benchmark
+    initialisation (normal(0, 0.02), zero biases), 256 positions, with the residual stream in the 16-bit type
+    (default) and in fp32.
+
+    WDL meets the 1e-2 bar everywhere. On THIS initialisation the reference's top-1/top-2 logit gap has a median
+    near 1e-3 against a logit standard deviation of 0.07, so agreement of the arg-max measures rounding noise against
+    near-ties; the test pins the logit error itself, that every position whose reference gap exceeds twice the
+    largest logit error picks the same move, and the agreement each variant reaches."""
     L, Cm, Fm, H = 15, 1024, 1536, 32
-    oracle = om.spec_init_(om.BT4ClassOracle(policy_leela, L, Cm, Fm, H), seed=0)
-    planes, mask = positions(256, seed=1, leela=True)
-    rpol, rwdl = oracle.forward_pv(planes)
-    m = models.BT4Class(L, Cm, Fm, H, act_dtype=act)
-    m.load_state_dict(oracle.state_dict())
+    ref = full_size_reference()
+    planes, mask, rpol, rwdl = ref["planes"], ref["mask"], ref["rpol"], ref["rwdl"]
+    m = models.BT4Class(L, Cm, Fm, H, act_dtype=act, stream_f32=stream_f32)
+    m.load_state_dict(ref["oracle"].state_dict())
     pol, wdl = m(planes.to(cuda))
     pol, wdl = pol.cpu(), wdl.cpu()
-    report("bt4class full size %s" % act, pol, rpol, mask, wdl, rwdl)
+    report("bt4class full size %s stream %s" % (act, "fp32" if stream_f32 else "16-bit"), pol, rpol, mask, wdl, rwdl)
     neg = (1.0 - mask.float()) * -999.0
     top2 = (rpol + neg).topk(2, -1).values
     gap = top2[:, 0] - top2[:, 1]
@@ -175,10 +209,228 @@ def test_bt4class_full_size(cuda, act):
     print("   logit std %.3e, median gap %.3e, max logit error %.3e, decisive positions %d of %d, agreement on them %.4f, overall %.4f"
           % (rpol.std().item(), gap.median().item(), err, int(decisive.sum()), len(gap),
              same[decisive].float().mean().item() if decisive.any() else 1.0, same.float().mean().item()))
-    assert rel_rms(pol, rpol) < (4e-2 if act == "bf16" else 6e-3)
-    assert (wdl - rwdl).abs().max() <= (1e-2 if act == "bf16" else 2e-3)
+    # measured: rel-rms 2.1e-2 / 2.7e-3 / 6.4e-3 / 8.7e-4, WDL 6.2e-3 / 7.8e-4 / 2.0e-3 / 2.3e-4, top-1 74 / 94 / 88 / 98 %
+    bars = {("bf16", False): (3e-2, 1e-2, 0.70), ("f16", False): (4e-3, 2e-3, 0.91),
+            ("bf16", True): (1e-2, 4e-3, 0.85), ("f16", True): (1.5e-3, 1e-3, 0.96)}[(act, stream_f32)]
+    assert rel_rms(pol, rpol) < bars[0]
+    assert (wdl - rwdl).abs().max() <= bars[1]
     assert bool(same[decisive].all())
-    assert same.float().mean() >= (0.6 if act == "bf16" else 0.9)
+    assert same.float().mean() >= bars[2]
+
+
+@pytest.mark.parametrize("act", ["bf16", "f16"])
+def test_bt4class_heads_only_error(cuda, act):
+    """Where the full-size error comes from: the same stem and heads (d=1024, benchmark initialisation) with no trunk
+    layers in between. The policy head alone (three linears, QK^T, gather) stays an order of magnitude under the
+    15-layer figures, so the trunk's stored activations and GEMM operands are what sets them."""
+    oracle = om.spec_init_(om.BT4ClassOracle(policy_leela, 0, 1024, 1536, 32), seed=0)
+    planes, mask = positions(256, seed=1, leela=True)
+    rpol, rwdl = oracle.forward_pv(planes)
+    m = models.BT4Class(0, 1024, 1536, 32, act_dtype=act)
+    m.load_state_dict(oracle.state_dict())
+    pol, wdl = m(planes.to(cuda))
+    report("bt4class stem + heads only, %s" % act, pol.cpu(), rpol, mask, wdl.cpu(), rwdl)
+    assert rel_rms(pol.cpu(), rpol) < (6e-3 if act == "bf16" else 8e-4)
+    assert (wdl.cpu() - rwdl).abs().max() <= (4e-3 if act == "bf16" else 5e-4)
+
+
+def test_bt4class_full_size_top1_bar(cuda):
+    """The benchmark's literal bar, top-1 move agreement >= 99.5 % and WDL max-abs <= 1e-2, on the full-size model with
+    weights whose policies are not near-ties: every parameter non-trivial (biases, norm gains, per-square gating), so
+    the tokens differ by square and the reference's top-1/top-2 gap has a median of 5e-3 instead of 8e-4. f16 operands
+    meet the bar with either residual stream; bf16 operands (8 significant bits in every GEMM input) reach 97 % with
+    the fp32 stream and 89 % without, which is what their measured logit error against these gaps gives. Scaling the
+    policy head (logit standard deviation 0.05 -> 6) scales errors and gaps alike and changes none of these figures."""
+    L, Cm, Fm, H = 15, 1024, 1536, 32
+    oracle = om.test_init_(om.BT4ClassOracle(policy_leela, L, Cm, Fm, H), seed=0)
+    planes, mask = positions(256, seed=1, leela=True)
+    rpol, rwdl = oracle.forward_pv(planes)
+    got = {}
+    for act, sf in (("f16", True), ("f16", False), ("bf16", True), ("bf16", False)):
+        m = models.BT4Class(L, Cm, Fm, H, act_dtype=act, stream_f32=sf)
+        m.load_state_dict(oracle.state_dict())
+        pol, wdl = m(planes.to(cuda))
+        pol, wdl = pol.cpu(), wdl.cpu()
+        report("bt4class full size, test weights, %s stream %s" % (act, "fp32" if sf else "16-bit"), pol, rpol, mask, wdl, rwdl)
+        got[(act, sf)] = (top1_agreement(pol, rpol, mask), (wdl - rwdl).abs().max().item())
+        del m
+    assert got[("f16", True)][0] >= 0.995 and got[("f16", True)][1] <= 1e-2        # the literal bar
+    assert got[("f16", False)][0] >= 0.98 and got[("f16", False)][1] <= 1e-2
+    assert got[("bf16", True)][0] >= 0.95 and got[("bf16", True)][1] <= 1e-2
+    assert got[("bf16", False)][0] >= 0.85 and got[("bf16", False)][1] <= 1e-2
+    assert got[("bf16", True)][0] > got[("bf16", False)][0]
+
+
+@pytest.mark.parametrize("B", [1, 8, 64, 256])
+def test_bt4class_full_size_latency_batches_with_legal_masks(cuda, B):
+    """Leaf-evaluation mode on the full-size bf16 model: batches of 1, 8, 64 and 256 positions with their legal-move
+    masks applied before the softmax (model_bis.py:373-392), against masked_policy(oracle.forward_pv) on the same
+    positions."""
+    ref = full_size_reference()
+    if "m_bf16" not in ref:
+        m = models.BT4Class(15, 1024, 1536, 32)
+        m.load_state_dict(ref["oracle"].state_dict())
+        ref["m_bf16"] = m
+    m = ref["m_bf16"]
+    planes, mask = ref["planes"][:B], ref["mask"][:B]
+    probs, wdl = m.evaluate(planes.to(cuda), legal_mask=mask.to(cuda), T=1.0, want_probs=True)
+    probs, wdl = probs.cpu(), wdl.cpu()
+    want = om.masked_policy(ref["rpol"][:B], mask, 1.0)
+    assert torch.equal(probs > 0, mask.bool())
+    assert torch.allclose(probs.sum(-1), torch.ones(B), atol=1e-5)
+    err = (probs - want).abs().max().item()
+    print("bt4class bf16 B=%d masked probabilities: max-abs error %.2e (largest probability %.3f), wdl max-abs %.2e"
+          % (B, err, want.max().item(), (wdl - ref["rwdl"][:B]).abs().max().item()))
+    assert err < 5e-3
+    assert (wdl - ref["rwdl"][:B]).abs().max() <= 1e-2
+    # temperature 0: one-hot at the arg-max of the masked logits the model itself produced
+    pol, _ = m.evaluate(planes.to(cuda))
+    onehot, _ = m.evaluate(planes.to(cuda), legal_mask=mask.to(cuda), T=0.0, want_probs=True)
+    assert torch.equal(onehot.argmax(-1).cpu(), (pol.cpu() + (1.0 - mask.float()) * -999.0).argmax(-1))
+    assert torch.equal(onehot.sum(-1).cpu(), torch.ones(B))
+
+
+def test_bt4class_fp8_headline_config(cuda):
+    """The headline configuration at full size: 15 x 1024 x 32 heads, FFN 1536, e4m3 trunk linears with static scales
+    from a 512-position calibration batch (seed 2), benchmark initialisation (seed 0), positions seed 1. The HIP path
+    against the quantise->dequantise oracle with the SAME amax table, against the fp32 oracle, and against itself with
+    the folded LayerNorm path switched off; then the benchmark's batch of 4096 once: the first 256 rows bit-equal to
+    the 256-position call, everything finite, legal-masked probabilities positive exactly on the mask."""
+    L, Cm, Fm, H = 15, 1024, 1536, 32
+    ref = full_size_reference()
+    oracle, planes, mask = ref["oracle"], ref["planes"], ref["mask"]
+    calib, _ = positions(512, seed=2, leela=True)
+    plan = om.Fp8Plan(L)
+    plan.recording = True
+    oracle.forward_pv(calib, plan)
+    plan.recording = False
+    rpol, rwdl = oracle.forward_pv(planes, plan)
+    sd = oracle.state_dict()
+    m = models.BT4Class(L, Cm, Fm, H, fp8=True)
+    m.load_state_dict(sd)
+    m.calibrate(calib.to(cuda))
+    own = m._engine.get_amax()
+    print("amax rel diff (own bf16 calibration vs oracle fp32): %.3e" % np.abs(own / plan.amax.numpy() - 1).max())
+    assert np.abs(own / plan.amax.numpy() - 1).max() < 0.05
+    m._engine.set_amax(plan.amax.numpy())
+    x = planes.to(cuda)
+    pol, wdl = m(x)
+    pol_d, wdl_d = pol.clone(), wdl.clone()
+    pol, wdl = pol.cpu(), wdl.cpu()
+    report("headline fp8 vs fp8-emulation", pol, rpol, mask, wdl, rwdl)
+    report("headline fp8 vs fp32", pol, ref["rpol"], mask, wdl, ref["rwdl"])
+    report("fp8-emulation vs fp32 (oracle only)", rpol, ref["rpol"], mask, rwdl, ref["rwdl"])
+    # Two e4m3 pipelines that differ in how the tensors BETWEEN the quantisation points are stored (bf16 here, fp32 in
+    # the emulation) round a few percent of the elements to the neighbouring e4m3 code (2^-9 against a code spacing of
+    # 2^-4 relative), and every such flip is a 6 % change of an operand that the next fifty-odd quantisation points
+    # amplify: the distance between the two saturates towards the e4m3 noise itself. Measured 4.0e-2 (3.3e-2 with f16
+    # storage) against 6.0e-2 between either and the fp32 model; the two-layer check below, where nothing has
+    # compounded yet, is the tight one.
+    assert rel_rms(pol, rpol) < 5e-2 and rel_rms(pol, rpol) < rel_rms(rpol, ref["rpol"])
+    assert (wdl - rwdl).abs().max() <= 1.5e-2
+    assert rel_rms(pol, ref["rpol"]) < 1.25 * rel_rms(rpol, ref["rpol"])
+    # f16 storage between the quantisation points (11 significant bits): the same kernels, unfolded norms
+    mh = models.BT4Class(L, Cm, Fm, H, fp8=True, act_dtype="f16")
+    mh.load_state_dict(sd)
+    mh._engine.set_amax(plan.amax.numpy())
+    polh, wdlh = mh(x)
+    polh, wdlh = polh.cpu(), wdlh.cpu()
+    report("headline fp8 with f16 storage vs fp8-emulation", polh, rpol, mask, wdlh, rwdl)
+    assert rel_rms(polh, rpol) < 4e-2 and (wdlh - rwdl).abs().max() <= 1e-2
+    del mh
+    # The same width with two layers (the second one's out-projection takes the first one's folded norm as its
+    # residual): 256 positions put every trunk product on the 256x256 tile the benchmark batch uses.
+    o2 = om.BT4ClassOracle(policy_leela, 2, Cm, Fm, H)
+    o2.load_state_dict({k: v for k, v in sd.items() if not k.startswith("layers.") or int(k.split(".")[1]) < 2})
+    plan2 = om.Fp8Plan(2)
+    plan2.recording = True
+    o2.forward_pv(calib[:128], plan2)
+    plan2.recording = False
+    r2pol, r2wdl = o2.forward_pv(planes, plan2)
+    f2pol, f2wdl = o2.forward_pv(planes)
+    for fold in (True, False):
+        ms = models.BT4Class(2, Cm, Fm, H, fp8=True, ln_fold=fold)
+        ms.load_state_dict(o2.state_dict())
+        ms._engine.set_amax(plan2.amax.numpy())
+        p2, w2 = ms(x)
+        p2, w2 = p2.cpu(), w2.cpu()
+        report("two layers at full width, fp8 %s vs fp8-emulation" % ("folded" if fold else "unfolded"), p2, r2pol, mask, w2, r2wdl)
+        print("   emulation vs fp32 at two layers: policy rel-rms %.2e" % rel_rms(r2pol, f2pol))
+        assert rel_rms(p2, r2pol) < 1.5e-2 and (w2 - r2wdl).abs().max() <= 5e-3
+        del ms
+    # the same weights and scales without the folded norms (every LayerNorm writes its 16-bit output)
+    m2 = models.BT4Class(L, Cm, Fm, H, fp8=True, ln_fold=False)
+    m2.load_state_dict(sd)
+    m2._engine.set_amax(plan.amax.numpy())
+    pol2, wdl2 = m2(x)
+    pol2, wdl2 = pol2.cpu(), wdl2.cpu()
+    report("headline fp8, unfolded norms, vs fp8-emulation", pol2, rpol, mask, wdl2, rwdl)
+    print("   folded vs unfolded: policy rel-rms %.2e, wdl max-abs %.2e" % (rel_rms(pol, pol2), (wdl - wdl2).abs().max().item()))
+    assert rel_rms(pol2, rpol) < 5e-2 and rel_rms(pol, pol2) < 5e-2
+    del m2
+    # batch 4096 (one micro-batch): rows of the 256-position call are reproduced bit for bit
+    big = board.random_positions(1, 4096, masks_leela=True)
+    xb = torch.from_numpy(big["planes"]).to(cuda)
+    mb = torch.from_numpy(big["masks_leela"]).to(cuda)
+    assert torch.equal(xb[:256].cpu().reshape(256, -1), planes.reshape(256, -1))
+    pol4, wdl4 = m(xb)
+    assert torch.equal(pol4[:256], pol_d) and torch.equal(wdl4[:256], wdl_d)
+    assert bool(torch.isfinite(pol4).all()) and bool(torch.isfinite(wdl4).all())
+    probs, _ = models.masked_softmax(pol4, mb, 1.0)
+    assert torch.equal(probs > 0, mb.bool())
+    assert torch.allclose(probs.sum(-1), torch.ones(4096, device=cuda), atol=1e-4)
+
+
+@pytest.mark.parametrize("fp8", [False, True])
+def test_micro_batch_walk_with_late_game_positions(cuda, fp8):
+    """A batch larger than micro_batch is walked in pieces (the large-batch sweep of rollout scoring: 8192 / 16384
+    positions through micro-batches of 4096). Here 200 positions, 30 % of them late-game (at most 10 pieces, sparse
+    legal masks), through micro-batches of 64: bit-equal to the single pass, and the legal-masked softmax is positive
+    exactly on each position's mask."""
+    r = board.random_positions(4, 200, late_fraction=0.3, masks_leela=True)
+    x = torch.from_numpy(r["planes"]).to(cuda)
+    mask = torch.from_numpy(r["masks_leela"]).to(cuda)
+    whole = models.BT4Class(3, 512, 768, 16, fp8=fp8)
+    walked = models.BT4Class(3, 512, 768, 16, fp8=fp8, micro_batch=64)
+    walked.load_state_dict(whole.state_dict())
+    if fp8:
+        whole.calibrate(x[:96])
+        walked._engine.set_amax(whole._engine.get_amax())
+    p1, w1 = whole(x)
+    p2, w2 = walked(x)          # 64 + 64 + 64 + 8
+    assert torch.equal(p1, p2) and torch.equal(w1, w2)
+    probs, _ = walked.evaluate(x, legal_mask=mask, T=1.0, want_probs=True)
+    assert torch.equal(probs > 0, mask.bool())
+    assert int(mask.sum(-1).min()) <= 12          # the late-game share really has sparse masks
+    # the FEN front-end walks the same micro-batches inside each of its chunks
+    fens = board.random_positions(4, 200, late_fraction=0.3, planes=False, fens=True)["fens"]
+    fp, fw, _ = walked.evaluate_fens(fens, T=1.0, chunk=150)
+    assert torch.equal(fp, probs.cpu()) and torch.equal(fw, w1.cpu())
+
+
+def test_bt4class_narrow_model_wide_ffn_fp8(cuda):
+    """d_model 256 with d_ff 4096 in e4m3: FFN-2 is a narrow output over a long K, the shape the fixed K-slice plan
+    takes for small batches. Its residual is normalised in the epilogue (folded norms), which the K-sliced second pass
+    cannot do, so this shape must stay on the tiled kernels: batch invariance and agreement with the emulation."""
+    L, Cm, Fm, H = 2, 256, 4096, 8
+    oracle = om.test_init_(om.BT4ClassOracle(policy_leela, L, Cm, Fm, H), seed=8)
+    calib, _ = positions(64, seed=2, leela=True)
+    planes, mask = positions(300, seed=3, leela=True)
+    plan = om.Fp8Plan(L)
+    plan.recording = True
+    oracle.forward_pv(calib, plan)
+    plan.recording = False
+    rpol, rwdl = oracle.forward_pv(planes, plan)
+    m = models.BT4Class(L, Cm, Fm, H, fp8=True)
+    m.load_state_dict(oracle.state_dict())
+    m._engine.set_amax(plan.amax.numpy())
+    x = planes.to(cuda)
+    pol, wdl = m(x)
+    report("bt4class 2x256 ffn 4096 fp8 vs fp8-emulation", pol.cpu(), rpol, mask, wdl.cpu(), rwdl)
+    assert rel_rms(pol.cpu(), rpol) < 5e-2 and (wdl.cpu() - rwdl).abs().max() <= 2e-2
+    for sl in (slice(3, 4), slice(0, 8), slice(10, 74), slice(0, 130)):
+        p2, w2 = m(x[sl].contiguous())
+        assert torch.equal(p2, pol[sl]) and torch.equal(w2, wdl[sl])
 
 
 def test_bt4class_fp8_vs_emulation(cuda):
@@ -254,6 +506,33 @@ def test_evaluate_fens_pipeline_equals_direct(cuda, arch):
         m = models.GPT(models.GPTConfig(block_size=256, vocab_size=1929, n_layer=2, n_head=8, n_embd=256))
     pol, wdl = m._engine.forward(planes)
     ref_probs, ref_best = models.masked_softmax(pol, mask, 1.0, want_probs=True)
+    # the direct path itself against the fp32 oracle with masks from the pure-Python rules (first 48 positions)
+    from chessrl_amd.vocab import policy_index
+    from oracle import chess_py
+    nb = 48
+    sd = m.state_dict()
+    if arch == "bt4class":
+        oracle = om.BT4ClassOracle(policy_leela, 2, 256, 384, 8)
+        oracle.load_state_dict(sd)
+        opol, owdl = oracle.forward_pv(r_planes_cpu(r)[:nb])
+        omask = torch.tensor([chess_py.legal_mask_leela(f, policy_leela) for f in fens[:nb]])
+    elif arch == "bt4":
+        oracle = om.BT4Oracle(2, 256, 368, 4)
+        oracle.load_state_dict(sd)
+        opol, owdl = oracle.forward_pv(r_planes_cpu(r)[:nb])
+        omask = torch.tensor([chess_py.legal_mask(f, policy_index) for f in fens[:nb]])
+    else:
+        oracle = om.GPTOracle(2, 8, 256)
+        oracle.load_state_dict(sd)
+        opol, owdl = oracle.forward_last(r_planes_cpu(r)[:nb]), None
+        omask = torch.tensor([chess_py.legal_mask(f, policy_index) for f in fens[:nb]])
+    assert torch.equal(omask.to(torch.uint8), mask[:nb].cpu())
+    want = om.masked_policy(opol, omask, 1.0)
+    perr = (ref_probs[:nb].cpu() - want).abs().max().item()
+    print("%s front-end vs oracle: masked probabilities max-abs %.2e" % (arch, perr))
+    assert perr < 5e-3 and torch.equal(ref_probs[:nb].cpu() > 0, omask.bool())
+    if owdl is not None:
+        assert (wdl[:nb].cpu() - owdl).abs().max() <= 1e-2
     for chunk in (64, 128, 1000):     # ragged last chunk, several chunks in flight, one chunk
         probs, w, best = m.evaluate_fens(fens, T=1.0, chunk=chunk)
         assert torch.equal(probs, ref_probs.cpu())
@@ -475,11 +754,13 @@ def test_empty_batch(cuda):
     assert m.evaluate_fens([], T=1.0)[0].shape == (0, 1858)
 
 
-def test_gpt_fp8_vs_emulation(cuda):
-    """The reference's own fp8 model is the GPT of model_fp8.py (te.Linear at :43,45,90,92, high-precision LayerNorm,
-    attention and residual stream): the HIP fp8 path against the quantise->dequantise oracle with the same static scales."""
+@pytest.mark.parametrize("vocab", [1929, 1936])
+def test_gpt_fp8_vs_emulation(cuda, vocab):
+    """The reference's own fp8 model is the GPT of model_fp8.py (te.Linear at :43,45,90,92 and lm_head at :140,
+    high-precision LayerNorm, attention and residual stream; pretrain_fp8.py:16 pads the vocabulary to 1936 rows): the HIP
+    fp8 path against the quantise->dequantise oracle with the same static scales, lm_head included."""
     L, H, Cm = 3, 8, 256
-    oracle = om.test_init_(om.GPTOracle(L, H, Cm), seed=11)
+    oracle = om.test_init_(om.GPTOracle(L, H, Cm, vocab_size=vocab), seed=11)
     calib, _ = positions(64, seed=5)
     planes, mask = positions(64, seed=6)
     plan = om.Fp8Plan(L)
@@ -488,19 +769,96 @@ def test_gpt_fp8_vs_emulation(cuda):
     plan.recording = False
     ref8 = oracle.forward_last(planes, plan)
     ref32 = oracle.forward_last(planes)
-    m = models.GPT(models.GPTConfig(block_size=256, vocab_size=1929, n_layer=L, n_head=H, n_embd=Cm), fp8=True)
+    m = models.GPT(models.GPTConfig(block_size=256, vocab_size=vocab, n_layer=L, n_head=H, n_embd=Cm), fp8=True)
     m.load_state_dict(oracle.state_dict())
     m.calibrate(calib.to(cuda))
-    own = m._engine.get_amax()[:, :4]
-    want = plan.amax.numpy()[:, :4]
-    print("gpt amax rel diff (own calibration vs oracle fp32):", np.abs(own / want - 1).max())
-    assert np.abs(own / want - 1).max() < 0.05
-    full = m._engine.get_amax()
-    full[:, :4] = want
-    m._engine.set_amax(full)
-    pol = m.forward((planes.to(cuda), None))[0][:, 0].cpu()
-    report("gpt fp8 vs fp8-emulation", pol, ref8, mask)
+    own = m._engine.get_amax(head=True)
+    want = plan.table(head=True)
+    used = np.ones_like(want, bool)
+    used[:L, 4] = False          # slot 4 belongs to the BT4-class bias generator
+    used[L, 1:] = False          # the last row only carries lm_head's input
+    print("gpt amax rel diff (own calibration vs oracle fp32):", np.abs(own[used] / want[used] - 1).max())
+    assert np.abs(own[used] / want[used] - 1).max() < 0.05 and want[L, 0] > 0
+    m._engine.set_amax(want)
+    logits = m.forward((planes.to(cuda), None))[0]
+    assert logits.shape == (64, 1, 1929)
+    pol = logits[:, 0].cpu()
+    report("gpt fp8 vs fp8-emulation (vocab %d)" % vocab, pol, ref8, mask)
     report("gpt fp8 vs fp32", pol, ref32, mask)
     report("fp8-emulation vs fp32 (oracle only)", ref8, ref32, mask)
     assert rel_rms(pol, ref8) < 5e-2
     assert rel_rms(pol, ref32) < 2 * rel_rms(ref8, ref32) + 1e-2
+    # lm_head kept in 16 bits on request: closer to fp32 in the head, same trunk
+    m16 = models.GPT(models.GPTConfig(block_size=256, vocab_size=vocab, n_layer=L, n_head=H, n_embd=Cm), fp8=True, fp8_lm_head=False)
+    m16.load_state_dict(oracle.state_dict())
+    m16._engine.set_amax(want)
+    pol16 = m16.forward((planes.to(cuda), None))[0][:, 0].cpu()
+    assert not torch.equal(pol16, pol) and rel_rms(pol16, ref32) < 2 * rel_rms(ref8, ref32) + 1e-2
+
+
+def test_bt4_forward_with_losses(cuda):
+    """BT4.forward(inp, compute_loss=True) of new_paradigm/value.py:197-202: the 6-tuple with both cross-entropies
+    (policy ignore_index 1928, value ignore_index 3), against the oracle's logits through F.cross_entropy."""
+    import torch.nn.functional as F
+    oracle = om.test_init_(om.BT4Oracle(2, 256, 368, 4), seed=13)
+    m = models.BT4(2, 256, 368, 4)
+    m.load_state_dict(oracle.state_dict())
+    b, s = 3, 8
+    planes, _ = positions(b * s, seed=14)
+    g = torch.Generator().manual_seed(2)
+    targets = torch.randint(0, 1858, (b, s), generator=g)
+    targets[0, 1] = 1928
+    values = torch.randint(0, 3, (b, s, 1), generator=g)
+    values[1, 2, 0] = 3
+    x = planes.view(b, s, 8, 8, 19).to(cuda)
+    policy, value_h, lp, lv, t_out, v_out = m.forward([x, targets.to(cuda), None, values.to(cuda)], compute_loss=True)
+    assert policy.shape == (b, s, 1929) and value_h.shape == (b, s, 3)
+    assert torch.equal(t_out.cpu(), targets) and torch.equal(v_out.cpu(), values)
+    rpol, rwdl = oracle.forward_pv(planes)
+    want_lp = F.cross_entropy(rpol, targets.view(-1), ignore_index=1928)
+    want_lv = F.cross_entropy(rwdl, values.view(-1), ignore_index=3)
+    print("bt4 losses: policy %.5f vs %.5f, value %.5f vs %.5f" % (lp.item(), want_lp.item(), lv.item(), want_lv.item()))
+    assert abs(lp.item() - want_lp.item()) < 5e-3 and abs(lv.item() - want_lv.item()) < 5e-3
+    # and exactly F.cross_entropy of the logits the call itself returned
+    assert abs(lp.item() - F.cross_entropy(policy.view(-1, 1929).cpu(), targets.view(-1), ignore_index=1928).item()) < 1e-5
+    assert abs(lv.item() - F.cross_entropy(value_h.view(-1, 3).cpu(), values.view(-1), ignore_index=3).item()) < 1e-5
+    assert torch.equal(m.forward([x]), policy)
+    with pytest.raises(ValueError):
+        m.forward([x, targets.to(cuda), None, torch.zeros(b, 3, device=cuda)], compute_loss=True)
+
+
+@pytest.mark.parametrize("arch", ["gpt", "bt4", "bt4class", "bt4class_fp8"])
+def test_rmsnorm_models(cuda, arch):
+    """norm_rms: the trunk's norms are RMSNorm (no mean subtraction, no offset). Against the oracle with the same switch,
+    for the pre-LN GPT, both post-LN trunks and the e4m3 path whose residual products normalise in their epilogue."""
+    planes, mask = positions(48, seed=15, leela=arch.startswith("bt4class"))
+    x = planes.to(cuda)
+    if arch == "gpt":
+        oracle = om.test_init_(om.GPTOracle(3, 8, 256, rms=True), seed=16)
+        m = models.GPT(models.GPTConfig(block_size=256, vocab_size=1929, n_layer=3, n_head=8, n_embd=256), norm_rms=True)
+        m.load_state_dict(oracle.state_dict())
+        pol, ref = m.forward((x, None))[0][:, 0].cpu(), oracle.forward_last(planes)
+        report("gpt rmsnorm", pol, ref, mask)
+        assert rel_rms(pol, ref) < 1e-2
+        assert rel_rms(pol, om.test_init_(om.GPTOracle(3, 8, 256), seed=16).forward_last(planes)) > 5e-2   # not LayerNorm
+        return
+    if arch == "bt4":
+        oracle = om.test_init_(om.BT4Oracle(2, 256, 368, 4, rms=True), seed=17)
+        m = models.BT4(2, 256, 368, 4, norm_rms=True)
+        tol = 2e-2
+    else:
+        oracle = om.test_init_(om.BT4ClassOracle(policy_leela, 3, 512, 768, 16, rms=True), seed=18)
+        m = models.BT4Class(3, 512, 768, 16, norm_rms=True, fp8=arch.endswith("fp8"))
+        tol = 5e-2 if arch.endswith("fp8") else 2e-2
+    m.load_state_dict(oracle.state_dict())
+    plan = None
+    if arch.endswith("fp8"):
+        plan = om.Fp8Plan(3)
+        plan.recording = True
+        oracle.forward_pv(planes, plan)
+        plan.recording = False
+        m._engine.set_amax(plan.amax.numpy())
+    rpol, rwdl = oracle.forward_pv(planes, plan) if plan else oracle.forward_pv(planes)
+    pol, wdl = m._engine.forward(x)
+    report("%s rmsnorm" % arch, pol.cpu(), rpol, mask, wdl.cpu(), rwdl)
+    assert rel_rms(pol.cpu(), rpol) < tol and (wdl.cpu() - rwdl).abs().max() <= (2e-2 if plan else 1e-2)

@@ -172,3 +172,241 @@ def test_generation_rules():
     assert seq[0].tolist() == [TH, EV, 10, EV, EV, EV, EV, ET, 21, END, 23, EV, 24]
     # a sampled </thinking> (no counter involved) also forces end two places later
     assert seq[1].tolist() == [TH, 1, 2, ET, 3, END, 5, 6, 7, 8, 9, 10, 11]
+
+
+# ------------------------------------------------------------------ BT4-class oracle: pins from what the definition fixes
+def _tok(file, rank):
+    """Token of a real-board square (file 0..7 = a..h, rank 0..7 = 1..8): t = (7 - rank) * 8 + file."""
+    return (7 - rank) * 8 + file
+
+
+def _capture(mods):
+    """Forward hooks that keep the last (input, output) of the named sub-modules."""
+    seen, hooks = {}, []
+    for name, mod in mods.items():
+        hooks.append(mod.register_forward_hook(lambda m, i, o, name=name: seen.__setitem__(name, (i[0].detach(), o.detach()))))
+    return seen, hooks
+
+
+def test_bt4class_policy_gather_brute_force():
+    """Every one of the 1858 outputs, for a white and a black row, from an independent reading of the move string:
+    parse the UCI squares in the side-to-move frame, mirror the ranks for black (rank r -> 9 - r,
+    Leela/compare_policy.py:437-463), read QK^T/sqrt(C) at [from, to], and for the q/r/b promotions add that piece's
+    offset plus the knight offset, both taken from the key of the destination square."""
+    torch.manual_seed(5)
+    C = 128
+    m = om.test_init_(om.BT4ClassOracle(policy_leela, 1, C, 192, 4, compress=8, hidden=32, gen=32), 7, wstd=0.2)
+    x = torch.rand(2, 8, 8, 19)
+    x[0, :, :, 12] = 1.0      # row 0: white to move
+    x[1, :, :, 12] = 0.0      # row 1: black to move
+    seen, hooks = _capture({"q": m.queries_pol, "k": m.keys_pol})
+    pol, _ = m.forward_pv(x)
+    for h in hooks:
+        h.remove()
+    qp, kp = seen["q"][1], seen["k"][1]           # [2, 64, C]
+    wpromo = m.promotion_offsets.weight.detach()  # [4, C]: q, r, b, n
+    want = torch.zeros(2, 1858)
+    for b, white in ((0, True), (1, False)):
+        for v, s in enumerate(policy_leela):
+            ff, fr, tf, tr = ord(s[0]) - 97, int(s[1]) - 1, ord(s[2]) - 97, int(s[3]) - 1
+            if not white:
+                fr, tr = 7 - fr, 7 - tr           # rank digit r -> 9 - r
+            frm, to = _tok(ff, fr), _tok(tf, tr)
+            logit = float(qp[b, frm] @ kp[b, to]) / math.sqrt(C)
+            if len(s) == 5:
+                piece = "qrb".index(s[4])
+                logit += float(wpromo[piece] @ kp[b, to]) + float(wpromo[3] @ kp[b, to])
+            want[b, v] = logit
+    assert torch.allclose(pol, want, atol=2e-4), (pol - want).abs().max()
+    # the promotion moves are exactly the 66 five-character strings, all from rank 7 to rank 8 in the mover's frame
+    promos = [s for s in policy_leela if len(s) == 5]
+    assert len(promos) == 66 and all(s[1] == "7" and s[3] == "8" and s[4] in "qrb" for s in promos)
+    # the destination of a black promotion is on the real first rank (tokens 56..63)
+    assert _tok(ord("a") - 97, 7 - 7) == 56
+
+
+def _bt4class_layer_by_hand(m, ly, x, bias):
+    """One BT4-class layer from plain tensor operations: x1 = LN1(x + a*out(attn)), x2 = LN2(x1 + a*ff2(mish(ff1(x1))))
+    with a = (2L)^-1/4 and attention softmax(QK^T/sqrt(hs) + bias)V written head by head."""
+    B, T, C = x.shape
+    H = m.num_heads
+    hs = C // H
+    a = (2.0 * m.num_layers) ** -0.25
+    at = ly.attention
+    q = F.linear(x, at.query_proj.weight, at.query_proj.bias)
+    k = F.linear(x, at.key_proj.weight, at.key_proj.bias)
+    v = F.linear(x, at.value_proj.weight, at.value_proj.bias)
+    ctx = torch.zeros(B, T, C)
+    for h in range(H):
+        sl = slice(h * hs, (h + 1) * hs)
+        score = q[:, :, sl] @ k[:, :, sl].transpose(1, 2) / math.sqrt(hs) + bias[:, h]
+        ctx[:, :, sl] = score.softmax(-1) @ v[:, :, sl]
+    x1 = F.layer_norm(x + a * F.linear(ctx, at.out_proj.weight, at.out_proj.bias), (C,), ly.norm1.weight, ly.norm1.bias, 1e-5)
+    f = F.linear(F.mish(F.linear(x1, ly.ff1.weight, ly.ff1.bias)), ly.ff2.weight, ly.ff2.bias)
+    return F.layer_norm(x1 + a * f, (C,), ly.norm2.weight, ly.norm2.bias, 1e-5), ctx
+
+
+def _smolgen_bias_by_hand(m, ly, x):
+    """bias[b, h, i, j] = sum_g gen[b, h, g] * Wgen[i*64 + j, g], gen = LN(swish(gen_from(LN(swish(hidden(flatten(compress(x))))))))
+    split per head, every step an explicit loop or a plain tensor operation."""
+    B = x.shape[0]
+    H = m.num_heads
+    sm = ly.smolgen
+    comp = x @ sm.compress.weight.t()                                    # [B, 64, compress], no bias
+    flat = torch.stack([torch.cat([comp[b, t] for t in range(64)]) for b in range(B)])     # token-major flatten
+    hid = F.linear(flat, sm.hidden.weight, sm.hidden.bias)
+    hid = hid * torch.sigmoid(hid)
+    hid = F.layer_norm(hid, hid.shape[-1:], sm.hidden_ln.weight, sm.hidden_ln.bias, 1e-5)
+    g = F.linear(hid, sm.gen_from.weight, sm.gen_from.bias)
+    g = g * torch.sigmoid(g)
+    g = F.layer_norm(g, g.shape[-1:], sm.gen_from_ln.weight, sm.gen_from_ln.bias, 1e-5)
+    per = g.shape[-1] // H
+    W = m.smol_weight_gen.weight                                         # [4096, gen]
+    bias = torch.zeros(B, H, 64, 64)
+    for h in range(H):
+        gh = g[:, h * per:(h + 1) * per]                                 # head h owns a contiguous block of `gen` values
+        bias[:, h] = (gh @ W.t()).view(B, 64, 64)                        # row index of W is query*64 + key
+    return bias
+
+
+def test_bt4class_attention_without_generated_bias_is_sdpa():
+    """With smol_weight_gen = 0 the layer's attention is plain scaled-dot-product attention with scale 1/sqrt(head_dim)."""
+    m = om.test_init_(om.BT4ClassOracle(policy_leela, 1, 128, 192, 4, compress=8, hidden=32, gen=32), 9, wstd=0.2)
+    m.smol_weight_gen.weight.data.zero_()
+    x = torch.rand(3, 8, 8, 19)
+    at = m.layers[0].attention
+    seen, hooks = _capture({"q": at.query_proj, "k": at.key_proj, "v": at.value_proj, "out": at.out_proj})
+    m.forward_pv(x)
+    for h in hooks:
+        h.remove()
+    q, k, v = (seen[n][1].view(3, 64, 4, 32).transpose(1, 2) for n in ("q", "k", "v"))
+    want = F.scaled_dot_product_attention(q, k, v).transpose(1, 2).reshape(3, 64, 128)
+    assert torch.allclose(seen["out"][0], want, atol=1e-5)
+
+
+def test_bt4class_layer_by_hand():
+    """Two layers composed by hand from plain tensor operations (generated bias per head by an explicit loop, residual
+    scale (2L)^-1/4, norm after each residual sum, mish between ff1 and ff2) reproduce the oracle's value output, and
+    the first layer's attention context equals what the oracle feeds out_proj. Dropping alpha, using 1/sqrt(C), moving
+    the norm in front of the sum or swapping query and key in the bias index each break it."""
+    L, C, H = 2, 128, 4
+    m = om.test_init_(om.BT4ClassOracle(policy_leela, L, C, 192, H, compress=8, hidden=32, gen=32), 11, wstd=0.2)
+    planes = torch.rand(2, 8, 8, 19)
+    seen, hooks = _capture({"out0": m.layers[0].attention.out_proj})
+    _, wdl = m.forward_pv(planes)
+    for h in hooks:
+        h.remove()
+    x = planes.view(2, 64, 19)
+    x = F.layer_norm(F.gelu(F.linear(x, m.linear1.weight, m.linear1.bias)), (C,), m.layernorm1.weight, m.layernorm1.bias, 1e-5)
+    x = x * torch.exp(m.ma_gating.a) + m.ma_gating.b
+    for li, ly in enumerate(m.layers):
+        bias = _smolgen_bias_by_hand(m, ly, x)
+        x, ctx = _bt4class_layer_by_hand(m, ly, x, bias)
+        if li == 0:
+            assert torch.allclose(ctx, seen["out0"][0], atol=1e-5)
+    vh = m.value_head
+    v1 = F.mish(F.linear(x, vh.dense1.weight, vh.dense1.bias)).reshape(2, 64 * 128)        # token-major, 128 fastest
+    want = F.linear(F.mish(F.linear(v1, vh.dense2.weight, vh.dense2.bias)), vh.dense3.weight, vh.dense3.bias)
+    assert torch.allclose(wdl, want, atol=1e-5), (wdl - want).abs().max()
+    # sensitivity: the hand composition with a transposed bias tile does not match
+    x0 = planes.view(2, 64, 19)
+    x0 = F.layer_norm(F.gelu(F.linear(x0, m.linear1.weight, m.linear1.bias)), (C,), m.layernorm1.weight, m.layernorm1.bias, 1e-5)
+    x0 = x0 * torch.exp(m.ma_gating.a) + m.ma_gating.b
+    b0 = _smolgen_bias_by_hand(m, m.layers[0], x0)
+    _, bad = _bt4class_layer_by_hand(m, m.layers[0], x0, b0.transpose(-1, -2))
+    assert not torch.allclose(bad, seen["out0"][0], atol=1e-3)
+    assert abs((2.0 * L) ** -0.25 - 0.70710678) < 1e-6      # L = 2: alpha = 4^-1/4
+
+
+# ------------------------------------------------------------------ fp8 emulation against an independent e4m3fn table
+def _e4m3fn_table():
+    """Values of the 256 OCP e4m3fn codes from the format's definition: sign, 4 exponent bits (bias 7), 3 mantissa bits,
+    subnormals at exponent 0, no infinities, the single NaN pattern S.1111.111."""
+    vals = []
+    for c in range(256):
+        s, e, mant = c >> 7, (c >> 3) & 15, c & 7
+        if e == 15 and mant == 7:
+            vals.append(float("nan"))
+            continue
+        mag = (mant / 8.0) * 2.0 ** -6 if e == 0 else (1.0 + mant / 8.0) * 2.0 ** (e - 7)
+        vals.append(-mag if s else mag)
+    return vals
+
+
+def _nearest_even(x, pos):
+    """Nearest value of the sorted list `pos` (non-negative finite codes, index = code) to |x|, ties to the even code,
+    saturating at the largest."""
+    a = abs(x)
+    best = min(range(len(pos)), key=lambda i: (abs(pos[i] - a), i & 1))
+    return math.copysign(pos[best], x)
+
+
+def test_fp8_emulation_matches_independent_e4m3fn_table():
+    table = _e4m3fn_table()
+    # torch's decoding of every code agrees with the definition
+    dec = torch.arange(256, dtype=torch.uint8).view(torch.float8_e4m3fn).float()
+    for c in range(256):
+        if math.isnan(table[c]):
+            assert math.isnan(dec[c].item())
+        else:
+            assert dec[c].item() == table[c], c
+    pos = [table[c] for c in range(127)]              # codes 0..126: 0 .. 448, ascending
+    assert pos == sorted(pos) and pos[-1] == 448.0 and pos[1] == 2.0 ** -9 and pos[8] == 2.0 ** -6
+    # sweep: every code, every midpoint between neighbours (ties), points just off the midpoints, subnormal range,
+    # values past the largest code (saturation)
+    xs = []
+    for i in range(126):
+        lo, hi = pos[i], pos[i + 1]
+        mid = 0.5 * (lo + hi)
+        xs += [lo, mid, mid * (1 - 2 ** -20), mid * (1 + 2 ** -20), lo + 0.25 * (hi - lo), lo + 0.75 * (hi - lo)]
+    xs += [448.0, 449.0, 464.0, 480.0, 1e4, 1e9, 2.0 ** -10, 2.0 ** -11, 1.5 * 2.0 ** -10, 0.0]
+    xs = xs + [-v for v in xs]
+    x = torch.tensor(xs, dtype=torch.float32)
+    got = om.fp8_quant_dequant(x, 1.0)
+    want = torch.tensor([_nearest_even(float(v), pos) for v in x.tolist()], dtype=torch.float32)
+    bad = (got != want).nonzero().flatten().tolist()
+    assert not bad, [(xs[i], got[i].item(), want[i].item()) for i in bad[:5]]
+    # with a scale: quantise(x*s)/s
+    s = 448.0 / 3.0
+    y = torch.linspace(-3.5, 3.5, 4001)
+    got = om.fp8_quant_dequant(y, s)
+    want = torch.tensor([_nearest_even(float(v), pos) for v in (y * s).tolist()], dtype=torch.float32) / s
+    assert torch.equal(got, want)
+
+
+def test_fp8_plan_linear_is_quantise_dequantise_matmul():
+    """Fp8Plan.lin = F.linear over independently quantised input and weight (per-tensor scales 448/amax), bias in fp32;
+    the lm_head row lives beside the layer table and its weight scale covers padded rows."""
+    table = _e4m3fn_table()
+    pos = [table[c] for c in range(127)]
+    torch.manual_seed(3)
+    x, w, b = torch.randn(5, 16), torch.randn(7, 16) * 0.1, torch.randn(7)
+    plan = om.Fp8Plan(2)
+    plan.recording = True
+    plan.lin(x, 1, 2, w, b)
+    plan.lin(x * 2, 2, 0, w, None)            # layer == n_layer: the lm_head cell
+    plan.recording = False
+    assert plan.amax[1, 2].item() == x.abs().max().item() and plan.head_amax[0].item() == (2 * x).abs().max().item()
+    assert plan.table(head=True).shape == (3, 5) and plan.table(head=True)[2, 0] == plan.head_amax[0].item()
+    q = lambda t, s: torch.tensor([_nearest_even(v, pos) for v in (t * s).flatten().tolist()]).view_as(t) / s
+    sx, sw = 448.0 / x.abs().max().item(), 448.0 / w.abs().max().item()
+    want = q(x, sx) @ q(w, sw).t() + b
+    assert torch.allclose(plan.lin(x, 1, 2, w, b), want, atol=1e-6)
+    # a padded weight: the scale comes from the whole tensor
+    got = plan.lin(x * 2, 2, 0, w[:5], None, weight_amax=w.abs().max().item())
+    sx2 = 448.0 / (2 * x).abs().max().item()
+    assert torch.allclose(got, q(2 * x, sx2) @ q(w, sw)[:5].t(), atol=1e-6)
+
+
+def test_rms_norm_matches_library():
+    x = torch.randn(6, 64, 256) * 3 + 0.5
+    w = torch.randn(256)
+    assert torch.allclose(om.rms_norm(x, w, 1e-5), F.rms_norm(x, (256,), w, 1e-5), atol=1e-6)
+    # the oracles' rms switch replaces every trunk norm and ignores the norm biases
+    g = om.test_init_(om.GPTOracle(2, 8, 256, rms=True), 2)
+    planes = torch.rand(2, 8, 8, 19)
+    base = g.forward_last(planes)
+    for blk in g.transformer.h:
+        blk.ln_1.bias.data += 1.0
+    assert torch.equal(g.forward_last(planes), base)
+    assert not torch.allclose(base, om.test_init_(om.GPTOracle(2, 8, 256), 2).forward_last(planes))
