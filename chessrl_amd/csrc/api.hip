@@ -223,6 +223,31 @@ int crl_gemm(const void* A, int64_t lda, const void* W, int64_t ldw, void* C, in
   return e == hipSuccess ? CRL_OK : hip_fail("crl_gemm", e);
 }
 
+int crl_gemm_static_scratch(const void* A, int64_t lda, const void* W, int64_t ldw, void* C, int64_t ldc, int M, int N, int K, int in_dtype,
+                            int out_dtype, const float* bias, int act, float descale, float alpha, const void* res, int64_t ldr,
+                            int res_dtype, float out_scale, float* amax, void* stream) {
+  if (!A || !W || !C || M < 0 || N < 0 || K <= 0) return arg_fail("crl_gemm_static_scratch: bad arguments");
+  if (in_dtype != DT_BF16 && in_dtype != DT_F16 && in_dtype != DT_FP8) return arg_fail("crl_gemm_static_scratch: in_dtype must be bf16, f16 or fp8");
+  if (out_dtype < 0 || out_dtype > 3) return arg_fail("crl_gemm_static_scratch: bad out_dtype");
+  GemmArgs g;
+  std::memset(&g, 0, sizeof(g));
+  g.A = A; g.lda = lda; g.W = W; g.ldw = ldw; g.C = C; g.ldc = ldc; g.M = M; g.N = N; g.K = K; g.nsplit = N;
+  g.bias = bias; g.act = act; g.descale = descale; g.alpha = alpha; g.res = res; g.ldr = ldr; g.res_dtype = res_dtype;
+  g.out_scale = out_scale; g.amax = amax;
+  bool too_big = false;
+  size_t need = 0;
+  hipError_t e = launch_gemm_static_ws(g, in_dtype, out_dtype, (hipStream_t)stream, &too_big, &need);
+  if (too_big) {
+    set_error("crl_gemm_static_scratch: the K slices of this product need " + std::to_string(need) + " bytes of partial sums, the fixed scratch array holds " +
+              std::to_string((size_t)STATIC_WS_BYTES) + " (use crl_gemm, which allocates)");
+    return CRL_ERR_ARG;
+  }
+  if (e == hipErrorInvalidValue)
+    return arg_fail("crl_gemm_static_scratch: operands must be 16-byte aligned with K*elem_size a multiple of 16");
+  return e == hipSuccess ? CRL_OK : hip_fail("crl_gemm_static_scratch", e);
+}
+int64_t crl_gemm_static_scratch_bytes(void) { return (int64_t)STATIC_WS_BYTES; }
+
 int crl_layernorm(const void* x, int64_t ldx, int in_dtype, const float* gamma, const float* beta, void* out, int out_dtype,
                   uint8_t* out_fp8, float fp8_scale, int64_t ldo, int rows, int C, float eps, float* amax, void* stream) {
   if (!x || !gamma || (!out && !out_fp8) || rows < 0) return arg_fail("crl_layernorm: bad arguments");

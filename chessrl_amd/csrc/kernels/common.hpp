@@ -274,6 +274,9 @@ hipError_t launch_gemm(GemmArgs a, int in_dt, int out_dt, int tile, hipStream_t 
 // True when launch_gemm (tile 0) would take the K-sliced path for these arguments, whose second pass can apply the
 // LayerNorm that follows the GEMM (GemmArgs::ln_*); launch_gemm rejects ln_out otherwise.
 bool gemm_folds_layernorm(const GemmArgs& a, int in_dt);
+// crl_gemm's tile 4 with the slices' partial sums in a fixed array of the library's device image (no allocation).
+constexpr size_t STATIC_WS_BYTES = 8u << 20;
+hipError_t launch_gemm_static_ws(GemmArgs a, int in_dt, int out_dt, hipStream_t st, bool* too_big, size_t* need_bytes);
 // Frees the device memory the GEMM launchers keep outside any model (per-stream K-slice workspaces, the zeros block).
 void release_gemm_globals();
 hipError_t launch_layernorm(const LayerNormArgs& a, hipStream_t st);

@@ -633,4 +633,44 @@ hipError_t launch_gemm(GemmArgs a, int in_dt, int out_dt, int tile, hipStream_t 
   return hipErrorInvalidValue;
 }
 
+// ---- K-sliced GEMM on a fixed scratch array -------------------------------------------------------
+// For callers that cannot allocate device memory: the partial sums of the K slices live in an array that is part of
+// the library's device image, one copy per GPU that loads it, held until the process ends. The array's name is a
+// host-side stand-in; the address the kernels take comes from hipGetSymbolAddress, once per device.
+static __device__ __align__(256) float scratch[STATIC_WS_BYTES / sizeof(float)];
+static float* g_scratch_ptr[16] = {};
+
+// rc: hipErrorInvalidValue with *too_big set when the slices need more than the array holds.
+hipError_t launch_gemm_static_ws(GemmArgs a, int in_dt, int out_dt, hipStream_t st, bool* too_big, size_t* need_bytes) {
+  *too_big = false;
+  *need_bytes = 0;
+  if (a.M <= 0 || a.N <= 0) return hipSuccess;
+  int dev = 0;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess) return e;
+  if (dev < 0 || dev >= 16) return hipErrorInvalidDevice;
+  float* ptr = nullptr;
+  {
+    std::lock_guard<std::mutex> lock(g_ws_mutex);
+    if (!g_scratch_ptr[dev]) {
+      void* sym = nullptr;
+      e = hipGetSymbolAddress(&sym, HIP_SYMBOL(scratch));   // the current device's copy of the array
+      if (e != hipSuccess) return e;
+      g_scratch_ptr[dev] = static_cast<float*>(sym);
+    }
+    ptr = g_scratch_ptr[dev];
+  }
+  // The plan crl_gemm's tile 4 would make (its own workspace is larger than this one): same slices or refuse.
+  GemmArgs plan = a;
+  plan.splitk_ws = nullptr;
+  int per = 0;
+  const int ks = splitk_plan(plan, in_dt == DT_FP8 ? 1 : 2, true, &per);
+  const size_t need = ks > 1 ? (size_t)ks * a.M * ((a.N + 7) / 8 * 8) * sizeof(float) : 0;
+  *need_bytes = need;
+  if (need > STATIC_WS_BYTES) { *too_big = true; return hipErrorInvalidValue; }
+  a.splitk_ws = ptr;
+  a.splitk_ws_bytes = (long)STATIC_WS_BYTES;
+  return launch_gemm(a, in_dt, out_dt, 4, st);
+}
+
 }  // namespace crl

@@ -115,6 +115,19 @@ int crl_gemm(const void* A, int64_t lda, const void* W, int64_t ldw, void* C, in
              const float* bias, int act, float descale, float alpha,
              const void* res, int64_t ldr, int res_dtype, float out_scale, float* amax,
              int tile, void* stream);
+/* No counterpart in the reference: crl_gemm with tile = 4 (K cut into slices, a second kernel adds them) for callers that
+ * cannot allocate device memory, i.e. code under HIP graph capture, serving loops and harnesses that forbid hipMalloc.
+ * The partial sums of the slices go to a fixed array of crl_gemm_static_scratch_bytes() = 8 MB inside the library's
+ * device image (one copy per GPU, held until the process ends) instead of the per-stream workspace crl_gemm allocates on
+ * first use; the call allocates and frees nothing. Arguments and result bits are those of crl_gemm(..., tile = 4, ...).
+ * Products whose slices need more (slices * M * round_up(N, 8) * 4 bytes; slices <= 16) fail with CRL_ERR_ARG and a
+ * message naming both sizes. Every call on a GPU uses that GPU's one array: calls that overlap in time on one GPU
+ * (different streams or threads) race. Nothing in the array has to start at zero (each launch overwrites what it reads). */
+int crl_gemm_static_scratch(const void* A, int64_t lda, const void* W, int64_t ldw, void* C, int64_t ldc,
+                            int M, int N, int K, int in_dtype, int out_dtype,
+                            const float* bias, int act, float descale, float alpha,
+                            const void* res, int64_t ldr, int res_dtype, float out_scale, float* amax, void* stream);
+int64_t crl_gemm_static_scratch_bytes(void);
 /* F.layer_norm(x,(C,),gamma,beta,eps) (model_bis.py:34). out (out_dtype) and/or out_fp8
  * (value*fp8_scale, e4m3) may be given. */
 int crl_layernorm(const void* x, int64_t ldx, int in_dtype, const float* gamma, const float* beta,
