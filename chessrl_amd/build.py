@@ -18,6 +18,8 @@ SOURCES = [
     "kernels/gemm.hip",
     "kernels/gemm_dma.hip",
     "kernels/gemm_dma_resnorm.hip",
+    "kernels/gemm_pp.hip",
+    "kernels/gemm_sp.hip",
     "kernels/norm_embed.hip",
     "kernels/attention.hip",
     "kernels/heads.hip",

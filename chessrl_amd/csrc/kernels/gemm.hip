@@ -585,7 +585,15 @@ static hipError_t launch_in_out(const GemmArgs& a, int tile, hipStream_t st) {
       if (ks > 1) return launch_splitk<CfgSmallK4, IN_DT, OUT_DT>(a, ks, per, st);
     }
   }
-  if (tile == 3) return launch_gemm_dma(a, IN_DT, OUT_DT, st);
+  if (tile == 6) {
+    if constexpr (IN_DT == DT_FP8 && (OUT_DT == DT_BF16 || OUT_DT == DT_FP8)) return launch_gemm_pp(a, OUT_DT, st);
+    else return hipErrorInvalidValue;
+  }
+  if (tile == 8) {
+    if constexpr (IN_DT == DT_FP8 && (OUT_DT == DT_BF16 || OUT_DT == DT_FP8)) return launch_gemm_sp(a, OUT_DT, st);
+    else return hipErrorInvalidValue;
+  }
+  if (tile == 3 || tile == 7) return launch_gemm_dma(a, IN_DT, OUT_DT, st);
   if (tile == 2) return launch_cfg<CfgMid, IN_DT, OUT_DT>(a, st);
   if (tile == 5) return launch_cfg<CfgSmallK4, IN_DT, OUT_DT>(a, st);
   return launch_cfg<CfgSmall, IN_DT, OUT_DT>(a, st);

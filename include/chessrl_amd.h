@@ -109,7 +109,9 @@ int crl_random_positions(uint64_t seed, int n, int max_plies, double late_fracti
  * LDS. Both are deterministic from launch to launch but differ from 1-3 in summation order. With tile 0, outputs of at
  * most 256 columns whose K is 4 KB or more per row are always K-sliced the same way (a function of N and K alone), so
  * the row-count independence holds for them too. The first K-sliced launch on a stream allocates that stream's
- * workspace: issue it once outside any graph capture. */
+ * workspace: issue it once outside any graph capture. 6-8 name the three 256x256 kernels for e4m3 operands with bf16 or
+ * e4m3 output explicitly (same sums, bit-equal results): 7 = eight waves in step (what 3 runs), 6 = the two waves of a
+ * SIMD out of step, 8 = four software-pipelined waves; 6 and 8 exist for measurement and are slower. */
 int crl_gemm(const void* A, int64_t lda, const void* W, int64_t ldw, void* C, int64_t ldc,
              int M, int N, int K, int in_dtype, int out_dtype,
              const float* bias, int act, float descale, float alpha,

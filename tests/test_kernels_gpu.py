@@ -190,6 +190,34 @@ def test_gemm_fp8(cuda, M, N, K, tile):
     assert mism < 0.01, mism  # rounding ties at fp32 summation-order noise only
 
 
+@pytest.mark.parametrize("M,N,K", [(256, 256, 64), (256, 256, 128), (256, 256, 192), (512, 1024, 1024), (4096, 1536, 1024), (2048, 3104, 1024), (1000, 3104, 1072),
+                                   (20000, 1024, 1536), (2048, 200, 512), (2048, 1700, 1040), (300, 700, 736), (256, 4096, 256), (4096, 1024, 4096)])
+@pytest.mark.parametrize("alt", [6, 8])
+def test_gemm_fp8_out_of_step_kernel_equals_in_step_kernel(cuda, M, N, K, alt):
+    """The two other 256x256 e4m3 kernels, the one whose two waves per SIMD alternate between fragment reads and MFMAs
+    (tile 6) and the four-wave software-pipelined one (tile 8), against the kernel whose eight waves work in step
+    (tile 7): all add up K in the same order, so the outputs are bit-equal; bf16 output with bias, activation and
+    residual, and e4m3 output with a scale. K of 1 to 64 steps, K tails, odd step counts, ragged M and N."""
+    torch.manual_seed(M + N + K)
+    A = (torch.randn(M, K, device=cuda) * 30).to(torch.float8_e4m3fn)
+    W = (torch.randn(N, K, device=cuda) * 30).to(torch.float8_e4m3fn)
+    bias = torch.randn(N, device=cuda)
+    ldc = (N + 7) // 8 * 8
+    res = torch.randn(M, ldc, device=cuda).bfloat16()
+    for kw in (dict(out_dt=_lib.BF16, bias=bias, act=2, descale=1e-3, alpha=0.43, res=res),
+               dict(out_dt=_lib.BF16, descale=1e-3),
+               dict(out_dt=_lib.FP8, bias=bias, act=2, descale=1e-3, out_scale=7.0)):
+        amax6, amax7 = torch.zeros(1, device=cuda), torch.zeros(1, device=cuda)
+        o6 = run_gemm(A, W, kw["out_dt"], tile=alt, ldc=ldc, amax=amax6, **{k: v for k, v in kw.items() if k != "out_dt"})
+        o7 = run_gemm(A, W, kw["out_dt"], tile=7, ldc=ldc, amax=amax7, **{k: v for k, v in kw.items() if k != "out_dt"})
+        assert torch.equal(o6, o7), (M, N, K, kw["out_dt"], (o6.float() - o7.float()).abs().max().item())
+        assert torch.equal(amax6, amax7)
+    # and against torch on the same operands
+    ref = (A.float() @ W.float().t()) * 1e-3
+    out = run_gemm(A, W, _lib.BF16, descale=1e-3, tile=alt, ldc=ldc)
+    assert torch.allclose(out.float(), ref, rtol=2 ** -7, atol=2 ** -7 * ref.abs().max().item()), (out.float() - ref).abs().max()
+
+
 @pytest.mark.parametrize("C_,in_dt", [(256, _lib.F32), (1024, _lib.BF16), (512, _lib.BF16), (8192, _lib.BF16), (768, _lib.F32), (1536, _lib.F32)])
 def test_layernorm(cuda, C_, in_dt):
     torch.manual_seed(C_)
