@@ -12,8 +12,9 @@
 // so the matrix pipe always has the next MFMA waiting while LDS and the memory pipe work under it.
 // Measured on MI355X against the eight-wave kernel: equal at long K (2.11 against 2.08 PFLOP/s at K = 8192), slower at
 // K = 1024 (1.33 against 1.52: four waves take twice as long over the epilogue, and the three K steps fetched past the
-// end cost as much as three real ones). With its loads switched off the same loop runs at 2.85 PFLOP/s, with its MFMAs
-// switched off the loads alone take 72 % of the full time: neither side is the bound by itself, they overlap by a third.
+// end cost as much as three real ones). With its loads switched off the same loop runs at 2.85 PFLOP/s (with or without
+// the barrier), with its MFMAs switched off the loads alone take 72 % of the full time (with or without the fragment
+// reads, with three or four K steps in flight): neither side is the bound by itself, they overlap by a third.
 // The model's products therefore stay on the eight-wave kernel; this one is kept as tile 8 of crl_gemm.
 // The ring holds four stages of 64-byte rows (256 weight rows, then 256 activation rows, 16-byte chunks XOR-swizzled as
 // in gemm_dma_kernel.hpp). One workgroup barrier per K step, at the top of the block:
