@@ -20,6 +20,8 @@ SOURCES = [
     "kernels/gemm_dma_resnorm.hip",
     "kernels/gemm_pp.hip",
     "kernels/gemm_sp.hip",
+    "kernels/gemm_sp2.hip",
+    "kernels/gemm_dmaf.hip",
     "kernels/norm_embed.hip",
     "kernels/attention.hip",
     "kernels/heads.hip",

@@ -558,7 +558,7 @@ static hipError_t launch_splitk(const GemmArgs& a, int ks, int per, hipStream_t 
 template <int IN_DT, int OUT_DT>
 static hipError_t launch_in_out(const GemmArgs& a, int tile, hipStream_t st) {
   if (a.ln_out && !gemm_folds_layernorm(a, IN_DT)) return hipErrorInvalidValue;   // only the K-sliced path has a whole row in one place
-  if (a.res_stats && (a.k_parallel || tile >= 4)) return hipErrorInvalidValue;   // tiles 1-3 only
+  if (a.res_stats && (a.k_parallel || (tile >= 4 && tile != 7 && tile != 9 && tile != 10))) return hipErrorInvalidValue;   // the tiled kernels only
   if ((tile == 0 && a.k_parallel) || tile == 4) {
     int per = 0;
     const int ks = splitk_plan(a, IN_DT == DT_FP8 ? 1 : 2, tile == 4, &per);
@@ -592,6 +592,18 @@ static hipError_t launch_in_out(const GemmArgs& a, int tile, hipStream_t st) {
   if (tile == 8) {
     if constexpr (IN_DT == DT_FP8 && (OUT_DT == DT_BF16 || OUT_DT == DT_FP8)) return launch_gemm_sp(a, OUT_DT, st);
     else return hipErrorInvalidValue;
+  }
+  // The 256x256 tile of e4m3 operands has two kernels: four software-pipelined waves (tile 9) where K is whole 128-byte
+  // slabs, and eight waves in step (tile 7). The first has the faster main loop (1.63 against 1.96 us per slab) and the
+  // slower prologue and epilogue (10.0 against 7.7 us per tile): it takes over from K = 768 on.
+  if (tile == 9 && a.K % 128 != 0) tile = 7;
+  if constexpr (IN_DT == DT_FP8 && OUT_DT != DT_F32) {
+    if (tile == 3 && a.K % 128 == 0) tile = a.K >= 4096 ? 9 : 10;
+    if (tile == 9) return launch_gemm_sp2(a, OUT_DT, st);
+    if (tile == 10 && a.K % 128 != 0) tile = 7;
+    if (tile == 10) return launch_gemm_dmaf(a, OUT_DT, st);
+  } else {
+    if (tile == 9 || tile == 10) return hipErrorInvalidValue;
   }
   if (tile == 3 || tile == 7) return launch_gemm_dma(a, IN_DT, OUT_DT, st);
   if (tile == 2) return launch_cfg<CfgMid, IN_DT, OUT_DT>(a, st);

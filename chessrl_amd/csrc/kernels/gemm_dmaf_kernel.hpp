@@ -1,0 +1,227 @@
+// C[M,N] = epilogue(A[M,K] · W[N,K]^T), e4m3 operands, K a whole number of 128-byte slabs: the eight-wave in-step
+// 256x256 kernel of gemm_dma_kernel.hpp with its address arithmetic taken out of the main loop. There a wave issues,
+// per slab of 16 MFMAs, 24 LDS reads and 8 loads, another 85 vector ALU instructions: a 64-bit add, a compare and two
+// selects per load (slab offset, K tail from a block of zeros), an add per fragment read. Here
+//  * LDS is laid out weight rows of stage 0, of stage 1 (32 KB each), then activation rows of stage 0, of stage 1, so a
+//    stage is bit 15 of an address: a fragment address is one of four lane registers per operand plus an instruction
+//    immediate, and all eight registers change stage with one XOR each per slab;
+//  * loads use buffer addressing: descriptor base = tile origin (scalar), a fixed lane offset, the slab offset in a
+//    scalar register; past the end of K they go through a descriptor of zero length (they move nothing and keep the
+//    instruction stream free of branches).
+// Same tile walk, same K order and same epilogue as gemm_dma_kernel.hpp: the outputs are bit-equal.
+#pragma once
+#include "gemm_dma_kernel.hpp"
+
+namespace crl {
+
+struct DmafCfg {
+  static constexpr int BM = 256, BN = 256, WGM = 2, WGN = 4, NW = 8, NT = 512;
+  static constexpr int WM = 128, WN = 64, TM = 4, TN = 2;
+  static constexpr int ROWB = 128, LOADS = 8;
+  static constexpr int RING_BYTES = 2 * (BM + BN) * ROWB;   // 128 KB
+  static constexpr int EPI_BYTES = NW * 32 * WN * 4;        // 64 KB: the two weight stages
+  static constexpr int STATS_OFF = RING_BYTES + 256;        // behind the landing strip of the L2 touches
+  static constexpr int LDS_BYTES = STATS_OFF + NW * 2 * WM * 4;
+};
+
+template <int OUT_DT, int RES_NORM = 0>
+__global__ void __launch_bounds__(DmafCfg::NT, 2) gemm_dmaf_kernel(const GemmArgs a, const int pf) {
+  typedef DmafCfg Cfg;
+  constexpr int IN_DT = DT_FP8;
+  constexpr int BM = Cfg::BM, BN = Cfg::BN, TM = Cfg::TM, TN = Cfg::TN, LOADS = Cfg::LOADS;
+  extern __shared__ __align__(16) uint8_t smem[];
+
+  // (the wave index as a scalar: everything derived from it, LDS destinations and descriptors, stays in scalar registers)
+  const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int wm = wave % Cfg::WGM, wn = wave / Cfg::WGM;
+  const int lr = lane & 31, g = lane >> 5;
+
+  const int tiles_n = (a.N + BN - 1) / BN;
+  const int nblk = gridDim.x;
+  int pid = blockIdx.x;
+  {
+    const int per = nblk >> 3;
+    if (pid < (per << 3)) pid = (pid & 7) * per + (pid >> 3);
+  }
+  // Tile order inside an XCD's range: groups of 8 x w tiles (M x N), w = 3 or 4, as in gemm_dma_kernel.hpp.
+  int tile_m = pid / tiles_n, tile_n = pid - tile_m * tiles_n;
+  int grp_w = 4, grp_q = tile_n & 3;
+  {
+    constexpr int GM = 8;
+    const int tiles_m = (a.M + BM - 1) / BM;
+    if (tiles_m % GM == 0) {
+      const int ngrp = (tiles_n + 3) >> 2, wb = tiles_n / ngrp, extra = tiles_n - wb * ngrp;
+      const int sr = pid / (GM * tiles_n), rem = pid - sr * (GM * tiles_n);
+      const int big = GM * (wb + 1) * extra;
+      int gi, r2;
+      if (rem < big) { grp_w = wb + 1; gi = rem / (GM * grp_w); r2 = rem - gi * GM * grp_w; }
+      else { grp_w = wb; const int rem2 = rem - big; gi = rem2 / (GM * wb); r2 = rem2 - gi * GM * wb; gi += extra; }
+      grp_q = r2 % grp_w;
+      tile_m = sr * GM + r2 / grp_w;
+      tile_n = gi * wb + (gi < extra ? gi : extra) + grp_q;
+    }
+  }
+  const int m0 = tile_m * BM, n0 = tile_n * BN;
+  const int nslab = a.K / Cfg::ROWB;        // the launcher sends only K % 128 == 0 here
+
+  if constexpr (RES_NORM != 0) {
+    // Statistics of this wave's 128 rows (two rows = 16 bytes per lane), requested before anything else and landed
+    // outside the ring.
+    int m = m0 + wm * Cfg::WM + 2 * lane;
+    m = m + 1 < a.M ? m : 0;
+    __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(a.res_stats + 2 * (long)m),
+                                     (__attribute__((address_space(3))) void*)(smem + Cfg::STATS_OFF + wave * (2 * Cfg::WM * 4)), 16, 0, 0);
+  }
+
+  // Loader role: waves 0-3 fill weight rows [64w, +64) of a stage, waves 4-7 activation rows [64(w-4), +64): 8 rows per
+  // wave-instruction, eight 16-byte chunks per row, the swizzle applied on the global side (row 8 i + lane / 8 of the
+  // wave's 64 has swizzle (lane / 8) ^ i).
+  const bool loads_a = wave >= 4;
+  const int rbase = (wave & 3) * 64;
+  const int ld = loads_a ? a.lda : a.ldw;
+  const int rows_left = loads_a ? a.M - m0 : a.N - n0;
+  uint32_t voff[LOADS];
+#pragma unroll
+  for (int i = 0; i < LOADS; ++i) {
+    int r = rbase + 8 * i + (lane >> 3);
+    r = r < rows_left ? r : rows_left - 1;
+    voff[i] = (uint32_t)r * (uint32_t)ld + (((lane & 7) ^ (lane >> 3) ^ i) << 4);
+  }
+  auto make_rsrc = [&](const void* base, long rows, long ldb) {
+    const long span = (rows < 256 ? rows : 256) * ldb;
+    return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(base), 0, (int)(span < 0x7fffffffL ? span : 0x7fffffffL), 0x00020000);
+  };
+  const __amdgpu_buffer_rsrc_t rsrc_w = make_rsrc(reinterpret_cast<const uint8_t*>(a.W) + (long)n0 * a.ldw, a.N - n0, a.ldw);
+  const __amdgpu_buffer_rsrc_t rsrc_x = make_rsrc(reinterpret_cast<const uint8_t*>(a.A) + (long)m0 * a.lda, a.M - m0, a.lda);
+  const __amdgpu_buffer_rsrc_t rsrc_none = __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(a.A), 0, 0, 0x00020000);
+  const __amdgpu_buffer_rsrc_t rsrc_mine = loads_a ? rsrc_x : rsrc_w;
+  const uint32_t lds_load0 = (loads_a ? 65536u : 0u) + rbase * Cfg::ROWB;   // stage 0
+  auto issue_one = [&](int slab, const __amdgpu_buffer_rsrc_t& r, auto ic) {
+    constexpr int i = decltype(ic)::value;
+    __builtin_amdgcn_raw_ptr_buffer_load_lds(r, (__attribute__((address_space(3))) void*)(smem + (lds_load0 ^ ((slab & 1) << 15)) + i * 1024), 16,
+                                             (int)voff[i], slab * Cfg::ROWB, 0, 0);
+  };
+
+  // L2 touches, as in gemm_dma_kernel.hpp: wave 0 touches its share of the activation lines of a slab `pf` slabs before
+  // anybody loads it, wave 1 its share of the weight lines; one dword per 128-byte line into an LDS strip nobody reads.
+  uint32_t pf_off = 0;
+  int pf_n = 0, pf_step = 0;
+  if (pf > 0 && wave < 2) {
+    if (wave == 0) {
+      pf_n = (4 + grp_w - 1) / grp_w;
+      int r = ((grp_q * pf_n) & 3) * 64 + lane;
+      r = r < a.M - m0 ? r : a.M - m0 - 1;
+      pf_off = (uint32_t)r * (uint32_t)a.lda;
+      pf_step = (m0 + 256 <= a.M) ? 64 * a.lda : 0;
+    } else {
+      pf_n = 1;
+      int r = (tile_m & 7) * 32 + (lane & 31);
+      r = r < a.N - n0 ? r : a.N - n0 - 1;
+      pf_off = (uint32_t)r * (uint32_t)a.ldw + (lane >> 5) * 64;
+    }
+  }
+  const __amdgpu_buffer_rsrc_t rsrc_pf = wave == 0 ? rsrc_x : rsrc_w;
+  auto prefetch = [&](int slab) {
+    if (pf_n > 0 && slab < nslab) {
+      for (int i = 0; i < pf_n; ++i)
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_pf, (__attribute__((address_space(3))) void*)(smem + Cfg::RING_BYTES), 4,
+                                                 (int)pf_off, slab * Cfg::ROWB + i * pf_step, 0, 0);
+    }
+  };
+
+  f32x16_t acc[TN][TM];
+#pragma unroll
+  for (int i = 0; i < TN; ++i)
+#pragma unroll
+    for (int j = 0; j < TM; ++j)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
+
+  // Fragment addresses. The 16-byte piece (K step ks, half) of row 32 t + lr of a wave's block sits at chunk
+  // (4 ks + half + 2g) ^ swizzle(row), and swizzle(row) = swizzle(lr) ^ 4 (t & 1): with L = 2g ^ swizzle(lr) the chunk is
+  // Kc ^ L for the compile-time Kc = (4 ks + half) ^ 4 (t & 1), one of 0, 1, 4, 5. Four lane addresses per operand (one
+  // per Kc) plus the immediate 4096 t cover every read of a stage.
+  const int L0 = (2 * g) ^ lds_swizzle(lr);
+  const uint32_t lds0 = (uint32_t)reinterpret_cast<uintptr_t>((__attribute__((address_space(3))) uint8_t*)smem);
+  uint32_t wb[4], xb[4];
+#pragma unroll
+  for (int k = 0; k < 4; ++k) {
+    const int kc = (k & 1) | ((k >> 1) << 2);
+    wb[k] = lds0 + (wn * Cfg::WN + lr) * Cfg::ROWB + ((kc ^ L0) << 4);
+    xb[k] = lds0 + 65536 + (wm * Cfg::WM + lr) * Cfg::ROWB + ((kc ^ L0) << 4);
+  }
+  auto read_piece = [&](bool is_w, int t, int ks, int half) -> i32x4_t {
+    const int kc = (4 * ks + half) ^ (4 * (t & 1));
+    const int k = (kc & 1) | ((kc >> 2) << 1);
+    return *reinterpret_cast<const __attribute__((address_space(3))) i32x4_t*>((is_w ? wb[k] : xb[k]) + t * 32 * Cfg::ROWB);
+  };
+
+  // A wave whose 128x64 part lies wholly outside C still takes its share of the loads and every barrier.
+  const bool wave_active = (m0 + wm * Cfg::WM < a.M) && (n0 + wn * Cfg::WN < a.N);
+
+  static_for<0, LOADS>([&](auto ic) { issue_one(0, rsrc_mine, ic); });
+  for (int s0 = 1; s0 < 1 + pf; ++s0) prefetch(s0);
+
+  for (int slab = 0; slab < nslab; ++slab) {
+    wait_vmcnt<0>();
+    __syncthreads();
+    const __amdgpu_buffer_rsrc_t rnext = slab + 1 < nslab ? rsrc_mine : rsrc_none;
+    prefetch(slab + 1 + pf);
+    if (!wave_active) {
+      static_for<0, LOADS>([&](auto ic) { issue_one(slab + 1, rnext, ic); });
+      continue;
+    }
+    static_for<0, 2>([&](auto ksc) {
+      constexpr int ks = decltype(ksc)::value;
+      Frag<IN_DT> wf[TN], xf[TM];
+#pragma unroll
+      for (int tn = 0; tn < TN; ++tn) { wf[tn].lo = read_piece(true, tn, ks, 0); wf[tn].hi = read_piece(true, tn, ks, 1); }
+#pragma unroll
+      for (int tm = 0; tm < TM; ++tm) { xf[tm].lo = read_piece(false, tm, ks, 0); xf[tm].hi = read_piece(false, tm, ks, 1); }
+      static_for<0, TN * TM>([&](auto ic) {
+        constexpr int i = decltype(ic)::value;
+        constexpr int tn = i / TM, tm = i % TM;
+        acc[tn][tm] = mfma_frag<IN_DT>(wf[tn], xf[tm], acc[tn][tm]);
+        // The next slab's loads go out one at a time, after every second MFMA, held in place by scheduling barriers.
+        if constexpr ((i & 1) == 1) {
+          __builtin_amdgcn_sched_barrier(0);
+          issue_one(slab + 1, rnext, std::integral_constant<int, ks * 4 + (i >> 1)>{});
+          __builtin_amdgcn_sched_barrier(0);
+        }
+      });
+    });
+    // The address registers follow the ring to the other stage.
+#pragma unroll
+    for (int k = 0; k < 4; ++k) { wb[k] ^= 32768u; xb[k] ^= 32768u; }
+  }
+
+  wait_vmcnt<0>();
+  __syncthreads();  // every wave is done with the ring (and the empty loads past the end have retired) before it becomes epilogue scratch
+
+  gemm_epilogue<Cfg::WM, Cfg::WN, OUT_DT, RES_NORM>(a, acc, reinterpret_cast<float*>(smem) + wave * (32 * Cfg::WN),
+                                                     m0 + wm * Cfg::WM, n0 + wn * Cfg::WN, lane,
+                                                     reinterpret_cast<float*>(smem + Cfg::STATS_OFF) + wave * (2 * Cfg::WM));
+}
+
+template <int OUT_DT, int RES_NORM = 0>
+static hipError_t launch_dmaf(const GemmArgs& a, hipStream_t st) {
+  static std::atomic<bool> attr_set[16] = {};
+  hipError_t e = hipSuccess;
+  // Whole slabs of K only, and lane offsets inside a tile's 256 rows that fit 31 bits.
+  if (a.K % DmafCfg::ROWB != 0 || a.K <= 0 || (long)a.lda * 256 >= (1L << 31) || (long)a.ldw * 256 >= (1L << 31)) return hipErrorInvalidValue;
+  int dev = 0;
+  (void)hipGetDevice(&dev);
+  auto kern = gemm_dmaf_kernel<OUT_DT, RES_NORM>;
+  if (!attr_set[dev]) {
+    e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, DmafCfg::LDS_BYTES);
+    if (e != hipSuccess) return e;
+    attr_set[dev] = true;
+  }
+  const int tiles_n = (a.N + DmafCfg::BN - 1) / DmafCfg::BN;
+  const int tiles = ((a.M + DmafCfg::BM - 1) / DmafCfg::BM) * tiles_n;
+  const int pf = (tiles_n % 4 == 0 && (long)a.K >= 8 * DmafCfg::ROWB) ? 2 : 0;
+  hipLaunchKernelGGL(kern, dim3(tiles), dim3(DmafCfg::NT), DmafCfg::LDS_BYTES, st, a, pf);
+  return hipGetLastError();
+}
+
+}  // namespace crl

@@ -130,6 +130,13 @@ __global__ void __launch_bounds__(SpCfg::NT) gemm_sp_kernel(const GemmArgs a, co
     for (int j = 0; j < TM; ++j)
 #pragma unroll
       for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
+  // The MFMAs below are inline assembly, so the compiler does not know that a matrix instruction must not read an
+  // accumulation register in the cycles right after a v_accvgpr_write to it, and it is free to sink the zeroing down to
+  // the first MFMA (seen: stale values in single registers of two tiles). This statement depends on every accumulator
+  // and every MFMA depends on it: the zeroing is complete, and some cycles old, before the first MFMA issues.
+  asm volatile("s_nop 7\n\ts_nop 7"
+               : "+a"(acc[0][0]), "+a"(acc[0][1]), "+a"(acc[0][2]), "+a"(acc[0][3]), "+a"(acc[1][0]), "+a"(acc[1][1]), "+a"(acc[1][2]), "+a"(acc[1][3]),
+                 "+a"(acc[2][0]), "+a"(acc[2][1]), "+a"(acc[2][2]), "+a"(acc[2][3]), "+a"(acc[3][0]), "+a"(acc[3][1]), "+a"(acc[3][2]), "+a"(acc[3][3]));
 
   // Byte offsets of this lane's two 16-byte fragment halves inside a stage (fixed for the whole kernel).
   int woff[TN][2], xoff[TM][2];

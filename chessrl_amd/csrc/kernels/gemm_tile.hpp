@@ -133,9 +133,11 @@ __device__ __forceinline__ void store8(void* base, long off, const float v[8]) {
 // s0 = 1/std and s1 = -mean/std of row m, from the row statistics a.res_stats and the norm's gain and offset (the normalised tensor then never travels
 // through memory). sStats: 2*WM floats of LDS of this wave's own for its rows' statistics, filled here (RES_NORM 1)
 // or by the kernel before its main loop (RES_NORM 2).
-template <int WM, int WN, int OUT_DT, int RES_NORM = 0>
-__device__ __forceinline__ void gemm_epilogue(const GemmArgs& a, f32x16_t (&acc)[WN / 32][WM / 32], float* sC, int mw0, int nw0, int lane,
+template <int WM, int WN, int OUT_DT, int RES_NORM = 0, typename AccArr>
+__device__ __forceinline__ void gemm_epilogue(const GemmArgs& a, AccArr& acc, float* sC, int mw0, int nw0, int lane,
                                               float* sStats = nullptr) {
+  // acc is f32x16_t[WN/32][WM/32] (32x32 MFMA tiles) or f32x4_t[WN/16][WM/16] (16x16 tiles).
+  constexpr bool MI16 = sizeof(acc[0][0]) == sizeof(f32x4_t);
   constexpr int TM = WM / 32, TN = WN / 32, CH4 = WN / 4, CP = WN / 8, RSTEP = 64 / CP, ITERS = 32 / RSTEP;
   const int lr = lane & 31, g = lane >> 5;
   const int ec = lane % CP, er = lane / CP;
@@ -227,14 +229,25 @@ __device__ __forceinline__ void gemm_epilogue(const GemmArgs& a, f32x16_t (&acc)
       if (res32) { load_res(tm, 0, 0); load_res(tm, 1, 1); }
       else if constexpr (tm + 1 < TM) load_res(tm + 1, (tm + 1) & 1, 0);
     }
+    if constexpr (MI16) {
+      // A 16x16 tile holds, per lane, columns 4 (lane / 16) + {0..3} of row lane % 16: one 16-byte chunk of the patch row.
 #pragma unroll
-    for (int tn = 0; tn < TN; ++tn)
+      for (int wi = 0; wi < WN / 16; ++wi)
 #pragma unroll
-      for (int rq = 0; rq < 4; ++rq) {
-        const int chunk = tn * 8 + 2 * rq + g;
-        f32x4_t v4 = {acc[tn][tm][4 * rq], acc[tn][tm][4 * rq + 1], acc[tn][tm][4 * rq + 2], acc[tn][tm][4 * rq + 3]};
-        *reinterpret_cast<f32x4_t*>(sC + lr * WN + ((chunk ^ (lr & (CH4 - 1))) << 2)) = v4;
-      }
+        for (int xi = 0; xi < 2; ++xi) {
+          const int row = 16 * xi + (lane & 15), chunk = wi * 4 + (lane >> 4);
+          *reinterpret_cast<f32x4_t*>(sC + row * WN + ((chunk ^ (row & (CH4 - 1))) << 2)) = acc[wi][2 * tm + xi];
+        }
+    } else {
+#pragma unroll
+      for (int tn = 0; tn < TN; ++tn)
+#pragma unroll
+        for (int rq = 0; rq < 4; ++rq) {
+          const int chunk = tn * 8 + 2 * rq + g;
+          f32x4_t v4 = {acc[tn][tm][4 * rq], acc[tn][tm][4 * rq + 1], acc[tn][tm][4 * rq + 2], acc[tn][tm][4 * rq + 3]};
+          *reinterpret_cast<f32x4_t*>(sC + lr * WN + ((chunk ^ (lr & (CH4 - 1))) << 2)) = v4;
+        }
+    }
     wave_lds_fence();
     float v[ITERS][8];
 #pragma unroll
@@ -367,5 +380,9 @@ hipError_t launch_gemm_dma_resnorm(const GemmArgs& a, hipStream_t st);   // gemm
 hipError_t launch_gemm_pp(const GemmArgs& a, int out_dt, hipStream_t st);
 // The same tile on four waves of 128x128, software-pipelined inside the wave (gemm_sp.hip): e4m3 operands, bf16 or e4m3 output.
 hipError_t launch_gemm_sp(const GemmArgs& a, int out_dt, hipStream_t st);
+// gemm_dmaf.hip: the eight-wave in-step tile with address arithmetic kept out of the main loop (e4m3 operands, K % 128 == 0).
+hipError_t launch_gemm_dmaf(const GemmArgs& a, int out_dt, hipStream_t st);
+// gemm_sp2.hip: the same four waves fed in 128-byte slabs of K.
+hipError_t launch_gemm_sp2(const GemmArgs& a, int out_dt, hipStream_t st);
 
 }  // namespace crl

@@ -191,8 +191,8 @@ def test_gemm_fp8(cuda, M, N, K, tile):
 
 
 @pytest.mark.parametrize("M,N,K", [(256, 256, 64), (256, 256, 128), (256, 256, 192), (512, 1024, 1024), (4096, 1536, 1024), (2048, 3104, 1024), (1000, 3104, 1072),
-                                   (20000, 1024, 1536), (2048, 200, 512), (2048, 1700, 1040), (300, 700, 736), (256, 4096, 256), (4096, 1024, 4096)])
-@pytest.mark.parametrize("alt", [6, 8])
+                                   (20000, 1024, 1536), (2048, 200, 512), (2048, 1700, 1040), (300, 700, 736), (256, 4096, 256), (4096, 1024, 4096), (16384, 3104, 1024), (33000, 1024, 320)])
+@pytest.mark.parametrize("alt", [6, 8, 9, 10])
 def test_gemm_fp8_out_of_step_kernel_equals_in_step_kernel(cuda, M, N, K, alt):
     """The two other 256x256 e4m3 kernels, the one whose two waves per SIMD alternate between fragment reads and MFMAs
     (tile 6) and the four-wave software-pipelined one (tile 8), against the kernel whose eight waves work in step
@@ -210,8 +210,18 @@ def test_gemm_fp8_out_of_step_kernel_equals_in_step_kernel(cuda, M, N, K, alt):
         amax6, amax7 = torch.zeros(1, device=cuda), torch.zeros(1, device=cuda)
         o6 = run_gemm(A, W, kw["out_dt"], tile=alt, ldc=ldc, amax=amax6, **{k: v for k, v in kw.items() if k != "out_dt"})
         o7 = run_gemm(A, W, kw["out_dt"], tile=7, ldc=ldc, amax=amax7, **{k: v for k, v in kw.items() if k != "out_dt"})
-        assert torch.equal(o6, o7), (M, N, K, kw["out_dt"], (o6.float() - o7.float()).abs().max().item())
-        assert torch.equal(amax6, amax7)
+        if alt != 9:
+            assert torch.equal(o6, o7), (M, N, K, kw["out_dt"], (o6.float() - o7.float()).abs().max().item())
+            assert torch.equal(amax6, amax7)
+        else:
+            # 16x16x128 MFMAs add 128 products per instruction, 32x32x64 ones 64: fp32 summation-order noise, which
+            # the output rounding turns into a rare neighbouring code.
+            f6 = o6.view(torch.float8_e4m3fn).float() if kw["out_dt"] == _lib.FP8 else o6.float()
+            f7 = o7.view(torch.float8_e4m3fn).float() if kw["out_dt"] == _lib.FP8 else o7.float()
+            ulp = 2 ** -3 if kw["out_dt"] == _lib.FP8 else 2 ** -7
+            assert torch.allclose(f6, f7, rtol=ulp, atol=ulp * 2 ** -6), (M, N, K, (f6 - f7).abs().max().item())
+            assert (f6 != f7).float().mean().item() < 0.01
+            assert abs(amax6.item() - amax7.item()) <= 1e-5 * amax7.item()
     # and against torch on the same operands
     ref = (A.float() @ W.float().t()) * 1e-3
     out = run_gemm(A, W, _lib.BF16, descale=1e-3, tile=alt, ldc=ldc)
