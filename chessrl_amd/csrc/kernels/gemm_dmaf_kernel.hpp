@@ -21,7 +21,8 @@ struct DmafCfg {
   static constexpr int RING_BYTES = 2 * (BM + BN) * ROWB;   // 128 KB
   static constexpr int EPI_BYTES = NW * 32 * WN * 4;        // 64 KB: the two weight stages
   static constexpr int STATS_OFF = RING_BYTES + 256;        // behind the landing strip of the L2 touches
-  static constexpr int LDS_BYTES = STATS_OFF + NW * 2 * WM * 4;
+  static constexpr int COLS_OFF = STATS_OFF + NW * 2 * WM * 4;   // per-column epilogue constants: [wave][bias, gain, offset][WN]
+  static constexpr int LDS_BYTES = COLS_OFF + NW * 3 * WN * 4;
 };
 
 template <int OUT_DT, int RES_NORM = 0>
@@ -64,6 +65,23 @@ __global__ void __launch_bounds__(DmafCfg::NT, 2) gemm_dmaf_kernel(const GemmArg
   const int m0 = tile_m * BM, n0 = tile_n * BN;
   const int nslab = a.K / Cfg::ROWB;        // the launcher sends only K % 128 == 0 here
 
+  // The per-column constants of the epilogue (bias; gain and offset of a residual normalised on the fly) for this wave's
+  // 64 columns, one column per lane, landed outside the ring: requested first, in LDS long before the epilogue asks.
+  // Columns past N repeat the last one; nothing of theirs is stored.
+  {
+    int n = n0 + wn * Cfg::WN + lane;
+    n = n < a.N ? n : a.N - 1;
+    uint8_t* cols = smem + Cfg::COLS_OFF + wave * (3 * Cfg::WN * 4);
+    if (a.bias)
+      __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(a.bias + n), (__attribute__((address_space(3))) void*)cols, 4, 0, 0);
+    if constexpr (RES_NORM != 0) {
+      __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(a.res_gamma + n),
+                                       (__attribute__((address_space(3))) void*)(cols + Cfg::WN * 4), 4, 0, 0);
+      if (a.res_beta)
+        __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(a.res_beta + n),
+                                         (__attribute__((address_space(3))) void*)(cols + 2 * Cfg::WN * 4), 4, 0, 0);
+    }
+  }
   if constexpr (RES_NORM != 0) {
     // Statistics of this wave's 128 rows (two rows = 16 bytes per lane), requested before anything else and landed
     // outside the ring.
@@ -159,6 +177,7 @@ __global__ void __launch_bounds__(DmafCfg::NT, 2) gemm_dmaf_kernel(const GemmArg
   // A wave whose 128x64 part lies wholly outside C still takes its share of the loads and every barrier.
   const bool wave_active = (m0 + wm * Cfg::WM < a.M) && (n0 + wn * Cfg::WN < a.N);
 
+
   static_for<0, LOADS>([&](auto ic) { issue_one(0, rsrc_mine, ic); });
   for (int s0 = 1; s0 < 1 + pf; ++s0) prefetch(s0);
 
@@ -200,7 +219,8 @@ __global__ void __launch_bounds__(DmafCfg::NT, 2) gemm_dmaf_kernel(const GemmArg
 
   gemm_epilogue<Cfg::WM, Cfg::WN, OUT_DT, RES_NORM>(a, acc, reinterpret_cast<float*>(smem) + wave * (32 * Cfg::WN),
                                                      m0 + wm * Cfg::WM, n0 + wn * Cfg::WN, lane,
-                                                     reinterpret_cast<float*>(smem + Cfg::STATS_OFF) + wave * (2 * Cfg::WM));
+                                                     reinterpret_cast<float*>(smem + Cfg::STATS_OFF) + wave * (2 * Cfg::WM),
+                                                     reinterpret_cast<const float*>(smem + Cfg::COLS_OFF) + wave * (3 * Cfg::WN));
 }
 
 template <int OUT_DT, int RES_NORM = 0>

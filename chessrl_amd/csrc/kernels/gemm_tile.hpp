@@ -135,7 +135,10 @@ __device__ __forceinline__ void store8(void* base, long off, const float v[8]) {
 // or by the kernel before its main loop (RES_NORM 2).
 template <int WM, int WN, int OUT_DT, int RES_NORM = 0, typename AccArr>
 __device__ __forceinline__ void gemm_epilogue(const GemmArgs& a, AccArr& acc, float* sC, int mw0, int nw0, int lane,
-                                              float* sStats = nullptr) {
+                                              float* sStats = nullptr, const float* sCols = nullptr) {
+  // sCols (optional, LDS): per-column constants of this wave's WN columns that the kernel has staged before its main
+  // loop, so that the epilogue does not start by waiting for global memory: bias at [0, WN), and for RES_NORM the
+  // residual gain at [WN, 2 WN) and offset at [2 WN, 3 WN) (the parts whose pointers are null are not read).
   // acc is f32x16_t[WN/32][WM/32] (32x32 MFMA tiles) or f32x4_t[WN/16][WM/16] (16x16 tiles).
   constexpr bool MI16 = sizeof(acc[0][0]) == sizeof(f32x4_t);
   constexpr int TM = WM / 32, TN = WN / 32, CH4 = WN / 4, CP = WN / 8, RSTEP = 64 / CP, ITERS = 32 / RSTEP;
@@ -145,7 +148,16 @@ __device__ __forceinline__ void gemm_epilogue(const GemmArgs& a, AccArr& acc, fl
   const bool n_ok = n < a.N;
   const bool full = a.vec_ok && (n + 7 < a.N) && ((n < a.nsplit) == (n + 7 < a.nsplit));
   float bias8[8];
-  if (__builtin_expect(a.bias != nullptr && n + 7 < a.N && (reinterpret_cast<uintptr_t>(a.bias) & 15) == 0, 1)) {
+  if (sCols != nullptr) {
+    if (a.bias) {
+      const f32x4_t b0 = *reinterpret_cast<const f32x4_t*>(sCols + ec * 8), b1 = *reinterpret_cast<const f32x4_t*>(sCols + ec * 8 + 4);
+#pragma unroll
+      for (int e = 0; e < 4; ++e) { bias8[e] = b0[e]; bias8[4 + e] = b1[e]; }
+    } else {
+#pragma unroll
+      for (int e = 0; e < 8; ++e) bias8[e] = 0.f;
+    }
+  } else if (__builtin_expect(a.bias != nullptr && n + 7 < a.N && (reinterpret_cast<uintptr_t>(a.bias) & 15) == 0, 1)) {
     const f32x4_t b0 = *reinterpret_cast<const f32x4_t*>(a.bias + n), b1 = *reinterpret_cast<const f32x4_t*>(a.bias + n + 4);
 #pragma unroll
     for (int e = 0; e < 4; ++e) { bias8[e] = b0[e]; bias8[4 + e] = b1[e]; }
@@ -160,11 +172,22 @@ __device__ __forceinline__ void gemm_epilogue(const GemmArgs& a, AccArr& acc, fl
   if constexpr (RES_NORM) {
     // offset_n joins the bias (which is multiplied by alpha below); the statistics of this wave's rows go to LDS.
     const float inv_alpha = 1.0f / alpha;
+    if (sCols != nullptr) {
+      const f32x4_t g0 = *reinterpret_cast<const f32x4_t*>(sCols + WN + ec * 8), g1 = *reinterpret_cast<const f32x4_t*>(sCols + WN + ec * 8 + 4);
 #pragma unroll
-    for (int e = 0; e < 8; ++e) {
-      const bool ok = n + e < a.N;
-      gain8[e] = ok ? a.res_gamma[n + e] : 0.f;
-      if (a.res_beta && ok) bias8[e] += a.res_beta[n + e] * inv_alpha;
+      for (int e = 0; e < 4; ++e) { gain8[e] = g0[e]; gain8[4 + e] = g1[e]; }
+      if (a.res_beta) {
+        const f32x4_t o0 = *reinterpret_cast<const f32x4_t*>(sCols + 2 * WN + ec * 8), o1 = *reinterpret_cast<const f32x4_t*>(sCols + 2 * WN + ec * 8 + 4);
+#pragma unroll
+        for (int e = 0; e < 4; ++e) { bias8[e] += o0[e] * inv_alpha; bias8[4 + e] += o1[e] * inv_alpha; }
+      }
+    } else {
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        const bool ok = n + e < a.N;
+        gain8[e] = ok ? a.res_gamma[n + e] : 0.f;
+        if (a.res_beta && ok) bias8[e] += a.res_beta[n + e] * inv_alpha;
+      }
     }
     if constexpr (RES_NORM == 1) {   // (2: the kernel has staged them before its main loop)
 #pragma unroll
