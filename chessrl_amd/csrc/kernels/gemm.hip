@@ -593,18 +593,24 @@ static hipError_t launch_in_out(const GemmArgs& a, int tile, hipStream_t st) {
     if constexpr (IN_DT == DT_FP8 && (OUT_DT == DT_BF16 || OUT_DT == DT_FP8)) return launch_gemm_sp(a, OUT_DT, st);
     else return hipErrorInvalidValue;
   }
-  // The 256x256 tile of e4m3 operands has two kernels: four software-pipelined waves (tile 9) where K is whole 128-byte
-  // slabs, and eight waves in step (tile 7). The first has the faster main loop (1.63 against 1.96 us per slab) and the
-  // slower prologue and epilogue (10.0 against 7.7 us per tile): it takes over from K = 768 on.
-  if (tile == 9 && a.K % 128 != 0) tile = 7;
-  if constexpr (IN_DT == DT_FP8 && OUT_DT != DT_F32) {
-    if (tile == 3 && a.K % 128 == 0) tile = a.K >= 4096 ? 9 : 10;
-    if (tile == 9) return launch_gemm_sp2(a, OUT_DT, st);
-    if (tile == 10 && a.K % 128 != 0) tile = 7;
-    if (tile == 10) return launch_gemm_dmaf(a, OUT_DT, st);
-  } else {
-    if (tile == 9 || tile == 10) return hipErrorInvalidValue;
+  // The 256x256 tile has three kernels. Eight waves in step (gemm_dma_kernel.hpp, tile 7): every operand type, any K. The
+  // same with its address arithmetic out of the main loop (gemm_dmaf_kernel.hpp, tile 10): K in whole 128-byte slabs;
+  // bit-equal and faster (the GEMMs of a 4096-position e4m3 forward: -4.9 %), so tile 3 means this one where it exists.
+  // Four software-pipelined waves with 16x16x128 MFMAs (gemm_sp2_kernel.hpp, tile 9): e4m3, whole slabs; the faster main
+  // loop (1.63 against 1.96 us per slab on random data) and the slower prologue and epilogue (10.0 against 7.7 us per
+  // tile): it takes over from K = 4096 on.
+  constexpr int ESZ = IN_DT == DT_FP8 ? 1 : 2;
+  const bool slabs = (a.K * ESZ) % 128 == 0;
+  if ((tile == 9 || tile == 10) && !slabs) tile = 7;
+  if (tile == 3 && slabs) {
+    if (IN_DT == DT_FP8 && OUT_DT != DT_F32 && a.K >= 4096 && !a.res_stats) tile = 9;
+    else if (gemm_dmaf_has(IN_DT, OUT_DT, a.res_stats != nullptr)) tile = 10;
   }
+  if (tile == 9) {
+    if constexpr (IN_DT == DT_FP8 && OUT_DT != DT_F32) return launch_gemm_sp2(a, OUT_DT, st);
+    else return hipErrorInvalidValue;
+  }
+  if (tile == 10) return gemm_dmaf_has(IN_DT, OUT_DT, a.res_stats != nullptr) ? launch_gemm_dmaf(a, IN_DT, OUT_DT, st) : hipErrorInvalidValue;
   if (tile == 3 || tile == 7) return launch_gemm_dma(a, IN_DT, OUT_DT, st);
   if (tile == 2) return launch_cfg<CfgMid, IN_DT, OUT_DT>(a, st);
   if (tile == 5) return launch_cfg<CfgSmallK4, IN_DT, OUT_DT>(a, st);

@@ -1,4 +1,4 @@
-// C[M,N] = epilogue(A[M,K] · W[N,K]^T), e4m3 operands, K a whole number of 128-byte slabs: the eight-wave in-step
+// C[M,N] = epilogue(A[M,K] · W[N,K]^T), e4m3 or 16-bit operands, K a whole number of 128-byte slabs: the eight-wave in-step
 // 256x256 kernel of gemm_dma_kernel.hpp with its address arithmetic taken out of the main loop. There a wave issues,
 // per slab of 16 MFMAs, 24 LDS reads and 8 loads, another 85 vector ALU instructions: a 64-bit add, a compare and two
 // selects per load (slab offset, K tail from a block of zeros), an add per fragment read. Here
@@ -25,10 +25,11 @@ struct DmafCfg {
   static constexpr int LDS_BYTES = COLS_OFF + NW * 3 * WN * 4;
 };
 
-template <int OUT_DT, int RES_NORM = 0>
+template <int IN_DT, int OUT_DT, int RES_NORM = 0>
 __global__ void __launch_bounds__(DmafCfg::NT, 2) gemm_dmaf_kernel(const GemmArgs a, const int pf) {
   typedef DmafCfg Cfg;
-  constexpr int IN_DT = DT_FP8;
+  constexpr int ESZ = IN_DT == DT_FP8 ? 1 : 2;                      // bytes per operand element
+  constexpr int KSTEPS = Cfg::ROWB / (IN_DT == DT_FP8 ? 64 : 32);   // MFMA K steps per slab
   constexpr int BM = Cfg::BM, BN = Cfg::BN, TM = Cfg::TM, TN = Cfg::TN, LOADS = Cfg::LOADS;
   extern __shared__ __align__(16) uint8_t smem[];
 
@@ -50,7 +51,8 @@ __global__ void __launch_bounds__(DmafCfg::NT, 2) gemm_dmaf_kernel(const GemmArg
   {
     constexpr int GM = 8;
     const int tiles_m = (a.M + BM - 1) / BM;
-    if (tiles_m % GM == 0) {
+    // (16-bit operands keep the plain row-major order unless the columns divide by four, as in gemm_dma_kernel.hpp)
+    if (tiles_m % GM == 0 && (IN_DT == DT_FP8 || tiles_n % 4 == 0)) {
       const int ngrp = (tiles_n + 3) >> 2, wb = tiles_n / ngrp, extra = tiles_n - wb * ngrp;
       const int sr = pid / (GM * tiles_n), rem = pid - sr * (GM * tiles_n);
       const int big = GM * (wb + 1) * extra;
@@ -63,7 +65,7 @@ __global__ void __launch_bounds__(DmafCfg::NT, 2) gemm_dmaf_kernel(const GemmArg
     }
   }
   const int m0 = tile_m * BM, n0 = tile_n * BN;
-  const int nslab = a.K / Cfg::ROWB;        // the launcher sends only K % 128 == 0 here
+  const int nslab = a.K * ESZ / Cfg::ROWB;  // the launcher sends only whole slabs of K here
 
   // The per-column constants of the epilogue (bias; gain and offset of a residual normalised on the fly) for this wave's
   // 64 columns, one column per lane, landed outside the ring: requested first, in LDS long before the epilogue asks.
@@ -96,7 +98,7 @@ __global__ void __launch_bounds__(DmafCfg::NT, 2) gemm_dmaf_kernel(const GemmArg
   // wave's 64 has swizzle (lane / 8) ^ i).
   const bool loads_a = wave >= 4;
   const int rbase = (wave & 3) * 64;
-  const int ld = loads_a ? a.lda : a.ldw;
+  const int ld = (loads_a ? a.lda : a.ldw) * ESZ;   // row stride in bytes
   const int rows_left = loads_a ? a.M - m0 : a.N - n0;
   uint32_t voff[LOADS];
 #pragma unroll
@@ -109,8 +111,8 @@ __global__ void __launch_bounds__(DmafCfg::NT, 2) gemm_dmaf_kernel(const GemmArg
     const long span = (rows < 256 ? rows : 256) * ldb;
     return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(base), 0, (int)(span < 0x7fffffffL ? span : 0x7fffffffL), 0x00020000);
   };
-  const __amdgpu_buffer_rsrc_t rsrc_w = make_rsrc(reinterpret_cast<const uint8_t*>(a.W) + (long)n0 * a.ldw, a.N - n0, a.ldw);
-  const __amdgpu_buffer_rsrc_t rsrc_x = make_rsrc(reinterpret_cast<const uint8_t*>(a.A) + (long)m0 * a.lda, a.M - m0, a.lda);
+  const __amdgpu_buffer_rsrc_t rsrc_w = make_rsrc(reinterpret_cast<const uint8_t*>(a.W) + (long)n0 * a.ldw * ESZ, a.N - n0, (long)a.ldw * ESZ);
+  const __amdgpu_buffer_rsrc_t rsrc_x = make_rsrc(reinterpret_cast<const uint8_t*>(a.A) + (long)m0 * a.lda * ESZ, a.M - m0, (long)a.lda * ESZ);
   const __amdgpu_buffer_rsrc_t rsrc_none = __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(a.A), 0, 0, 0x00020000);
   const __amdgpu_buffer_rsrc_t rsrc_mine = loads_a ? rsrc_x : rsrc_w;
   const uint32_t lds_load0 = (loads_a ? 65536u : 0u) + rbase * Cfg::ROWB;   // stage 0
@@ -129,13 +131,13 @@ __global__ void __launch_bounds__(DmafCfg::NT, 2) gemm_dmaf_kernel(const GemmArg
       pf_n = (4 + grp_w - 1) / grp_w;
       int r = ((grp_q * pf_n) & 3) * 64 + lane;
       r = r < a.M - m0 ? r : a.M - m0 - 1;
-      pf_off = (uint32_t)r * (uint32_t)a.lda;
-      pf_step = (m0 + 256 <= a.M) ? 64 * a.lda : 0;
+      pf_off = (uint32_t)r * (uint32_t)(a.lda * ESZ);
+      pf_step = (m0 + 256 <= a.M) ? 64 * a.lda * ESZ : 0;
     } else {
       pf_n = 1;
       int r = (tile_m & 7) * 32 + (lane & 31);
       r = r < a.N - n0 ? r : a.N - n0 - 1;
-      pf_off = (uint32_t)r * (uint32_t)a.ldw + (lane >> 5) * 64;
+      pf_off = (uint32_t)r * (uint32_t)(a.ldw * ESZ) + (lane >> 5) * 64;
     }
   }
   const __amdgpu_buffer_rsrc_t rsrc_pf = wave == 0 ? rsrc_x : rsrc_w;
@@ -155,22 +157,23 @@ __global__ void __launch_bounds__(DmafCfg::NT, 2) gemm_dmaf_kernel(const GemmArg
 #pragma unroll
       for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
 
-  // Fragment addresses. The 16-byte piece (K step ks, half) of row 32 t + lr of a wave's block sits at chunk
-  // (4 ks + half + 2g) ^ swizzle(row), and swizzle(row) = swizzle(lr) ^ 4 (t & 1): with L = 2g ^ swizzle(lr) the chunk is
-  // Kc ^ L for the compile-time Kc = (4 ks + half) ^ 4 (t & 1), one of 0, 1, 4, 5. Four lane addresses per operand (one
-  // per Kc) plus the immediate 4096 t cover every read of a stage.
-  const int L0 = (2 * g) ^ lds_swizzle(lr);
+  // Fragment addresses. A lane's 16-byte piece of row 32 t + lr of a wave's block sits at chunk c ^ swizzle(row) with
+  // c = 4 ks + half + 2g for e4m3 (two pieces per K step of 64 bytes) and c = 2 ks + g for 16-bit operands (one piece
+  // per K step of 32 bytes), and swizzle(row) = swizzle(lr) ^ 4 (t & 1). With L = (2g or g) ^ swizzle(lr) the chunk is
+  // Kc ^ L for a compile-time Kc that takes four values (0, 1, 4, 5 or 0, 2, 4, 6): four lane addresses per operand
+  // plus the immediate 4096 t cover every read of a stage.
+  const int L0 = (IN_DT == DT_FP8 ? 2 * g : g) ^ lds_swizzle(lr);
   const uint32_t lds0 = (uint32_t)reinterpret_cast<uintptr_t>((__attribute__((address_space(3))) uint8_t*)smem);
   uint32_t wb[4], xb[4];
 #pragma unroll
   for (int k = 0; k < 4; ++k) {
-    const int kc = (k & 1) | ((k >> 1) << 2);
+    const int kc = IN_DT == DT_FP8 ? ((k & 1) | ((k >> 1) << 2)) : 2 * k;
     wb[k] = lds0 + (wn * Cfg::WN + lr) * Cfg::ROWB + ((kc ^ L0) << 4);
     xb[k] = lds0 + 65536 + (wm * Cfg::WM + lr) * Cfg::ROWB + ((kc ^ L0) << 4);
   }
   auto read_piece = [&](bool is_w, int t, int ks, int half) -> i32x4_t {
-    const int kc = (4 * ks + half) ^ (4 * (t & 1));
-    const int k = (kc & 1) | ((kc >> 2) << 1);
+    const int kc = (IN_DT == DT_FP8 ? 4 * ks + half : 2 * ks) ^ (4 * (t & 1));
+    const int k = IN_DT == DT_FP8 ? ((kc & 1) | ((kc >> 2) << 1)) : kc >> 1;
     return *reinterpret_cast<const __attribute__((address_space(3))) i32x4_t*>((is_w ? wb[k] : xb[k]) + t * 32 * Cfg::ROWB);
   };
 
@@ -190,19 +193,28 @@ __global__ void __launch_bounds__(DmafCfg::NT, 2) gemm_dmaf_kernel(const GemmArg
       static_for<0, LOADS>([&](auto ic) { issue_one(slab + 1, rnext, ic); });
       continue;
     }
-    static_for<0, 2>([&](auto ksc) {
+    constexpr bool SPREAD = IN_DT == DT_FP8;   // 16-bit operands measure 2-3 % slower with their loads spread out
+    if constexpr (!SPREAD) static_for<0, LOADS>([&](auto ic) { issue_one(slab + 1, rnext, ic); });
+    static_for<0, KSTEPS>([&](auto ksc) {
       constexpr int ks = decltype(ksc)::value;
       Frag<IN_DT> wf[TN], xf[TM];
 #pragma unroll
-      for (int tn = 0; tn < TN; ++tn) { wf[tn].lo = read_piece(true, tn, ks, 0); wf[tn].hi = read_piece(true, tn, ks, 1); }
+      for (int tn = 0; tn < TN; ++tn) {
+        wf[tn].lo = read_piece(true, tn, ks, 0);
+        if constexpr (IN_DT == DT_FP8) wf[tn].hi = read_piece(true, tn, ks, 1);
+      }
 #pragma unroll
-      for (int tm = 0; tm < TM; ++tm) { xf[tm].lo = read_piece(false, tm, ks, 0); xf[tm].hi = read_piece(false, tm, ks, 1); }
+      for (int tm = 0; tm < TM; ++tm) {
+        xf[tm].lo = read_piece(false, tm, ks, 0);
+        if constexpr (IN_DT == DT_FP8) xf[tm].hi = read_piece(false, tm, ks, 1);
+      }
       static_for<0, TN * TM>([&](auto ic) {
         constexpr int i = decltype(ic)::value;
         constexpr int tn = i / TM, tm = i % TM;
         acc[tn][tm] = mfma_frag<IN_DT>(wf[tn], xf[tm], acc[tn][tm]);
-        // The next slab's loads go out one at a time, after every second MFMA, held in place by scheduling barriers.
-        if constexpr ((i & 1) == 1) {
+        // With e4m3 operands the next slab's loads go out one at a time, after every second MFMA, held in place by
+        // scheduling barriers.
+        if constexpr (SPREAD && (i & 1) == 1) {
           __builtin_amdgcn_sched_barrier(0);
           issue_one(slab + 1, rnext, std::integral_constant<int, ks * 4 + (i >> 1)>{});
           __builtin_amdgcn_sched_barrier(0);
@@ -223,15 +235,16 @@ __global__ void __launch_bounds__(DmafCfg::NT, 2) gemm_dmaf_kernel(const GemmArg
                                                      reinterpret_cast<const float*>(smem + Cfg::COLS_OFF) + wave * (3 * Cfg::WN));
 }
 
-template <int OUT_DT, int RES_NORM = 0>
+template <int IN_DT, int OUT_DT, int RES_NORM = 0>
 static hipError_t launch_dmaf(const GemmArgs& a, hipStream_t st) {
   static std::atomic<bool> attr_set[16] = {};
   hipError_t e = hipSuccess;
   // Whole slabs of K only, and lane offsets inside a tile's 256 rows that fit 31 bits.
-  if (a.K % DmafCfg::ROWB != 0 || a.K <= 0 || (long)a.lda * 256 >= (1L << 31) || (long)a.ldw * 256 >= (1L << 31)) return hipErrorInvalidValue;
+  constexpr int ESZ = IN_DT == DT_FP8 ? 1 : 2;
+  if ((a.K * ESZ) % DmafCfg::ROWB != 0 || a.K <= 0 || (long)a.lda * ESZ * 256 >= (1L << 31) || (long)a.ldw * ESZ * 256 >= (1L << 31)) return hipErrorInvalidValue;
   int dev = 0;
   (void)hipGetDevice(&dev);
-  auto kern = gemm_dmaf_kernel<OUT_DT, RES_NORM>;
+  auto kern = gemm_dmaf_kernel<IN_DT, OUT_DT, RES_NORM>;
   if (!attr_set[dev]) {
     e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, DmafCfg::LDS_BYTES);
     if (e != hipSuccess) return e;
@@ -239,7 +252,8 @@ static hipError_t launch_dmaf(const GemmArgs& a, hipStream_t st) {
   }
   const int tiles_n = (a.N + DmafCfg::BN - 1) / DmafCfg::BN;
   const int tiles = ((a.M + DmafCfg::BM - 1) / DmafCfg::BM) * tiles_n;
-  const int pf = (tiles_n % 4 == 0 && (long)a.K >= 8 * DmafCfg::ROWB) ? 2 : 0;
+  // (the L2 touches pay for e4m3 operands only: the 16-bit instances lose 2-6 % with them)
+  const int pf = (IN_DT == DT_FP8 && tiles_n % 4 == 0 && (long)a.K >= 8 * DmafCfg::ROWB) ? 2 : 0;
   hipLaunchKernelGGL(kern, dim3(tiles), dim3(DmafCfg::NT), DmafCfg::LDS_BYTES, st, a, pf);
   return hipGetLastError();
 }

@@ -1,10 +1,5 @@
 // Instances of the four-wave software-pipelined 256x256 e4m3 GEMM fed in 128-byte slabs (gemm_sp2_kernel.hpp), in a
 // translation unit of their own.
-#ifdef CRL_STAMP
-#include <hip/hip_runtime.h>
-namespace crl { __device__ long g_sp2_stamps[4 * 4096]; }
-extern "C" int crl_debug_stamps(long* out, int n) { return (int)hipMemcpyFromSymbol(out, HIP_SYMBOL(crl::g_sp2_stamps), n * sizeof(long)); }
-#endif
 #include "gemm_sp2_kernel.hpp"
 
 namespace crl {

@@ -59,9 +59,6 @@ __global__ void __launch_bounds__(Sp2Cfg::NT) gemm_sp2_kernel(const GemmArgs a) 
   typedef Sp2Cfg Cfg;
   constexpr int BM = Cfg::BM, BN = Cfg::BN;
   extern __shared__ __align__(16) uint8_t smem[];
-#ifdef CRL_STAMP
-  const long stamp0 = wall_clock64();
-#endif
 
   // (the wave index as a scalar: everything derived from it, LDS destinations and global bases, stays in scalar registers)
   const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -211,9 +208,6 @@ __global__ void __launch_bounds__(Sp2Cfg::NT) gemm_sp2_kernel(const GemmArgs a) 
   issue_loads(1, nslab > 1);
   wait_vmcnt<16>();
   sp_barrier();
-#ifdef CRL_STAMP
-  const long stamp1 = wall_clock64();
-#endif
 
   if (wave_active) {
     // Slab 0: every fragment but the three that slots 0 and 1 fetch, then its slots 0-3. The loop body runs from slot
@@ -244,17 +238,10 @@ __global__ void __launch_bounds__(Sp2Cfg::NT) gemm_sp2_kernel(const GemmArgs a) 
   // the accumulators.
   asm volatile("s_nop 15\n\ts_nop 15\n\ts_nop 15" ::: "memory");
   sp_barrier();   // every wave is done with the ring before it becomes epilogue scratch
-#ifdef CRL_STAMP
-  const long stamp2 = wall_clock64();
-#endif
 
   gemm_epilogue<Cfg::WM, Cfg::WN, OUT_DT, RES_NORM>(a, acc, reinterpret_cast<float*>(smem) + wave * (32 * Cfg::WN),
                                                      m0 + wm * Cfg::WM, n0 + wn * Cfg::WN, lane,
                                                      reinterpret_cast<float*>(smem + Cfg::STATS_OFF) + wave * (2 * Cfg::WM));
-#ifdef CRL_STAMP
-  __builtin_amdgcn_s_waitcnt(0);
-  if (threadIdx.x == 0 && blockIdx.x < 4096) { long* o = g_sp2_stamps + 4 * blockIdx.x; o[0] = stamp0; o[1] = stamp1; o[2] = stamp2; o[3] = wall_clock64(); }
-#endif
 }
 
 template <int OUT_DT, int RES_NORM = 0>

@@ -403,8 +403,9 @@ hipError_t launch_gemm_dma_resnorm(const GemmArgs& a, hipStream_t st);   // gemm
 hipError_t launch_gemm_pp(const GemmArgs& a, int out_dt, hipStream_t st);
 // The same tile on four waves of 128x128, software-pipelined inside the wave (gemm_sp.hip): e4m3 operands, bf16 or e4m3 output.
 hipError_t launch_gemm_sp(const GemmArgs& a, int out_dt, hipStream_t st);
-// gemm_dmaf.hip: the eight-wave in-step tile with address arithmetic kept out of the main loop (e4m3 operands, K % 128 == 0).
-hipError_t launch_gemm_dmaf(const GemmArgs& a, int out_dt, hipStream_t st);
+// gemm_dmaf.hip: the eight-wave in-step tile with address arithmetic kept out of the main loop (K in whole 128-byte slabs).
+bool gemm_dmaf_has(int in_dt, int out_dt, bool res_norm);
+hipError_t launch_gemm_dmaf(const GemmArgs& a, int in_dt, int out_dt, hipStream_t st);
 // gemm_sp2.hip: the same four waves fed in 128-byte slabs of K.
 hipError_t launch_gemm_sp2(const GemmArgs& a, int out_dt, hipStream_t st);
 
