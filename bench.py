@@ -46,7 +46,51 @@ def parse():
     ap.add_argument("--act-dtype", default="bf16", choices=["bf16", "f16"], help="16-bit element type of activations and weights")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run three 1 GiB device copies, a kernel of known traffic to scale profiler byte counters with")
+    ap.add_argument("--gemm", default="", metavar="M,N,K",
+                    help="instead of a workload: time one crl_gemm product (3 warm-up + --steps launches, Gaussian operands) and print one JSON line")
+    ap.add_argument("--gemm-tile", type=int, default=0, help="tile code of crl_gemm for --gemm (0 = the library's choice)")
+    ap.add_argument("--gemm-in", default="fp8", choices=["fp8", "bf16"], help="operand type for --gemm (output is bf16)")
+    ap.add_argument("--gemm-vendor", action="store_true",
+                    help="with --gemm: time the vendor library on the same product instead (torch._scaled_mm / torch.matmul), as a yardstick")
     return ap.parse_args()
+
+
+def gemm_probe(a, torch, _lib, dev):
+    """One product C[M,N] = A[M,K] W[N,K]^T through the C-ABI (or, as a yardstick, through the vendor library), for
+    profiler runs on a single kernel: operands ~ N(0, 100^2) rounded to e4m3 (or N(0,1) in bf16), bf16 output."""
+    import ctypes as ct
+    M, N, K = [int(x) for x in a.gemm.split(",")]
+    fp8 = a.gemm_in == "fp8"
+    if fp8:
+        A = (torch.randn(M, K, device=dev) * 100).to(torch.float8_e4m3fn)
+        W = (torch.randn(N, K, device=dev) * 100).to(torch.float8_e4m3fn)
+    else:
+        A = torch.randn(M, K, device=dev).bfloat16()
+        W = torch.randn(N, K, device=dev).bfloat16()
+    out = torch.empty(M, N, dtype=torch.bfloat16, device=dev)
+    p = lambda t: ct.c_void_p(t.data_ptr())
+    st = ct.c_void_p(torch.cuda.current_stream().cuda_stream)
+    if a.gemm_vendor:
+        one = torch.tensor(1.0, device=dev)
+        run = (lambda: torch._scaled_mm(A, W.t(), scale_a=one, scale_b=one, out_dtype=torch.bfloat16)) if fp8 else (lambda: torch.matmul(A, W.t()))
+    else:
+        lib = _lib.lib()
+        def run():
+            _lib.check(lib.crl_gemm(p(A), K, p(W), K, p(out), N, M, N, K, _lib.FP8 if fp8 else _lib.BF16, _lib.BF16, None, 0, 1.0, 1.0,
+                                    None, N, _lib.BF16, 1.0, None, a.gemm_tile, st))
+    for _ in range(3):
+        run()
+    torch.cuda.synchronize()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    e0.record()
+    for _ in range(a.steps):
+        run()
+    e1.record()
+    torch.cuda.synchronize()
+    us = e0.elapsed_time(e1) / a.steps * 1e3
+    print(json.dumps({"metric": "one GEMM product", "M": M, "N": N, "K": K, "operands": a.gemm_in, "tile": a.gemm_tile,
+                      "vendor_yardstick": bool(a.gemm_vendor), "us_per_launch": round(us, 1), "tflops": round(2.0 * M * N * K / us / 1e6, 1),
+                      "launches": a.steps + 3}))
 
 
 def grpo_scoring(a, torch, models, board, dev):
@@ -140,6 +184,8 @@ def main():
         print("bench.py needs an MI355X (no CPU fallback for the measured path)", file=sys.stderr)
         sys.exit(2)
     dev = torch.device("cuda:0")
+    if a.gemm:
+        return gemm_probe(a, torch, _lib, dev)
     if a.workload.startswith("grpo_scoring"):
         return grpo_scoring(a, torch, models, board, dev)
     if a.workload.startswith("grpo_rollout"):
@@ -185,7 +231,7 @@ def main():
     peak = PEAK_TFLOPS["fp8" if fp8 else "bf16"]
     achieved = g["flops"] / (g["ms"] * 1e-3) / 1e12 if g["ms"] > 0 else 0.0
     roofline = {
-        "bound": "mfma", "kernel": "gemm_dma_kernel<256x256, %s>" % ("fp8" if fp8 else a.act_dtype),
+        "bound": "mfma", "kernel": "gemm_dmaf_kernel<%s> (256x256 tile)" % ("fp8" if fp8 else a.act_dtype),
         "achieved": round(achieved, 1), "peak": peak, "unit": "TFLOP/s", "frac": round(achieved / peak, 4),
         "traffic": TRAFFIC_BYTES.get(a.workload, (None, None))[0], "traffic_source": TRAFFIC_BYTES.get(a.workload, (None, None))[1],
         "avg_launch_us": round(g["ms"] * 1e3 / max(g["launches"], 1), 2), "launches": g["launches"],

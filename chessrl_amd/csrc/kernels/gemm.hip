@@ -386,11 +386,10 @@ __global__ void __launch_bounds__(256) splitk_reduce_ln_kernel(const GemmArgs a,
 //                 BM   BN  WGM WGN stages frag_db min_waves
 // Measured on MI355X (M=65536, N=1024..3072, K=1024..8192, fp8 and bf16, same job): the 256x256
 // tile fed by direct-to-LDS loads with 128-byte rows and two stages (DmaCfg2) is 10-20 % faster
-// than the same 8-wave tile with register staging; the 4-wave 256x256 tile (one wave per SIMD,
-// with or without double-buffered fragments), a 256x128 single-stage tile at two workgroups per
-// CU, a 4-stage ring of 64-byte rows (twice the barriers) and a persistent
-// one-workgroup-per-CU loop (epilogue stores of tile t delay the first slab of tile t+1 because
-// loads and stores share vmcnt) were all slower. The register-staged kernel serves the small tiles.
+// than the same 8-wave tile with register staging; a 256x128 single-stage tile at two workgroups per
+// CU, a 4-stage ring of 64-byte rows (twice the barriers) and a one-workgroup-per-CU loop over several
+// tiles (with bare barriers and a counted wait past the previous tile's stores too) were slower or equal.
+// The register-staged kernel serves the small tiles.
 typedef GemmCfg<128, 128, 2, 2, 2, 0, 2> CfgMid;    // 4 waves, 64x64 per wave, two workgroups per CU
 typedef GemmCfg<64, 64, 2, 2, 2, 0, 2> CfgSmall;    // 4 waves, 32x32 per wave
 typedef GemmCfg<64, 64, 2, 2, 2, 0, 2, 4> CfgSmallK4;   // the same tile walked by 4 groups of 4 waves, K slabs in turn

@@ -109,9 +109,13 @@ int crl_random_positions(uint64_t seed, int n, int max_plies, double late_fracti
  * LDS. Both are deterministic from launch to launch but differ from 1-3 in summation order. With tile 0, outputs of at
  * most 256 columns whose K is 4 KB or more per row are always K-sliced the same way (a function of N and K alone), so
  * the row-count independence holds for them too. The first K-sliced launch on a stream allocates that stream's
- * workspace: issue it once outside any graph capture. 6-8 name the three 256x256 kernels for e4m3 operands with bf16 or
- * e4m3 output explicitly (same sums, bit-equal results): 7 = eight waves in step (what 3 runs), 6 = the two waves of a
- * SIMD out of step, 8 = four software-pipelined waves; 6 and 8 exist for measurement and are slower. */
+ * workspace: issue it once outside any graph capture. 6-10 name the 256x256 kernels explicitly: 7 = eight waves in
+ * step (any K, any operand type), 10 = the same with its address arithmetic kept out of the main loop (K in whole
+ * 128-byte slabs; 3 runs this one where it applies), both with the sums and result bits of 1-3; 9 = four
+ * software-pipelined waves with 16x16x128 MFMAs (e4m3 operands, whole slabs; what 3 runs from K = 4096 on; these MFMAs
+ * add 128 products per instruction instead of 64, so a sum can differ from the others' in its last fp32 bits); 6 = the
+ * two waves of a SIMD out of step and 8 = four software-pipelined waves fed in 64-byte pieces (e4m3 operands, bit-equal
+ * to 7) exist for measurement and are slower. 9 and 10 fall back to 7 where K is not whole slabs. */
 int crl_gemm(const void* A, int64_t lda, const void* W, int64_t ldw, void* C, int64_t ldc,
              int M, int N, int K, int in_dtype, int out_dtype,
              const float* bias, int act, float descale, float alpha,
