@@ -603,7 +603,7 @@ static hipError_t launch_in_out(const GemmArgs& a, int tile, hipStream_t st) {
   if ((tile == 9 || tile == 10) && !slabs) tile = 7;
   if (tile == 3 && slabs) {
     if (IN_DT == DT_FP8 && OUT_DT != DT_F32 && a.K >= 4096 && !a.res_stats) tile = 9;
-    else if (gemm_dmaf_has(IN_DT, OUT_DT, a.res_stats != nullptr)) tile = 10;
+    else if (gemm_dmaf_has(IN_DT, OUT_DT, a.res_stats != nullptr) && (long)((a.M + 255) / 256) * ((a.N + 255) / 256) < 65536) tile = 10;
   }
   if (tile == 9) {
     if constexpr (IN_DT == DT_FP8 && OUT_DT != DT_F32) return launch_gemm_sp2(a, OUT_DT, st);

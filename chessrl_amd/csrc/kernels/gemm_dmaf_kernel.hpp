@@ -25,8 +25,33 @@ struct DmafCfg {
   static constexpr int LDS_BYTES = COLS_OFF + NW * 3 * WN * 4;
 };
 
+// The tile walk's constants, worked out once on the host: the walk divides a workgroup index by six launch constants,
+// and as generic integer divisions those were most of the ~410 instructions a workgroup issued before its first load.
+// q = n / d for n, d < 65536 is the high half of n * ceil(2^32 / d) (d = 1: n itself).
+struct DmafWalk {
+  int tiles_n, grouped, wb, extra, big;
+  uint32_t m_tn, m_8tn, m_8w1, m_8w0, m_w1, m_w0;   // magics of tiles_n, 8 tiles_n, 8 (wb+1), 8 wb, wb+1, wb
+};
+inline uint32_t dmaf_magic(uint32_t d) { return d <= 1 ? 0u : (uint32_t)(((1ull << 32) + d - 1) / d); }
+__device__ __forceinline__ int dmaf_div(int n, uint32_t magic) { return magic ? (int)__umulhi((uint32_t)n, magic) : n; }
+inline DmafWalk dmaf_walk(int M, int N, bool fp8) {
+  DmafWalk w{};
+  const int tiles_n = (N + 255) / 256, tiles_m = (M + 255) / 256;
+  w.tiles_n = tiles_n;
+  // (16-bit operands keep the plain row-major order unless the columns divide by four, as in gemm_dma_kernel.hpp)
+  w.grouped = tiles_m % 8 == 0 && (fp8 || tiles_n % 4 == 0);
+  const int ngrp = (tiles_n + 3) >> 2;
+  w.wb = tiles_n / ngrp;
+  w.extra = tiles_n - w.wb * ngrp;
+  w.big = 8 * (w.wb + 1) * w.extra;
+  w.m_tn = dmaf_magic(tiles_n); w.m_8tn = dmaf_magic(8 * tiles_n);
+  w.m_8w1 = dmaf_magic(8 * (w.wb + 1)); w.m_8w0 = dmaf_magic(8 * w.wb);
+  w.m_w1 = dmaf_magic(w.wb + 1); w.m_w0 = dmaf_magic(w.wb);
+  return w;
+}
+
 template <int IN_DT, int OUT_DT, int RES_NORM = 0>
-__global__ void __launch_bounds__(DmafCfg::NT, 2) gemm_dmaf_kernel(const GemmArgs a, const int pf) {
+__global__ void __launch_bounds__(DmafCfg::NT, 2) gemm_dmaf_kernel(const GemmArgs a, const int pf, const DmafWalk wk) {
   typedef DmafCfg Cfg;
   constexpr int ESZ = IN_DT == DT_FP8 ? 1 : 2;                      // bytes per operand element
   constexpr int KSTEPS = Cfg::ROWB / (IN_DT == DT_FP8 ? 64 : 32);   // MFMA K steps per slab
@@ -38,7 +63,7 @@ __global__ void __launch_bounds__(DmafCfg::NT, 2) gemm_dmaf_kernel(const GemmArg
   const int wm = wave % Cfg::WGM, wn = wave / Cfg::WGM;
   const int lr = lane & 31, g = lane >> 5;
 
-  const int tiles_n = (a.N + BN - 1) / BN;
+  const int tiles_n = wk.tiles_n;
   const int nblk = gridDim.x;
   int pid = blockIdx.x;
   {
@@ -46,52 +71,21 @@ __global__ void __launch_bounds__(DmafCfg::NT, 2) gemm_dmaf_kernel(const GemmArg
     if (pid < (per << 3)) pid = (pid & 7) * per + (pid >> 3);
   }
   // Tile order inside an XCD's range: groups of 8 x w tiles (M x N), w = 3 or 4, as in gemm_dma_kernel.hpp.
-  int tile_m = pid / tiles_n, tile_n = pid - tile_m * tiles_n;
+  int tile_m = dmaf_div(pid, wk.m_tn), tile_n = pid - tile_m * tiles_n;
   int grp_w = 4, grp_q = tile_n & 3;
-  {
+  if (wk.grouped) {
     constexpr int GM = 8;
-    const int tiles_m = (a.M + BM - 1) / BM;
-    // (16-bit operands keep the plain row-major order unless the columns divide by four, as in gemm_dma_kernel.hpp)
-    if (tiles_m % GM == 0 && (IN_DT == DT_FP8 || tiles_n % 4 == 0)) {
-      const int ngrp = (tiles_n + 3) >> 2, wb = tiles_n / ngrp, extra = tiles_n - wb * ngrp;
-      const int sr = pid / (GM * tiles_n), rem = pid - sr * (GM * tiles_n);
-      const int big = GM * (wb + 1) * extra;
-      int gi, r2;
-      if (rem < big) { grp_w = wb + 1; gi = rem / (GM * grp_w); r2 = rem - gi * GM * grp_w; }
-      else { grp_w = wb; const int rem2 = rem - big; gi = rem2 / (GM * wb); r2 = rem2 - gi * GM * wb; gi += extra; }
-      grp_q = r2 % grp_w;
-      tile_m = sr * GM + r2 / grp_w;
-      tile_n = gi * wb + (gi < extra ? gi : extra) + grp_q;
-    }
+    const int wb = wk.wb, extra = wk.extra, big = wk.big;
+    const int sr = dmaf_div(pid, wk.m_8tn), rem = pid - sr * (GM * tiles_n);
+    int gi, r2, rq;
+    if (rem < big) { grp_w = wb + 1; gi = dmaf_div(rem, wk.m_8w1); r2 = rem - gi * GM * grp_w; rq = dmaf_div(r2, wk.m_w1); }
+    else { grp_w = wb; const int rem2 = rem - big; gi = dmaf_div(rem2, wk.m_8w0); r2 = rem2 - gi * GM * wb; rq = dmaf_div(r2, wk.m_w0); gi += extra; }
+    grp_q = r2 - rq * grp_w;
+    tile_m = sr * GM + rq;
+    tile_n = gi * wb + (gi < extra ? gi : extra) + grp_q;
   }
   const int m0 = tile_m * BM, n0 = tile_n * BN;
   const int nslab = a.K * ESZ / Cfg::ROWB;  // the launcher sends only whole slabs of K here
-
-  // The per-column constants of the epilogue (bias; gain and offset of a residual normalised on the fly) for this wave's
-  // 64 columns, one column per lane, landed outside the ring: requested first, in LDS long before the epilogue asks.
-  // Columns past N repeat the last one; nothing of theirs is stored.
-  {
-    int n = n0 + wn * Cfg::WN + lane;
-    n = n < a.N ? n : a.N - 1;
-    uint8_t* cols = smem + Cfg::COLS_OFF + wave * (3 * Cfg::WN * 4);
-    if (a.bias)
-      __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(a.bias + n), (__attribute__((address_space(3))) void*)cols, 4, 0, 0);
-    if constexpr (RES_NORM != 0) {
-      __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(a.res_gamma + n),
-                                       (__attribute__((address_space(3))) void*)(cols + Cfg::WN * 4), 4, 0, 0);
-      if (a.res_beta)
-        __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(a.res_beta + n),
-                                         (__attribute__((address_space(3))) void*)(cols + 2 * Cfg::WN * 4), 4, 0, 0);
-    }
-  }
-  if constexpr (RES_NORM != 0) {
-    // Statistics of this wave's 128 rows (two rows = 16 bytes per lane), requested before anything else and landed
-    // outside the ring.
-    int m = m0 + wm * Cfg::WM + 2 * lane;
-    m = m + 1 < a.M ? m : 0;
-    __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(a.res_stats + 2 * (long)m),
-                                     (__attribute__((address_space(3))) void*)(smem + Cfg::STATS_OFF + wave * (2 * Cfg::WM * 4)), 16, 0, 0);
-  }
 
   // Loader role: waves 0-3 fill weight rows [64w, +64) of a stage, waves 4-7 activation rows [64(w-4), +64): 8 rows per
   // wave-instruction, eight 16-byte chunks per row, the swizzle applied on the global side (row 8 i + lane / 8 of the
@@ -121,6 +115,36 @@ __global__ void __launch_bounds__(DmafCfg::NT, 2) gemm_dmaf_kernel(const GemmArg
     __builtin_amdgcn_raw_ptr_buffer_load_lds(r, (__attribute__((address_space(3))) void*)(smem + (lds_load0 ^ ((slab & 1) << 15)) + i * 1024), 16,
                                              (int)voff[i], slab * Cfg::ROWB, 0, 0);
   };
+  // The first slab is requested as early as its addresses exist; everything else the prologue sets up follows.
+  static_for<0, LOADS>([&](auto ic) { issue_one(0, rsrc_mine, ic); });
+  __builtin_amdgcn_sched_barrier(0);
+
+  // The per-column constants of the epilogue (bias; gain and offset of a residual normalised on the fly) for this wave's
+  // 64 columns, one column per lane, landed outside the ring: requested first, in LDS long before the epilogue asks.
+  // Columns past N repeat the last one; nothing of theirs is stored.
+  {
+    int n = n0 + wn * Cfg::WN + lane;
+    n = n < a.N ? n : a.N - 1;
+    uint8_t* cols = smem + Cfg::COLS_OFF + wave * (3 * Cfg::WN * 4);
+    if (a.bias)
+      __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(a.bias + n), (__attribute__((address_space(3))) void*)cols, 4, 0, 0);
+    if constexpr (RES_NORM != 0) {
+      __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(a.res_gamma + n),
+                                       (__attribute__((address_space(3))) void*)(cols + Cfg::WN * 4), 4, 0, 0);
+      if (a.res_beta)
+        __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(a.res_beta + n),
+                                         (__attribute__((address_space(3))) void*)(cols + 2 * Cfg::WN * 4), 4, 0, 0);
+    }
+  }
+  if constexpr (RES_NORM != 0) {
+    // Statistics of this wave's 128 rows (two rows = 16 bytes per lane), requested before anything else and landed
+    // outside the ring.
+    int m = m0 + wm * Cfg::WM + 2 * lane;
+    m = m + 1 < a.M ? m : 0;
+    __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(a.res_stats + 2 * (long)m),
+                                     (__attribute__((address_space(3))) void*)(smem + Cfg::STATS_OFF + wave * (2 * Cfg::WM * 4)), 16, 0, 0);
+  }
+
 
   // L2 touches, as in gemm_dma_kernel.hpp: wave 0 touches its share of the activation lines of a slab `pf` slabs before
   // anybody loads it, wave 1 its share of the weight lines; one dword per 128-byte line into an LDS strip nobody reads.
@@ -128,7 +152,7 @@ __global__ void __launch_bounds__(DmafCfg::NT, 2) gemm_dmaf_kernel(const GemmArg
   int pf_n = 0, pf_step = 0;
   if (pf > 0 && wave < 2) {
     if (wave == 0) {
-      pf_n = (4 + grp_w - 1) / grp_w;
+      pf_n = grp_w >= 4 ? 1 : grp_w >= 2 ? 2 : 4;   // ceil(4 / grp_w)
       int r = ((grp_q * pf_n) & 3) * 64 + lane;
       r = r < a.M - m0 ? r : a.M - m0 - 1;
       pf_off = (uint32_t)r * (uint32_t)(a.lda * ESZ);
@@ -181,7 +205,6 @@ __global__ void __launch_bounds__(DmafCfg::NT, 2) gemm_dmaf_kernel(const GemmArg
   const bool wave_active = (m0 + wm * Cfg::WM < a.M) && (n0 + wn * Cfg::WN < a.N);
 
 
-  static_for<0, LOADS>([&](auto ic) { issue_one(0, rsrc_mine, ic); });
   for (int s0 = 1; s0 < 1 + pf; ++s0) prefetch(s0);
 
   for (int slab = 0; slab < nslab; ++slab) {
@@ -254,7 +277,8 @@ static hipError_t launch_dmaf(const GemmArgs& a, hipStream_t st) {
   const int tiles = ((a.M + DmafCfg::BM - 1) / DmafCfg::BM) * tiles_n;
   // (the L2 touches pay for e4m3 operands only: the 16-bit instances lose 2-6 % with them)
   const int pf = (IN_DT == DT_FP8 && tiles_n % 4 == 0 && (long)a.K >= 8 * DmafCfg::ROWB) ? 2 : 0;
-  hipLaunchKernelGGL(kern, dim3(tiles), dim3(DmafCfg::NT), DmafCfg::LDS_BYTES, st, a, pf);
+  if (tiles >= 65536) return hipErrorInvalidValue;   // (the walk's divisions are exact below that; the caller has another kernel)
+  hipLaunchKernelGGL(kern, dim3(tiles), dim3(DmafCfg::NT), DmafCfg::LDS_BYTES, st, a, pf, dmaf_walk(a.M, a.N, IN_DT == DT_FP8));
   return hipGetLastError();
 }
 
