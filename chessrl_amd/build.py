@@ -22,6 +22,7 @@ SOURCES = [
     "kernels/gemm_sp.hip",
     "kernels/gemm_sp2.hip",
     "kernels/gemm_dmaf.hip",
+    "kernels/gemm_dmam.hip",
     "kernels/norm_embed.hip",
     "kernels/attention.hip",
     "kernels/heads.hip",

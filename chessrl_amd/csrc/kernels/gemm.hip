@@ -394,6 +394,19 @@ typedef GemmCfg<128, 128, 2, 2, 2, 0, 2> CfgMid;    // 4 waves, 64x64 per wave, 
 typedef GemmCfg<64, 64, 2, 2, 2, 0, 2> CfgSmall;    // 4 waves, 32x32 per wave
 typedef GemmCfg<64, 64, 2, 2, 2, 0, 2, 4> CfgSmallK4;   // the same tile walked by 4 groups of 4 waves, K slabs in turn
 
+// Compute units of the current device (0 if the query fails: callers then take their conservative branch).
+static int device_cus() {
+  static std::atomic<int> cus[16] = {};
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 16) return 0;
+  int n = cus[dev];
+  if (n == 0) {
+    if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess) return 0;
+    cus[dev] = n;
+  }
+  return n;
+}
+
 template <typename Cfg, int IN_DT, int OUT_DT, int RES_NORM = 0>
 static hipError_t launch_cfg(const GemmArgs& a, hipStream_t st) {
   if constexpr (!RES_NORM) {
@@ -557,7 +570,7 @@ static hipError_t launch_splitk(const GemmArgs& a, int ks, int per, hipStream_t 
 template <int IN_DT, int OUT_DT>
 static hipError_t launch_in_out(const GemmArgs& a, int tile, hipStream_t st) {
   if (a.ln_out && !gemm_folds_layernorm(a, IN_DT)) return hipErrorInvalidValue;   // only the K-sliced path has a whole row in one place
-  if (a.res_stats && (a.k_parallel || (tile >= 4 && tile != 7 && tile != 9 && tile != 10))) return hipErrorInvalidValue;   // the tiled kernels only
+  if (a.res_stats && (a.k_parallel || (tile >= 4 && tile != 7 && tile != 9 && tile != 10 && tile != 12))) return hipErrorInvalidValue;   // the tiled kernels only
   if ((tile == 0 && a.k_parallel) || tile == 4) {
     int per = 0;
     const int ks = splitk_plan(a, IN_DT == DT_FP8 ? 1 : 2, tile == 4, &per);
@@ -611,7 +624,19 @@ static hipError_t launch_in_out(const GemmArgs& a, int tile, hipStream_t st) {
   }
   if (tile == 10) return gemm_dmaf_has(IN_DT, OUT_DT, a.res_stats != nullptr) ? launch_gemm_dmaf(a, IN_DT, OUT_DT, st) : hipErrorInvalidValue;
   if (tile == 3 || tile == 7) return launch_gemm_dma(a, IN_DT, OUT_DT, st);
-  if (tile == 2) return launch_cfg<CfgMid, IN_DT, OUT_DT>(a, st);
+  // The 128x128 tile has the register-staged kernel (any K, fp32 outputs, normalised residuals; two workgroups per CU;
+  // tile 12 names it) and, for K in whole slabs, the direct-to-LDS kernel with three slabs in flight
+  // (gemm_dmam_kernel.hpp, tile 11; bit-equal; one workgroup per CU). The second is 10 % faster while every tile has a
+  // CU of its own (M=4096, N=1024: 19.1 -> 17.1 us at K=1024, 25.5 -> 22.8 at K=1536) and slower beyond (384 tiles: 25.9
+  // -> 29.8 us), so tile 2 picks it for at most as many tiles as there are CUs.
+  if (tile == 11 && !slabs) tile = 12;
+  if (tile == 2 || tile == 11) {
+    const long mid_tiles = (long)((a.M + 127) / 128) * ((a.N + 127) / 128);
+    const bool can = slabs && !a.res_stats && gemm_dmam_has(IN_DT, OUT_DT) && mid_tiles < 65536;
+    if (can && (tile == 11 || mid_tiles <= device_cus())) return launch_gemm_dmam(a, IN_DT, OUT_DT, st);
+    if (tile == 11) return hipErrorInvalidValue;
+  }
+  if (tile == 2 || tile == 12) return launch_cfg<CfgMid, IN_DT, OUT_DT>(a, st);
   if (tile == 5) return launch_cfg<CfgSmallK4, IN_DT, OUT_DT>(a, st);
   return launch_cfg<CfgSmall, IN_DT, OUT_DT>(a, st);
 }

@@ -1,0 +1,26 @@
+// Instances of the 128x128 GEMM fed by direct-to-LDS loads through a four-stage ring (gemm_dmam_kernel.hpp), in a
+// translation unit of their own.
+#include "gemm_dmam_kernel.hpp"
+
+namespace crl {
+
+// false: no instance for this combination (the caller keeps the register-staged kernel).
+bool gemm_dmam_has(int in_dt, int out_dt) {
+  if (in_dt == DT_FP8) return out_dt == DT_BF16 || out_dt == DT_F16 || out_dt == DT_FP8;
+  return in_dt == out_dt && (in_dt == DT_BF16 || in_dt == DT_F16);
+}
+
+hipError_t launch_gemm_dmam(const GemmArgs& a, int in_dt, int out_dt, hipStream_t st) {
+  if (in_dt == DT_FP8) {
+    switch (out_dt) {
+      case DT_BF16: return launch_dmam<DT_FP8, DT_BF16>(a, st);
+      case DT_F16: return launch_dmam<DT_FP8, DT_F16>(a, st);
+      case DT_FP8: return launch_dmam<DT_FP8, DT_FP8>(a, st);
+    }
+  }
+  if (in_dt == DT_BF16 && out_dt == DT_BF16) return launch_dmam<DT_BF16, DT_BF16>(a, st);
+  if (in_dt == DT_F16 && out_dt == DT_F16) return launch_dmam<DT_F16, DT_F16>(a, st);
+  return hipErrorInvalidValue;
+}
+
+}  // namespace crl

@@ -406,6 +406,9 @@ hipError_t launch_gemm_sp(const GemmArgs& a, int out_dt, hipStream_t st);
 // gemm_dmaf.hip: the eight-wave in-step tile with address arithmetic kept out of the main loop (K in whole 128-byte slabs).
 bool gemm_dmaf_has(int in_dt, int out_dt, bool res_norm);
 hipError_t launch_gemm_dmaf(const GemmArgs& a, int in_dt, int out_dt, hipStream_t st);
+// gemm_dmam.hip: the 128x128 tile fed by direct-to-LDS loads through a four-stage ring (K in whole 128-byte slabs, no normalised residual).
+bool gemm_dmam_has(int in_dt, int out_dt);
+hipError_t launch_gemm_dmam(const GemmArgs& a, int in_dt, int out_dt, hipStream_t st);
 // gemm_sp2.hip: the same four waves fed in 128-byte slabs of K.
 hipError_t launch_gemm_sp2(const GemmArgs& a, int out_dt, hipStream_t st);
 

@@ -115,7 +115,9 @@ int crl_random_positions(uint64_t seed, int n, int max_plies, double late_fracti
  * software-pipelined waves with 16x16x128 MFMAs (e4m3 operands, whole slabs; what 3 runs from K = 4096 on; these MFMAs
  * add 128 products per instruction instead of 64, so a sum can differ from the others' in its last fp32 bits); 6 = the
  * two waves of a SIMD out of step and 8 = four software-pipelined waves fed in 64-byte pieces (e4m3 operands, bit-equal
- * to 7) exist for measurement and are slower. 9 and 10 fall back to 7 where K is not whole slabs. */
+ * to 7) exist for measurement and are slower. 9 and 10 fall back to 7 where K is not whole slabs. 11 and 12 name the two
+ * 128x128 kernels (same sums and bits as 2): 11 = fed by direct-to-LDS loads through a four-stage ring (whole slabs; what 2
+ * runs for at most one tile per CU), 12 = register-staged (any K; 11 hands over to it where K is not whole slabs). */
 int crl_gemm(const void* A, int64_t lda, const void* W, int64_t ldw, void* C, int64_t ldc,
              int M, int N, int K, int in_dtype, int out_dtype,
              const float* bias, int act, float descale, float alpha,

@@ -230,6 +230,40 @@ def test_gemm_fp8_out_of_step_kernel_equals_in_step_kernel(cuda, M, N, K, alt):
     assert torch.allclose(out.float(), ref, rtol=2 ** -7, atol=2 ** -7 * ref.abs().max().item()), (out.float() - ref).abs().max()
 
 
+@pytest.mark.parametrize("M,N,K", [(128, 128, 64), (128, 128, 256), (4096, 1024, 1024), (4096, 1536, 1024), (4096, 1024, 1536), (2048, 4096, 256),
+                                   (300, 700, 512), (1000, 3104, 1024), (4096, 200, 192), (130, 129, 128), (640, 3104, 1088)])
+@pytest.mark.parametrize("dt", ["bf16", "fp8"])
+def test_gemm_mid_tile_direct_to_lds_equals_register_staged(cuda, M, N, K, dt):
+    """The 128x128 tile fed by direct-to-LDS loads through a four-stage ring (tile 11, what the library picks for a few
+    hundred such tiles when K is whole 128-byte slabs) against the register-staged kernel on the same tile (tile 12): same
+    sums, bit-equal outputs; with bias, activation, residual and a scaled e4m3 output. 1 to 12 slabs (fewer slabs than ring
+    stages included), ragged M and N, K that is not whole slabs (where 11 hands over to 12)."""
+    torch.manual_seed(M + N + K)
+    if dt == "fp8":
+        A = (torch.randn(M, K, device=cuda) * 30).to(torch.float8_e4m3fn)
+        W = (torch.randn(N, K, device=cuda) * 30).to(torch.float8_e4m3fn)
+        descale = 1e-3
+    else:
+        A = torch.randn(M, K, device=cuda).bfloat16()
+        W = (torch.randn(N, K, device=cuda) / K ** 0.5).bfloat16()
+        descale = 1.0
+    bias = torch.randn(N, device=cuda)
+    ldc = (N + 7) // 8 * 8
+    res = torch.randn(M, ldc, device=cuda).bfloat16()
+    cases = [dict(out_dt=_lib.BF16, bias=bias, act=2, descale=descale, alpha=0.43, res=res), dict(out_dt=_lib.BF16, descale=descale)]
+    if dt == "fp8":
+        cases.append(dict(out_dt=_lib.FP8, bias=bias, act=2, descale=descale, out_scale=7.0))
+    for kw in cases:
+        a11, a12 = torch.zeros(1, device=cuda), torch.zeros(1, device=cuda)
+        o11 = run_gemm(A, W, kw["out_dt"], tile=11, ldc=ldc, amax=a11, **{k: v for k, v in kw.items() if k != "out_dt"})
+        o12 = run_gemm(A, W, kw["out_dt"], tile=12, ldc=ldc, amax=a12, **{k: v for k, v in kw.items() if k != "out_dt"})
+        assert torch.equal(o11, o12), (M, N, K, dt, kw["out_dt"], (o11.float() - o12.float()).abs().max().item())
+        assert torch.equal(a11, a12)
+    ref = (A.float() @ W.float().t()) * descale
+    out = run_gemm(A, W, _lib.BF16, descale=descale, tile=11, ldc=ldc)
+    assert torch.allclose(out.float(), ref, rtol=2 ** -7, atol=2 ** -7 * ref.abs().max().item()), (out.float() - ref).abs().max()
+
+
 @pytest.mark.parametrize("C_,in_dt", [(256, _lib.F32), (1024, _lib.BF16), (512, _lib.BF16), (8192, _lib.BF16), (768, _lib.F32), (1536, _lib.F32)])
 def test_layernorm(cuda, C_, in_dt):
     torch.manual_seed(C_)
