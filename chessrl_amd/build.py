@@ -23,6 +23,7 @@ SOURCES = [
     "kernels/gemm_sp2.hip",
     "kernels/gemm_dmaf.hip",
     "kernels/gemm_dmam.hip",
+    "kernels/gemm_shortk.hip",
     "kernels/norm_embed.hip",
     "kernels/attention.hip",
     "kernels/heads.hip",

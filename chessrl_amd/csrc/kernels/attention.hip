@@ -97,14 +97,23 @@ __global__ void __launch_bounds__(64 * AttnWaves<MODE>::N, (AttnMinWaves<HS, MOD
   // transposed and the scores are formed.
   uint4 braw[2][2][2];
   if constexpr (MODE == ATTN_BIAS) {
-    const uint16_t* bp = reinterpret_cast<const uint16_t*>(a.bias) + (long)unit * 4096;
+    // Element k = 512 L + 8 lane + e of the unit's 4096 (L = (it, jt, rh)): row-major, or in blocks of 256 units x 128
+    // elements (the layout the bias generator's GEMM writes fastest), where a load of 1 KB is four pieces of 256 bytes.
+    const uint16_t* bp = reinterpret_cast<const uint16_t*>(a.bias);
+    long lstride = 512;
+    if (a.bias_blocked) {
+      bp += (long)(unit >> 8) * (256 * 4096) + ((long)(lane >> 4) * 256 + (unit & 255)) * 128 + ((lane & 15) << 3);
+      lstride = 4 * 256 * 128;
+    } else {
+      bp += (long)unit * 4096 + (lane << 3);
+    }
 #pragma unroll
     for (int it = 0; it < 2; ++it)
 #pragma unroll
       for (int jt = 0; jt < 2; ++jt)
 #pragma unroll
         for (int rh = 0; rh < 2; ++rh)
-          braw[it][jt][rh] = *reinterpret_cast<const uint4*>(bp + ((((it * 2 + jt) * 2 + rh) * 64 + lane) << 3));
+          braw[it][jt][rh] = *reinterpret_cast<const uint4*>(bp + ((it * 2 + jt) * 2 + rh) * lstride);
   }
 
   // ---- V -> V^T in LDS ------------------------------------------------------------
@@ -598,6 +607,7 @@ hipError_t launch_attention(const AttnArgs& a, int head_dim, hipStream_t st) {
       (reinterpret_cast<uintptr_t>(a.q) & 15) || (reinterpret_cast<uintptr_t>(a.k) & 15) || (reinterpret_cast<uintptr_t>(a.v) & 15))
     return hipErrorInvalidValue;
   if (a.mode == ATTN_BIAS && !a.bias) return hipErrorInvalidValue;
+  if (a.mode == ATTN_BIAS && a.bias_blocked && ((long)a.B * a.H) % 256 != 0) return hipErrorInvalidValue;
   if (a.mode == ATTN_RELSHIFT && (!a.pos || !a.u_bias || !a.v_bias)) return hipErrorInvalidValue;
   if (a.T != 0 && a.T != 64) {
     if (a.mode != ATTN_CAUSAL || a.T < 1 || a.T > 4096) return hipErrorInvalidValue;

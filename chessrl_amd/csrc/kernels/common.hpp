@@ -137,6 +137,9 @@ struct GemmArgs {
   // res_stats [M,2] = (1/std, -mean/std) a LayerNorm launch left behind and that norm's gain and offset [N]
   // (256x256 tile with a 16-bit residual only; see gemm_takes_res_norm).
   const float* res_stats; const float* res_gamma; const float* res_beta;
+  // 1: C (ldc == N) is written in contiguous blocks of 256 rows x 128 columns, block (m / 256, n / 128) at index
+  // (m / 256) * (N / 128) + n / 128, instead of row-major (only where gemm_shortk_can says so).
+  int c_blocked;
 };
 
 struct LayerNormArgs {
@@ -191,6 +194,7 @@ struct AttnArgs {
   const void* q; const void* k; const void* v;  // bf16 or f16, [B*64, ld*] with head h at column h*HS
   long ldq, ldk, ldv;
   const void* bias;     // ATTN_BIAS: bf16 [B,H,4096] in the kernel's register order
+  int bias_blocked;     // 1: the [B*H, 4096] bias matrix is stored in blocks of 256 rows x 128 columns (GemmArgs::c_blocked); B*H % 256 == 0
   const void* pos;      // ATTN_RELSHIFT: bf16 [64, H*HS] projected positional table
   const float* u_bias;  // ATTN_RELSHIFT: [H*HS]
   const float* v_bias;  // ATTN_RELSHIFT: [H*HS]
@@ -274,6 +278,8 @@ hipError_t launch_gemm(GemmArgs a, int in_dt, int out_dt, int tile, hipStream_t 
 // True when launch_gemm (tile 0) would take the K-sliced path for these arguments, whose second pass can apply the
 // LayerNorm that follows the GEMM (GemmArgs::ln_*); launch_gemm rejects ln_out otherwise.
 bool gemm_folds_layernorm(const GemmArgs& a, int in_dt);
+// Whether the product can be written in the blocked layout of GemmArgs::c_blocked (gemm_shortk.hip has the one kernel that does).
+bool gemm_shortk_can(const GemmArgs& a, int in_dt, int out_dt);
 // crl_gemm's tile 4 with the slices' partial sums in a fixed array of the library's device image (no allocation).
 constexpr size_t STATIC_WS_BYTES = 8u << 20;
 hipError_t launch_gemm_static_ws(GemmArgs a, int in_dt, int out_dt, hipStream_t st, bool* too_big, size_t* need_bytes);

@@ -571,6 +571,11 @@ template <int IN_DT, int OUT_DT>
 static hipError_t launch_in_out(const GemmArgs& a, int tile, hipStream_t st) {
   if (a.ln_out && !gemm_folds_layernorm(a, IN_DT)) return hipErrorInvalidValue;   // only the K-sliced path has a whole row in one place
   if (a.res_stats && (a.k_parallel || (tile >= 4 && tile != 7 && tile != 9 && tile != 10 && tile != 12))) return hipErrorInvalidValue;   // the tiled kernels only
+  // K = 256 e4m3 elements into a large 16-bit output (the attention-bias generator): the kernel whose workgroups keep
+  // their rows of A and walk N (gemm_shortk_kernel.hpp; tile 13). It is the only one that writes the blocked layout, and
+  // that is what it is for: M = 131072, N = 4096 takes 280 us through the 256x256 tile, 310 us here row-major and 191 us
+  // here in blocks, so nothing picks it for a row-major output unasked.
+  if (a.c_blocked || tile == 13) return launch_gemm_shortk(a, IN_DT, OUT_DT, st);
   if ((tile == 0 && a.k_parallel) || tile == 4) {
     int per = 0;
     const int ks = splitk_plan(a, IN_DT == DT_FP8 ? 1 : 2, tile == 4, &per);
@@ -675,6 +680,7 @@ hipError_t launch_gemm(GemmArgs a, int in_dt, int out_dt, int tile, hipStream_t 
   // An output beyond the 32 MB of L2 (8 XCDs x 4 MB) cannot be kept for the consumer anyway: stream it past the
   // caches so it does not push the operand tiles out (measured +6..10 % on the 0.5-1.6 GB outputs of a 4096-position batch).
   a.stream_out = (long)a.M * a.N * dtype_size(out_dt) > (64L << 20) ? 1 : 0;
+  if (tile == 14) { a.c_blocked = 1; tile = 13; }
   switch (in_dt) {
     case DT_BF16: return launch_in<DT_BF16>(a, out_dt, tile, st);
     case DT_F16: return launch_in<DT_F16>(a, out_dt, tile, st);

@@ -416,6 +416,8 @@ struct GOpt {
   const float* ln_g = nullptr; const float* ln_b = nullptr; void* ln_out = nullptr; int ln_dt = DT_BF16; bool* ln_folded = nullptr;
   // The residual is LayerNorm(res), normalised in the epilogue from these row statistics, gain and offset.
   const float* res_stats = nullptr; const float* res_g = nullptr; const float* res_b = nullptr;
+  // Ask for the blocked output layout (GemmArgs::c_blocked) where the GEMM has a kernel for it; *c_blocked says whether it was used.
+  bool* c_blocked = nullptr;
 };
 
 int Model::gemm(const Lin& L, const void* A, long lda, int in_dt, void* C, long ldc, int out_dt, int M, const GOpt& o, hipStream_t st) {
@@ -438,6 +440,11 @@ int Model::gemm(const Lin& L, const void* A, long lda, int in_dt, void* C, long 
     const bool fold = !profiling && gemm_folds_layernorm(g, in_dt == DT_FP8 ? DT_FP8 : L.dt);
     if (o.ln_folded) *o.ln_folded = fold;
     if (!fold) { g.ln_gamma = g.ln_beta = nullptr; g.ln_out = nullptr; }
+  }
+  if (o.c_blocked) {
+    g.c_blocked = 1;
+    if (!gemm_shortk_can(g, in_dt == DT_FP8 ? DT_FP8 : L.dt, out_dt)) g.c_blocked = 0;
+    *o.c_blocked = g.c_blocked != 0;
   }
   const int fam = in_dt == DT_FP8 ? 0 : 5;
   if (profiling) prof_flops[fam] += 2.0 * M * (double)L.N * L.K;
@@ -573,6 +580,7 @@ int Model::forward_chunk(const float* planes, const uint8_t* ids, const uint8_t*
     }
     if (kv_capture) HIPCHK(launch_kv_store(ws.qkv, kv_layers[l], mb, T, kv_Tmax, C, st));
     const void* bias_tile = nullptr;
+    bool bias_blocked = false;
     if (cfg.arch == CRL_ARCH_BT4CLASS) {
       const int sc = cfg.smolgen_compress, sh = cfg.smolgen_hidden, sg = cfg.smolgen_gen;
       GOpt o; o.act = ACT_SWISH;
@@ -583,7 +591,9 @@ int Model::forward_chunk(const float* planes, const uint8_t* ids, const uint8_t*
       // configuration it takes e4m3 inputs like the trunk linears; the two small layers before it stay 16-bit.
       RUN(lnorm(ws.sg1, H * sg, ad, ly.sm_ln2_g, ly.sm_ln2_b, f8 ? nullptr : ws.sg2, ad, f8 ? ws.sg2_8 : nullptr, f8 ? act_scale(l, 4) : 1.f,
                 H * sg, mb, H * sg, am(l, 4), st, nullptr, nullptr, DT_BF16, false));
-      GOpt o2; o2.a_scale = f8 ? act_scale(l, 4) : 1.f;
+      // (with e4m3 inputs and whole blocks of 256 (position, head) rows the product is written in the blocked layout,
+      // which the attention kernel reads as it stands)
+      GOpt o2; o2.a_scale = f8 ? act_scale(l, 4) : 1.f; o2.c_blocked = &bias_blocked;
       RUN(gemm(sm_weight_gen, f8 ? (const void*)ws.sg2_8 : (const void*)ws.sg2, sg, f8 ? DT_FP8 : ad, ws.bias, 4096, ad, mb * H, o2, st));
       bias_tile = ws.bias;
     }
@@ -593,7 +603,7 @@ int Model::forward_chunk(const float* planes, const uint8_t* ids, const uint8_t*
       std::memset(&a, 0, sizeof(a));
       const uint16_t* base = reinterpret_cast<const uint16_t*>(ws.qkv);
       a.q = base; a.k = base + C; a.v = base + 2 * C; a.ldq = a.ldk = a.ldv = 3 * C;
-      a.bias = bias_tile; a.pos = ly.pos; a.u_bias = ly.u_bias; a.v_bias = ly.v_bias;
+      a.bias = bias_tile; a.bias_blocked = bias_blocked ? 1 : 0; a.pos = ly.pos; a.u_bias = ly.u_bias; a.v_bias = ly.v_bias;
       a.out = f8 ? (void*)ws.ao8 : (void*)ws.ao; a.ldo = C; a.out_dtype = f8 ? DT_FP8 : ad;
       a.out_scale = f8 ? act_scale(l, 1) : 1.f; a.amax = am(l, 1);
       a.B = mb; a.H = H; a.scale = attn_scale; a.in_dtype = ad; a.T = T;

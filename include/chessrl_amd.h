@@ -117,7 +117,12 @@ int crl_random_positions(uint64_t seed, int n, int max_plies, double late_fracti
  * two waves of a SIMD out of step and 8 = four software-pipelined waves fed in 64-byte pieces (e4m3 operands, bit-equal
  * to 7) exist for measurement and are slower. 9 and 10 fall back to 7 where K is not whole slabs. 11 and 12 name the two
  * 128x128 kernels (same sums and bits as 2): 11 = fed by direct-to-LDS loads through a four-stage ring (whole slabs; what 2
- * runs for at most one tile per CU), 12 = register-staged (any K; 11 hands over to it where K is not whole slabs). */
+ * runs for at most one tile per CU), 12 = register-staged (any K; 11 hands over to it where K is not whole slabs).
+ * 13 and 14 name the kernel for K = 256 e4m3 elements whose workgroups keep 256 rows of A in registers and walk N (the
+ * attention-bias generator's product): a bare scaled product (no bias, activation, residual or amax; alpha = 1) into a
+ * bf16/f16 output of more than 64 MB, M a multiple of 256, N of 128; anything else is CRL_ERR_ARG. 13 writes C row-major
+ * (same result bits as 3); 14 writes it (ldc == N) in contiguous blocks of 256 rows x 128 columns, element (m, n) at
+ * ((m / 256) * (N / 128) + n / 128) * 32768 + (m % 256) * 128 + n % 128, which is 1.6 times faster and what the model uses. */
 int crl_gemm(const void* A, int64_t lda, const void* W, int64_t ldw, void* C, int64_t ldc,
              int M, int N, int K, int in_dtype, int out_dtype,
              const float* bias, int act, float descale, float alpha,

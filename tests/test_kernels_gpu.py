@@ -264,6 +264,47 @@ def test_gemm_mid_tile_direct_to_lds_equals_register_staged(cuda, M, N, K, dt):
     assert torch.allclose(out.float(), ref, rtol=2 ** -7, atol=2 ** -7 * ref.abs().max().item()), (out.float() - ref).abs().max()
 
 
+@pytest.mark.parametrize("M,N,out_dt", [(8448, 4096, _lib.BF16), (16384, 4096, _lib.F16), (131328, 384, _lib.BF16), (131072, 4096, _lib.BF16)])
+def test_gemm_short_k_rows_resident_equals_tiled(cuda, M, N, out_dt):
+    """K = 256 e4m3 elements into a large 16-bit output (the attention-bias generator's product): the kernel whose
+    workgroups keep 256 rows of A in registers and walk N (tile 13; tile 14 = the same with C stored in contiguous blocks
+    of 256 rows x 128 columns, the layout the model hands to the attention kernel) against the 256x256 tile (tile 10).
+    Same sums and the same rounding: bit-equal outputs, the blocked one after undoing its layout; the last case is the
+    headline batch's own size (4096 positions x 32 heads), where every CU streams its stores at full rate."""
+    torch.manual_seed(M + N)
+    A = (torch.randn(M, 256, device=cuda) * 2).to(torch.float8_e4m3fn)
+    W = (torch.randn(N, 256, device=cuda) * 2).to(torch.float8_e4m3fn)
+    ref = run_gemm(A, W, out_dt, descale=0.013, tile=10)
+    rows = run_gemm(A, W, out_dt, descale=0.013, tile=13)
+    assert torch.equal(ref, rows), (ref.float() - rows.float()).abs().max().item()
+    blocks = run_gemm(A, W, out_dt, descale=0.013, tile=14)
+    blocks = blocks.reshape(M // 256, N // 128, 256, 128).permute(0, 2, 1, 3).reshape(M, N)
+    assert torch.equal(ref, blocks), (ref.float() - blocks.float()).abs().max().item()
+    sample = slice(0, 512)
+    exact = (A[sample].float() @ W.float().t()) * 0.013
+    assert torch.allclose(rows[sample].float(), exact, rtol=2 ** -7, atol=2 ** -7 * exact.abs().max().item())
+
+
+def test_gemm_short_k_rows_resident_rejects_what_it_cannot_do(cuda):
+    """Tile 13 is a bare scaled product for K = 256, whole blocks of 256 rows and outputs beyond 64 MB: anything else
+    is refused (CRL_ERR_ARG), never computed by another kernel behind the caller's back."""
+    A = torch.zeros(8448, 256, device=cuda).to(torch.float8_e4m3fn)
+    W = torch.zeros(4096, 256, device=cuda).to(torch.float8_e4m3fn)
+    out = torch.zeros(8448, 4096, dtype=torch.bfloat16, device=cuda)
+    bias = torch.zeros(4096, device=cuda)
+    def call(M, N, K, bias_t=None, act=0, tile=13):
+        return lib().crl_gemm(p(A), 256, p(W), 256, p(out), N, M, N, K, _lib.FP8, _lib.BF16, p(bias_t), act, 1.0, 1.0, p(None), 0, _lib.BF16,
+                              1.0, p(None), tile, stream())
+    assert call(8448, 4096, 256) == 0
+    assert call(8448, 4096, 128) != 0          # K
+    assert call(8400, 4096, 256) != 0          # M not in whole blocks
+    assert call(4096, 4096, 256) != 0          # output small enough for the caches
+    assert call(8448, 4096, 256, bias_t=bias) != 0
+    assert call(8448, 4096, 256, act=2) != 0
+    assert call(8448, 4000, 256, tile=14) != 0  # N not in whole steps of 128 columns
+    torch.cuda.synchronize()
+
+
 @pytest.mark.parametrize("C_,in_dt", [(256, _lib.F32), (1024, _lib.BF16), (512, _lib.BF16), (8192, _lib.BF16), (768, _lib.F32), (1536, _lib.F32)])
 def test_layernorm(cuda, C_, in_dt):
     torch.manual_seed(C_)
