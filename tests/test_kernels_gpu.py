@@ -337,16 +337,17 @@ def split_heads(qkv, B, H, hs):
     return [t.view(B, 64, H, hs).transpose(1, 2) for t in (q, k, v)]
 
 
-def run_attn(qkv, B, H, hs, mode, scale, bias=None, pos=None, u=None, v=None, out_dt=None, out_scale=1.0):
+def run_attn(qkv, B, H, hs, mode, scale, bias=None, pos=None, u=None, v=None, out_dt=None, out_scale=1.0, ldo=None):
     Cm = H * hs
     in_dt = _lib.F16 if qkv.dtype == torch.float16 else _lib.BF16
     out_dt = in_dt if out_dt is None else out_dt
-    out = torch.zeros(B * 64, Cm, dtype=qkv.dtype if out_dt != _lib.FP8 else torch.uint8, device=qkv.device)
+    ldo = ldo or Cm
+    out = torch.zeros(B * 64, ldo, dtype=qkv.dtype if out_dt != _lib.FP8 else torch.uint8, device=qkv.device)
     base = qkv.data_ptr()
     check(lib().crl_attention(C.c_void_p(base), 3 * Cm, C.c_void_p(base + 2 * Cm), 3 * Cm, C.c_void_p(base + 4 * Cm), 3 * Cm, in_dt,
-                              p(out), Cm, out_dt, out_scale, B, H, hs, mode, scale, p(bias), p(pos), p(u), p(v), None, stream()), "attn")
+                              p(out), ldo, out_dt, out_scale, B, H, hs, mode, scale, p(bias), p(pos), p(u), p(v), None, stream()), "attn")
     torch.cuda.synchronize()
-    return out
+    return out[:, :Cm]
 
 
 @pytest.mark.parametrize("H,hs", [(8, 32), (12, 64), (32, 32)])
@@ -382,6 +383,25 @@ def test_attention_bias(cuda):
     o8 = run_attn(qkv, B, H, hs, _lib.ATTN_BIAS, 1 / math.sqrt(hs), bias=packed, out_dt=_lib.FP8, out_scale=so)
     deq = o8.view(torch.float8_e4m3fn).float() / so
     assert (deq - ref).abs().max() <= ref.abs().max() * 2 ** -3
+
+
+@pytest.mark.parametrize("mode", [_lib.ATTN_PLAIN, _lib.ATTN_CAUSAL, _lib.ATTN_BIAS])
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+def test_attention_whole_line_stores_equal_per_wave_stores(cuda, mode, dtype):
+    """At head size 32 with the heads in fours, a workgroup gathers its four heads' outputs in LDS and stores whole row
+    segments; otherwise (here: an output row stride that is not a multiple of 16 bytes) every wave stores its own 32- or
+    64-byte row pieces. Same values either way, bit for bit, in the 16-bit and the e4m3 output; B = 37 leaves nothing
+    to chance in the workgroup count."""
+    B, H, hs = 37, 32, 32
+    qkv, Cm = make_qkv(B, H, hs, cuda, 5 + mode, dtype)
+    bias = None
+    if mode == _lib.ATTN_BIAS:
+        bias = torch.randn(B, H, 4096, device=cuda).to(dtype)
+    for out_dt, pad in ((None, 4), (_lib.FP8, 8)):
+        whole = run_attn(qkv, B, H, hs, mode, 1 / math.sqrt(hs), bias=bias, out_dt=out_dt, out_scale=37.0)
+        pieces = run_attn(qkv, B, H, hs, mode, 1 / math.sqrt(hs), bias=bias, out_dt=out_dt, out_scale=37.0, ldo=Cm + pad)
+        assert torch.equal(whole, pieces), (mode, dtype, out_dt)
+        assert whole.float().abs().max() > 0
 
 
 def test_attention_relshift(cuda):
