@@ -89,14 +89,32 @@ __device__ __forceinline__ float apply_act(float x, int act) {
 }
 
 // ---- wave reductions (64 lanes) ---------------------------------------------------
+// An xor butterfly over lane distances 1, 2, 4, 8, 16, 32. The four short distances are data-parallel-primitive moves
+// inside a row of 16 lanes (no trip through the LDS crossbar, which is what __shfl_xor compiles to: six dependent ones per
+// reduction were most of a LayerNorm wave's latency). At distance 4 and 8 the partner is the mirrored lane of the half row
+// or row: after the shorter steps every lane of a group of 4 or 8 holds the group's partial result, so the mirrored lane
+// holds exactly what the xor partner holds.
+template <int CTRL>
+__device__ __forceinline__ float dpp_move(float v) {
+  return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), CTRL, 0xF, 0xF, false));
+}
+constexpr int DPP_XOR1 = 0xB1, DPP_XOR2 = 0x4E, DPP_HALF_MIRROR = 0x141, DPP_MIRROR = 0x140;
 __device__ __forceinline__ float wave_sum(float v) {
-#pragma unroll
-  for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, 64);
+  v += dpp_move<DPP_XOR1>(v);
+  v += dpp_move<DPP_XOR2>(v);
+  v += dpp_move<DPP_HALF_MIRROR>(v);
+  v += dpp_move<DPP_MIRROR>(v);
+  v += __shfl_xor(v, 16, 64);
+  v += __shfl_xor(v, 32, 64);
   return v;
 }
 __device__ __forceinline__ float wave_max(float v) {
-#pragma unroll
-  for (int o = 32; o > 0; o >>= 1) v = fmaxf(v, __shfl_xor(v, o, 64));
+  v = fmaxf(v, dpp_move<DPP_XOR1>(v));
+  v = fmaxf(v, dpp_move<DPP_XOR2>(v));
+  v = fmaxf(v, dpp_move<DPP_HALF_MIRROR>(v));
+  v = fmaxf(v, dpp_move<DPP_MIRROR>(v));
+  v = fmaxf(v, __shfl_xor(v, 16, 64));
+  v = fmaxf(v, __shfl_xor(v, 32, 64));
   return v;
 }
 

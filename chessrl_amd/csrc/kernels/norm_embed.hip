@@ -63,13 +63,14 @@ __device__ __forceinline__ void store8_fp8(uint8_t* base, long off, const float 
 
 // Normalise the VPL*8 values a lane holds (columns col0(i) = (i*64+lane)*8) and write them.
 // rms: RMSNorm (mean taken as zero, no offset): y = x * rsqrt(mean(x^2) + eps) * gamma.
-template <int VPL>
+// FULL: C == VPL * 512, every lane holds VPL whole vectors (no column guards in the instruction stream).
+template <int VPL, bool FULL = false>
 __device__ __forceinline__ void ln_finish(float (&x)[VPL][8], int lane, int C, const float* gamma, const float* beta,
                                            float eps, float (&y)[VPL][8], float* stats = nullptr, bool rms = false) {
   float s = 0.f;
 #pragma unroll
   for (int i = 0; i < VPL; ++i) {
-    if ((i * 64 + lane) * 8 < C) {
+    if (FULL || (i * 64 + lane) * 8 < C) {
 #pragma unroll
       for (int e = 0; e < 8; ++e) s += x[i][e];
     }
@@ -79,7 +80,7 @@ __device__ __forceinline__ void ln_finish(float (&x)[VPL][8], int lane, int C, c
   float q = 0.f;
 #pragma unroll
   for (int i = 0; i < VPL; ++i) {
-    if ((i * 64 + lane) * 8 < C) {
+    if (FULL || (i * 64 + lane) * 8 < C) {
 #pragma unroll
       for (int e = 0; e < 8; ++e) { const float d = x[i][e] - mean; q += d * d; }
     }
@@ -89,7 +90,7 @@ __device__ __forceinline__ void ln_finish(float (&x)[VPL][8], int lane, int C, c
 #pragma unroll
   for (int i = 0; i < VPL; ++i) {
     const int col = (i * 64 + lane) * 8;
-    if (col < C) {
+    if (FULL || col < C) {
       float gv[8], bv[8];
       load8<DT_F32>(gamma, col, gv);
       if (beta) load8<DT_F32>(beta, col, bv);
@@ -99,7 +100,7 @@ __device__ __forceinline__ void ln_finish(float (&x)[VPL][8], int lane, int C, c
   }
 }
 
-template <int IN_DT, int VPL>
+template <int IN_DT, int VPL, bool FULL = false>
 __global__ void __launch_bounds__(256) layernorm_kernel(const LayerNormArgs a) {
   const int lane = threadIdx.x & 63;
   const int row = blockIdx.x * 4 + (threadIdx.x >> 6);
@@ -108,14 +109,14 @@ __global__ void __launch_bounds__(256) layernorm_kernel(const LayerNormArgs a) {
 #pragma unroll
   for (int i = 0; i < VPL; ++i) {
     const int col = (i * 64 + lane) * 8;
-    if (col < a.C) load8<IN_DT>(a.x, (long)row * a.ldx + col, x[i]);
+    if (FULL || col < a.C) load8<IN_DT>(a.x, (long)row * a.ldx + col, x[i]);
   }
-  ln_finish<VPL>(x, lane, a.C, a.gamma, a.beta, a.eps, y, a.stats ? a.stats + 2 * (long)row : nullptr, a.rms != 0);
+  ln_finish<VPL, FULL>(x, lane, a.C, a.gamma, a.beta, a.eps, y, a.stats ? a.stats + 2 * (long)row : nullptr, a.rms != 0);
   float am = 0.f;
 #pragma unroll
   for (int i = 0; i < VPL; ++i) {
     const int col = (i * 64 + lane) * 8;
-    if (col < a.C) {
+    if (FULL || col < a.C) {
       if (a.out) store8(a.out, (long)row * a.ldo + col, y[i], a.out_dtype);
       if (a.out_b) store8(a.out_b, (long)row * a.ldo + col, y[i], a.out_b_dtype);
       if (a.out_fp8) store8_fp8(a.out_fp8, (long)row * a.ldo + col, y[i], a.fp8_scale);
@@ -200,6 +201,7 @@ static hipError_t launch_ln_dt(const LayerNormArgs& a, hipStream_t st) {
   const dim3 grid((a.rows + 3) / 4), block(256);
   const int vecs = (a.C / 8 + 63) / 64;
   if (vecs <= 1) hipLaunchKernelGGL((layernorm_kernel<IN_DT, 1>), grid, block, 0, st, a);
+  else if (a.C == 1024) hipLaunchKernelGGL((layernorm_kernel<IN_DT, 2, true>), grid, block, 0, st, a);   // (the trunk's width: no column guards)
   else if (vecs <= 2) hipLaunchKernelGGL((layernorm_kernel<IN_DT, 2>), grid, block, 0, st, a);
   else if (vecs <= 4) hipLaunchKernelGGL((layernorm_kernel<IN_DT, 4>), grid, block, 0, st, a);
   else if (vecs <= 16) hipLaunchKernelGGL((layernorm_wide_kernel<IN_DT>), dim3(a.rows), block, 0, st, a);
