@@ -50,7 +50,8 @@ inline DmafWalk dmaf_walk(int M, int N, bool fp8) {
   return w;
 }
 
-template <int IN_DT, int OUT_DT, int RES_NORM = 0>
+// LEAN: the epilogue without its edge and type guards (gemm_epilogue's LEAN; dmaf_lean_ok says when).
+template <int IN_DT, int OUT_DT, int RES_NORM = 0, bool LEAN = false>
 __global__ void __launch_bounds__(DmafCfg::NT, 2) gemm_dmaf_kernel(const GemmArgs a, const int pf, const DmafWalk wk) {
   typedef DmafCfg Cfg;
   constexpr int ESZ = IN_DT == DT_FP8 ? 1 : 2;                      // bytes per operand element
@@ -252,13 +253,18 @@ __global__ void __launch_bounds__(DmafCfg::NT, 2) gemm_dmaf_kernel(const GemmArg
   wait_vmcnt<0>();
   __syncthreads();  // every wave is done with the ring (and the empty loads past the end have retired) before it becomes epilogue scratch
 
-  gemm_epilogue<Cfg::WM, Cfg::WN, OUT_DT, RES_NORM>(a, acc, reinterpret_cast<float*>(smem) + wave * (32 * Cfg::WN),
+  gemm_epilogue<Cfg::WM, Cfg::WN, OUT_DT, RES_NORM, LEAN>(a, acc, reinterpret_cast<float*>(smem) + wave * (32 * Cfg::WN),
                                                      m0 + wm * Cfg::WM, n0 + wn * Cfg::WN, lane,
                                                      reinterpret_cast<float*>(smem + Cfg::STATS_OFF) + wave * (2 * Cfg::WM),
                                                      reinterpret_cast<const float*>(smem + Cfg::COLS_OFF) + wave * (3 * Cfg::WN));
 }
 
-template <int IN_DT, int OUT_DT, int RES_NORM = 0>
+inline bool dmaf_lean_ok(const GemmArgs& a) {
+  return a.M % DmafCfg::BM == 0 && a.vec_ok && a.N % 8 == 0 && a.nsplit % 8 == 0 && !a.amax && a.res_rows == 0 && !a.ln_out &&
+         (!a.res || a.res_dtype == DT_BF16);
+}
+
+template <int IN_DT, int OUT_DT, int RES_NORM = 0, bool LEAN = false>
 static hipError_t launch_dmaf(const GemmArgs& a, hipStream_t st) {
   static std::atomic<bool> attr_set[16] = {};
   hipError_t e = hipSuccess;
@@ -267,7 +273,7 @@ static hipError_t launch_dmaf(const GemmArgs& a, hipStream_t st) {
   if ((a.K * ESZ) % DmafCfg::ROWB != 0 || a.K <= 0 || (long)a.lda * ESZ * 256 >= (1L << 31) || (long)a.ldw * ESZ * 256 >= (1L << 31)) return hipErrorInvalidValue;
   int dev = 0;
   (void)hipGetDevice(&dev);
-  auto kern = gemm_dmaf_kernel<IN_DT, OUT_DT, RES_NORM>;
+  auto kern = gemm_dmaf_kernel<IN_DT, OUT_DT, RES_NORM, LEAN>;
   if (!attr_set[dev]) {
     e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, DmafCfg::LDS_BYTES);
     if (e != hipSuccess) return e;

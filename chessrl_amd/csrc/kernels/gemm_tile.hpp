@@ -133,7 +133,10 @@ __device__ __forceinline__ void store8(void* base, long off, const float v[8]) {
 // s0 = 1/std and s1 = -mean/std of row m, from the row statistics a.res_stats and the norm's gain and offset (the normalised tensor then never travels
 // through memory). sStats: 2*WM floats of LDS of this wave's own for its rows' statistics, filled here (RES_NORM 1)
 // or by the kernel before its main loop (RES_NORM 2).
-template <int WM, int WN, int OUT_DT, int RES_NORM = 0, typename AccArr>
+// LEAN (the launcher says when): every row of the tile is inside C, N and nsplit are multiples of 8 with 16-byte aligned
+// rows everywhere, a residual (if any) is bf16 with one row per output row, and no maximum is asked for; the row and
+// alignment guards, the scalar edge stores, the fp32/f16 residual blocks and the maximum then are not in the code at all.
+template <int WM, int WN, int OUT_DT, int RES_NORM = 0, bool LEAN = false, typename AccArr>
 __device__ __forceinline__ void gemm_epilogue(const GemmArgs& a, AccArr& acc, float* sC, int mw0, int nw0, int lane,
                                               float* sStats = nullptr, const float* sCols = nullptr) {
   // sCols (optional, LDS): per-column constants of this wave's WN columns that the kernel has staged before its main
@@ -146,7 +149,7 @@ __device__ __forceinline__ void gemm_epilogue(const GemmArgs& a, AccArr& acc, fl
   const int ec = lane % CP, er = lane / CP;
   const int n = nw0 + ec * 8;
   const bool n_ok = n < a.N;
-  const bool full = a.vec_ok && (n + 7 < a.N) && ((n < a.nsplit) == (n + 7 < a.nsplit));
+  const bool full = LEAN ? true : a.vec_ok && (n + 7 < a.N) && ((n < a.nsplit) == (n + 7 < a.nsplit));
   float bias8[8];
   if (sCols != nullptr) {
     if (a.bias) {
@@ -165,7 +168,7 @@ __device__ __forceinline__ void gemm_epilogue(const GemmArgs& a, AccArr& acc, fl
 #pragma unroll
     for (int e = 0; e < 8; ++e) bias8[e] = (a.bias && n + e < a.N) ? a.bias[n + e] : 0.f;
   }
-  const int res_dt = a.res_dtype;
+  const int res_dt = LEAN ? (int)DT_BF16 : a.res_dtype;
   const float descale = a.descale, alpha = a.alpha;
   float local_amax = 0.f;
   // e4m3(out_scale * mish(descale * acc + bias)) with nothing else asked for (the FFN's first product): the activation in
@@ -230,15 +233,15 @@ __device__ __forceinline__ void gemm_epilogue(const GemmArgs& a, AccArr& acc, fl
   // Raw residual bits, 16 bytes per step and set. 16-bit residuals use the two sets as a double
   // buffer over strips; an fp32 residual (8 values = 32 bytes) uses both sets for the current
   // strip (low and high half), i.e. it is fetched at the start of its own strip.
-  const bool res32 = res_dt == DT_F32;
+  const bool res32 = LEAN ? false : res_dt == DT_F32;
   uint4 rraw[2][ITERS];
   auto load_res = [&](int tm, int set, int half) {
 #pragma unroll
     for (int it = 0; it < ITERS; ++it) {
       const int m = mw0 + tm * 32 + er + it * RSTEP;
       uint4 val = make_uint4(0, 0, 0, 0);
-      if (__builtin_expect(m < a.M && n_ok, 1)) {
-        const long rrow = a.res_rows > 0 ? m % a.res_rows : m;
+      if (__builtin_expect((LEAN || m < a.M) && n_ok, 1)) {
+        const long rrow = (!LEAN && a.res_rows > 0) ? m % a.res_rows : m;
         const long ro = rrow * a.ldr + n;
         if (res32) {
           const float* rp = reinterpret_cast<const float*>(a.res) + ro + 4 * half;
@@ -383,7 +386,7 @@ __device__ __forceinline__ void gemm_epilogue(const GemmArgs& a, AccArr& acc, fl
 #pragma unroll
         for (int e = 0; e < 8; ++e) v[it][e] *= alpha;
     }
-    if (a.amax) {
+    if (!LEAN && a.amax) {
 #pragma unroll
       for (int it = 0; it < ITERS; ++it)
 #pragma unroll
@@ -401,7 +404,7 @@ __device__ __forceinline__ void gemm_epilogue(const GemmArgs& a, AccArr& acc, fl
 #pragma unroll
     for (int it = 0; it < ITERS; ++it) {
       const int m = mw0 + tm * 32 + er + it * RSTEP;
-      if (__builtin_expect(m >= a.M || !n_ok, 0)) continue;
+      if (__builtin_expect((!LEAN && m >= a.M) || !n_ok, 0)) continue;
       if (__builtin_expect(full, 1)) {
         char* dst = out_base + m * out_stride;
         if (a.stream_out) store8<OUT_DT, 1>(dst, 0, v[it]);
@@ -417,7 +420,7 @@ __device__ __forceinline__ void gemm_epilogue(const GemmArgs& a, AccArr& acc, fl
     }
     wave_lds_fence();
   });
-  if (a.amax) {
+  if (!LEAN && a.amax) {
     local_amax = wave_max(local_amax);
     if (lane == 0) atomic_amax(a.amax, local_amax);
   }
