@@ -235,7 +235,21 @@ __device__ __forceinline__ void gemm_epilogue(const GemmArgs& a, AccArr& acc, fl
   // strip (low and high half), i.e. it is fetched at the start of its own strip.
   const bool res32 = LEAN ? false : res_dt == DT_F32;
   uint4 rraw[2][ITERS];
+  // LEAN: rows are visited in order, RSTEP apart, by the residual loads and by the stores alike, so each keeps a running
+  // pointer (one 64-bit add per access where base + row * stride costs a 64-bit multiply-add and its two 32-bit products).
+  const char* res_cur = res_base + (long)(mw0 + er) * res_stride;
+  const long res_step = RSTEP * res_stride;
+  char* out_cur = out_base + (long)(mw0 + er) * out_stride;
+  const long out_step = RSTEP * out_stride;
   auto load_res = [&](int tm, int set, int half) {
+    if constexpr (LEAN) {
+#pragma unroll
+      for (int it = 0; it < ITERS; ++it) {
+        rraw[set][it] = n_ok ? nt_load16(res_cur) : make_uint4(0, 0, 0, 0);
+        res_cur += res_step;
+      }
+      return;
+    }
 #pragma unroll
     for (int it = 0; it < ITERS; ++it) {
       const int m = mw0 + tm * 32 + er + it * RSTEP;
@@ -404,6 +418,14 @@ __device__ __forceinline__ void gemm_epilogue(const GemmArgs& a, AccArr& acc, fl
 #pragma unroll
     for (int it = 0; it < ITERS; ++it) {
       const int m = mw0 + tm * 32 + er + it * RSTEP;
+      if constexpr (LEAN) {
+        if (n_ok) {
+          if (a.stream_out) store8<OUT_DT, 1>(out_cur, 0, v[it]);
+          else store8<OUT_DT, 0>(out_cur, 0, v[it]);
+        }
+        out_cur += out_step;
+        continue;
+      }
       if (__builtin_expect((!LEAN && m >= a.M) || !n_ok, 0)) continue;
       if (__builtin_expect(full, 1)) {
         char* dst = out_base + m * out_stride;
