@@ -15,18 +15,22 @@ hipError_t launch_gemm_dmaf(const GemmArgs& a, int in_dt, int out_dt, hipStream_
   if (a.res_stats) {
     if (in_dt != DT_FP8 || out_dt != DT_BF16 || !a.res || a.res_dtype != DT_BF16 || !a.res_gamma || a.res_rows > 0 || a.alpha == 0.f || (a.M & 1))
       return hipErrorInvalidValue;
-    return dmaf_lean_ok(a) ? launch_dmaf<DT_FP8, DT_BF16, 2, true>(a, st) : launch_dmaf<DT_FP8, DT_BF16, 2>(a, st);
+    switch (dmaf_lean_level(a, out_dt, true)) {
+      case 2: return launch_dmaf<DT_FP8, DT_BF16, 2, 2>(a, st);
+      case 1: return launch_dmaf<DT_FP8, DT_BF16, 2, 1>(a, st);
+    }
+    return launch_dmaf<DT_FP8, DT_BF16, 2>(a, st);
   }
   // (whole tiles in M, aligned rows, a bf16 residual or none, no maximum: the instances without the epilogue's guards)
-  const bool lean = dmaf_lean_ok(a);
+  const int lean = dmaf_lean_level(a, out_dt, false);
   if (in_dt == DT_FP8) {
     switch (out_dt) {
-      case DT_BF16: return lean ? launch_dmaf<DT_FP8, DT_BF16, 0, true>(a, st) : launch_dmaf<DT_FP8, DT_BF16, 0>(a, st);
+      case DT_BF16: return lean == 2 ? launch_dmaf<DT_FP8, DT_BF16, 0, 2>(a, st) : lean == 1 ? launch_dmaf<DT_FP8, DT_BF16, 0, 1>(a, st) : launch_dmaf<DT_FP8, DT_BF16, 0>(a, st);
       case DT_F16: return launch_dmaf<DT_FP8, DT_F16, 0>(a, st);
-      case DT_FP8: return lean ? launch_dmaf<DT_FP8, DT_FP8, 0, true>(a, st) : launch_dmaf<DT_FP8, DT_FP8, 0>(a, st);
+      case DT_FP8: return lean == 2 ? launch_dmaf<DT_FP8, DT_FP8, 0, 2>(a, st) : lean == 1 ? launch_dmaf<DT_FP8, DT_FP8, 0, 1>(a, st) : launch_dmaf<DT_FP8, DT_FP8, 0>(a, st);
     }
   }
-  if (in_dt == DT_BF16 && out_dt == DT_BF16) return lean ? launch_dmaf<DT_BF16, DT_BF16, 0, true>(a, st) : launch_dmaf<DT_BF16, DT_BF16, 0>(a, st);
+  if (in_dt == DT_BF16 && out_dt == DT_BF16) return lean == 2 ? launch_dmaf<DT_BF16, DT_BF16, 0, 2>(a, st) : lean == 1 ? launch_dmaf<DT_BF16, DT_BF16, 0, 1>(a, st) : launch_dmaf<DT_BF16, DT_BF16, 0>(a, st);
   if (in_dt == DT_F16 && out_dt == DT_F16) return launch_dmaf<DT_F16, DT_F16, 0>(a, st);
   return hipErrorInvalidValue;
 }

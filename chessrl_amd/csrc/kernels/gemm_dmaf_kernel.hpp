@@ -51,7 +51,7 @@ inline DmafWalk dmaf_walk(int M, int N, bool fp8) {
 }
 
 // LEAN: the epilogue without its edge and type guards (gemm_epilogue's LEAN; dmaf_lean_ok says when).
-template <int IN_DT, int OUT_DT, int RES_NORM = 0, bool LEAN = false>
+template <int IN_DT, int OUT_DT, int RES_NORM = 0, int LEAN = 0>
 __global__ void __launch_bounds__(DmafCfg::NT, 2) gemm_dmaf_kernel(const GemmArgs a, const int pf, const DmafWalk wk) {
   typedef DmafCfg Cfg;
   constexpr int ESZ = IN_DT == DT_FP8 ? 1 : 2;                      // bytes per operand element
@@ -259,12 +259,23 @@ __global__ void __launch_bounds__(DmafCfg::NT, 2) gemm_dmaf_kernel(const GemmArg
                                                      reinterpret_cast<const float*>(smem + Cfg::COLS_OFF) + wave * (3 * Cfg::WN));
 }
 
+// 0: the general epilogue; 1: without edge, alignment and type guards; 2: with the call's shape fixed at compile time as well
+// (see gemm_epilogue), which is what the products of a large forward pass are.
+inline int dmaf_lean_level(const GemmArgs& a, int out_dt, bool res_norm);
 inline bool dmaf_lean_ok(const GemmArgs& a) {
   return a.M % DmafCfg::BM == 0 && a.vec_ok && a.N % 8 == 0 && a.nsplit % 8 == 0 && !a.amax && a.res_rows == 0 && !a.ln_out &&
          (!a.res || a.res_dtype == DT_BF16);
 }
 
-template <int IN_DT, int OUT_DT, int RES_NORM = 0, bool LEAN = false>
+inline int dmaf_lean_level(const GemmArgs& a, int out_dt, bool res_norm) {
+  if (!dmaf_lean_ok(a)) return 0;
+  if (!a.stream_out) return 1;
+  if (res_norm) return a.act == ACT_NONE ? 2 : 1;
+  if (a.res || a.alpha != 1.f) return 1;
+  return a.act == (out_dt == DT_FP8 ? ACT_MISH : ACT_NONE) ? 2 : 1;
+}
+
+template <int IN_DT, int OUT_DT, int RES_NORM = 0, int LEAN = 0>
 static hipError_t launch_dmaf(const GemmArgs& a, hipStream_t st) {
   static std::atomic<bool> attr_set[16] = {};
   hipError_t e = hipSuccess;

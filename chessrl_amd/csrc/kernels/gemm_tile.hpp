@@ -112,6 +112,22 @@ __device__ __forceinline__ void store8(void* base, long off, const float v[8]) {
   }
 }
 
+// 8 values as 16 bytes of a 16-bit type (all four dwords) or 8 bytes of e4m3 (the first two dwords).
+template <int OUT_DT>
+__device__ __forceinline__ i32x4_t pack8(const float v[8]) {
+  static_assert(OUT_DT != DT_F32, "converted outputs only");
+  if constexpr (OUT_DT == DT_BF16) {
+    return i32x4_t{(int)pack_bf16x2(v[0], v[1]), (int)pack_bf16x2(v[2], v[3]), (int)pack_bf16x2(v[4], v[5]), (int)pack_bf16x2(v[6], v[7])};
+  } else if constexpr (OUT_DT == DT_F16) {
+    uint32_t w[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) w[i] = (uint32_t)f32_to_f16_bits(v[2 * i]) | ((uint32_t)f32_to_f16_bits(v[2 * i + 1]) << 16);
+    return i32x4_t{(int)w[0], (int)w[1], (int)w[2], (int)w[3]};
+  } else {
+    return i32x4_t{(int)pack_fp8x4(v[0], v[1], v[2], v[3]), (int)pack_fp8x4(v[4], v[5], v[6], v[7]), 0, 0};
+  }
+}
+
 // Shared epilogue. acc[tn][tm][r] is output row m = mw0 + tm*32 + lr, column
 // n = nw0 + tn*32 + 8*(r/4) + 4*g + (r%4) (lr = lane%32, g = lane/32); sC is this wave's
 // private LDS patch of 32 x WN floats.
@@ -136,7 +152,9 @@ __device__ __forceinline__ void store8(void* base, long off, const float v[8]) {
 // LEAN (the launcher says when): every row of the tile is inside C, N and nsplit are multiples of 8 with 16-byte aligned
 // rows everywhere, a residual (if any) is bf16 with one row per output row, and no maximum is asked for; the row and
 // alignment guards, the scalar edge stores, the fp32/f16 residual blocks and the maximum then are not in the code at all.
-template <int WM, int WN, int OUT_DT, int RES_NORM = 0, bool LEAN = false, typename AccArr>
+// LEAN == 2 on top of that fixes what the call does at compile time: no activation (for an e4m3 output: the fused mish and
+// nothing else), a residual exactly when RES_NORM says so, alpha = 1 without one, a streamed output.
+template <int WM, int WN, int OUT_DT, int RES_NORM = 0, int LEAN = 0, typename AccArr>
 __device__ __forceinline__ void gemm_epilogue(const GemmArgs& a, AccArr& acc, float* sC, int mw0, int nw0, int lane,
                                               float* sStats = nullptr, const float* sCols = nullptr) {
   // sCols (optional, LDS): per-column constants of this wave's WN columns that the kernel has staged before its main
@@ -144,6 +162,7 @@ __device__ __forceinline__ void gemm_epilogue(const GemmArgs& a, AccArr& acc, fl
   // residual gain at [WN, 2 WN) and offset at [2 WN, 3 WN) (the parts whose pointers are null are not read).
   // acc is f32x16_t[WN/32][WM/32] (32x32 MFMA tiles) or f32x4_t[WN/16][WM/16] (16x16 tiles).
   constexpr bool MI16 = sizeof(acc[0][0]) == sizeof(f32x4_t);
+  constexpr bool EXACT = LEAN == 2;
   constexpr int TM = WM / 32, TN = WN / 32, CH4 = WN / 4, CP = WN / 8, RSTEP = 64 / CP, ITERS = 32 / RSTEP;
   const int lr = lane & 31, g = lane >> 5;
   const int ec = lane % CP, er = lane / CP;
@@ -180,7 +199,7 @@ __device__ __forceinline__ void gemm_epilogue(const GemmArgs& a, AccArr& acc, fl
   bool fused_mish = false;
   float bias_l2[8], d_l2 = 0.f, os_m2 = 0.f, os_1 = 0.f;
   if constexpr (OUT_DT == DT_FP8) {
-    fused_mish = a.act == ACT_MISH && !a.res && alpha == 1.f && !a.amax;
+    fused_mish = EXACT || (a.act == ACT_MISH && !a.res && alpha == 1.f && !a.amax);
     if (fused_mish) {
       constexpr float L2E = 1.4426950408889634f;
       os_1 = a.out_scale; os_m2 = -2.f * os_1;
@@ -280,10 +299,11 @@ __device__ __forceinline__ void gemm_epilogue(const GemmArgs& a, AccArr& acc, fl
       rraw[set][it] = val;
     }
   };
-  if (a.res && !res32) load_res(0, 0, 0);
+  const bool has_res = EXACT ? RES_NORM != 0 : a.res != nullptr;
+  if (has_res && !res32) load_res(0, 0, 0);
   static_for<0, TM>([&](auto tmc) {
     constexpr int tm = decltype(tmc)::value;
-    if (a.res) {
+    if (has_res) {
       if (res32) { load_res(tm, 0, 0); load_res(tm, 1, 1); }
       else if constexpr (tm + 1 < TM) load_res(tm + 1, (tm + 1) & 1, 0);
     }
@@ -332,7 +352,7 @@ __device__ __forceinline__ void gemm_epilogue(const GemmArgs& a, AccArr& acc, fl
       }
     }
     if (fused_mish) goto store_strip;
-    switch (a.act) {  // uniform
+    if constexpr (!EXACT) switch (a.act) {  // uniform
       case ACT_GELU:
 #pragma unroll
         for (int it = 0; it < ITERS; ++it)
@@ -353,7 +373,7 @@ __device__ __forceinline__ void gemm_epilogue(const GemmArgs& a, AccArr& acc, fl
         break;
       default: break;
     }
-    if (a.res) {
+    if (has_res) {
       // One straight block per residual type (the type test per element compiles to a chain of branches).
       if (res32) {
 #pragma unroll
@@ -394,7 +414,7 @@ __device__ __forceinline__ void gemm_epilogue(const GemmArgs& a, AccArr& acc, fl
             v[it][e] = fmaf(v[it][e], alpha, __uint_as_float((e & 1) ? (w[e >> 1] & 0xffff0000u) : (w[e >> 1] << 16)));
         }
       }
-    } else if (alpha != 1.f) {
+    } else if (!EXACT && alpha != 1.f) {
 #pragma unroll
       for (int it = 0; it < ITERS; ++it)
 #pragma unroll
@@ -415,12 +435,54 @@ __device__ __forceinline__ void gemm_epilogue(const GemmArgs& a, AccArr& acc, fl
         for (int e = 0; e < 8; ++e) v[it][e] *= os;
     }
   store_strip:
+
+    if constexpr (LEAN != 0 && OUT_DT != DT_F32) {
+      // All of the strip's vectors are converted into registers of their own before the first store and kept alive past
+      // the last: a 16-byte store written as inline assembly reads its data some cycles after it issues, the compiler
+      // keeps that distance only for stores it generates itself, and in code this tight the next conversion would land in
+      // the registers of a store still reading them.
+      i32x4_t x[ITERS];
+#pragma unroll
+      for (int it = 0; it < ITERS; ++it) x[it] = pack8<OUT_DT>(v[it]);
+      if (n_ok) {
+        if (EXACT || a.stream_out) {
+#pragma unroll
+          for (int it = 0; it < ITERS; ++it) {
+            if constexpr (OUT_DT == DT_FP8) {
+              typedef int i32x2_t __attribute__((ext_vector_type(2)));
+              const i32x2_t x2 = {x[it][0], x[it][1]};
+              asm volatile("global_store_dwordx2 %0, %1, off nt" ::"v"(out_cur), "v"(x2) : "memory");
+            } else {
+              asm volatile("global_store_dwordx4 %0, %1, off nt" ::"v"(out_cur), "v"(x[it]) : "memory");
+            }
+            out_cur += out_step;
+          }
+        } else {
+#pragma unroll
+          for (int it = 0; it < ITERS; ++it) {
+            if constexpr (OUT_DT == DT_FP8) {
+              typedef int i32x2_t __attribute__((ext_vector_type(2)));
+              *reinterpret_cast<i32x2_t*>(out_cur) = i32x2_t{x[it][0], x[it][1]};
+            } else {
+              *reinterpret_cast<i32x4_t*>(out_cur) = x[it];
+            }
+            out_cur += out_step;
+          }
+        }
+      } else {
+        out_cur += ITERS * out_step;
+      }
+      static_assert(ITERS == 4 || ITERS == 2 || ITERS == 8, "strip shapes of the tiled kernels");
+      if constexpr (ITERS == 4) asm volatile("s_nop 7" ::"v"(x[0]), "v"(x[1]), "v"(x[2]), "v"(x[3]));
+      else if constexpr (ITERS == 2) asm volatile("s_nop 7" ::"v"(x[0]), "v"(x[1]));
+      else asm volatile("s_nop 7" ::"v"(x[0]), "v"(x[1]), "v"(x[2]), "v"(x[3]), "v"(x[4]), "v"(x[5]), "v"(x[6]), "v"(x[7]));
+    } else
 #pragma unroll
     for (int it = 0; it < ITERS; ++it) {
       const int m = mw0 + tm * 32 + er + it * RSTEP;
-      if constexpr (LEAN) {
+      if constexpr (LEAN != 0) {
         if (n_ok) {
-          if (a.stream_out) store8<OUT_DT, 1>(out_cur, 0, v[it]);
+          if (EXACT || a.stream_out) store8<OUT_DT, 1>(out_cur, 0, v[it]);
           else store8<OUT_DT, 0>(out_cur, 0, v[it]);
         }
         out_cur += out_step;

@@ -230,6 +230,35 @@ def test_gemm_fp8_out_of_step_kernel_equals_in_step_kernel(cuda, M, N, K, alt):
     assert torch.allclose(out.float(), ref, rtol=2 ** -7, atol=2 ** -7 * ref.abs().max().item()), (out.float() - ref).abs().max()
 
 
+@pytest.mark.parametrize("M,N,K", [(4096, 1536, 1024), (16384, 3104, 1024), (65536, 1536, 1024), (32768, 1024, 1536), (256, 256, 128)])
+def test_gemm_guardless_epilogue_instances_equal_general_kernel(cuda, M, N, K):
+    """With M in whole 256-row tiles, aligned rows, a bf16 residual or none and no running maximum, tile 10 runs instances
+    whose epilogue has no edge, alignment or type guards, and for outputs beyond 64 MB ones whose activation, residual and
+    store kind are fixed at compile time as well (what a 4096-position forward runs: a plain scaled product into bf16, mish
+    into scaled e4m3). Same arithmetic: bit-equal to the general kernel (tile 7) in every combination, including the ones
+    that fall back to the guarded instance (activation with a residual) and a last tile column that is mostly outside N."""
+    torch.manual_seed(M + N + K)
+    A = (torch.randn(M, K, device=cuda) * 30).to(torch.float8_e4m3fn)
+    W = (torch.randn(N, K, device=cuda) * 30).to(torch.float8_e4m3fn)
+    bias = torch.randn(N, device=cuda)
+    res = torch.randn(M, N, device=cuda).bfloat16()
+    for kw in (dict(out_dt=_lib.BF16, descale=1e-3), dict(out_dt=_lib.BF16, bias=bias, descale=1e-3),
+               dict(out_dt=_lib.BF16, bias=bias, descale=1e-3, alpha=0.43, res=res),
+               dict(out_dt=_lib.BF16, bias=bias, act=2, descale=1e-3, alpha=0.43, res=res),
+               dict(out_dt=_lib.FP8, bias=bias, act=2, descale=1e-3, out_scale=7.0),
+               dict(out_dt=_lib.FP8, descale=1e-3, out_scale=7.0)):
+        args = {k: v for k, v in kw.items() if k != "out_dt"}
+        lean = run_gemm(A, W, kw["out_dt"], tile=10, **args)
+        general = run_gemm(A, W, kw["out_dt"], tile=7, **args)
+        if kw["out_dt"] == _lib.FP8 and kw.get("act") == 2:
+            # the e4m3 mish of tile 10 is the fused form (1 - 2 / (n (n + 2) + 2) with the scale folded in): the same
+            # function to fp32 rounding, so a code differs only where the value sits on a rounding boundary
+            a8, b8 = lean.view(torch.float8_e4m3fn).float(), general.view(torch.float8_e4m3fn).float()
+            assert (a8 != b8).float().mean().item() < 1e-4 and torch.allclose(a8, b8, rtol=2 ** -3, atol=2 ** -9)
+        else:
+            assert torch.equal(lean, general), (M, N, K, kw["out_dt"], sorted(args))
+
+
 @pytest.mark.parametrize("M,N,K", [(128, 128, 64), (128, 128, 256), (4096, 1024, 1024), (4096, 1536, 1024), (4096, 1024, 1536), (2048, 4096, 256),
                                    (300, 700, 512), (1000, 3104, 1024), (4096, 200, 192), (130, 129, 128), (640, 3104, 1088)])
 @pytest.mark.parametrize("dt", ["bf16", "fp8"])
