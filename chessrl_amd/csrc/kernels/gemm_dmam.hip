@@ -11,6 +11,12 @@ bool gemm_dmam_has(int in_dt, int out_dt) {
 }
 
 hipError_t launch_gemm_dmam(const GemmArgs& a, int in_dt, int out_dt, hipStream_t st) {
+  // (whole tiles in M, aligned rows, a bf16 residual or none, no maximum: the instances without the epilogue's guards)
+  const bool lean = a.M % DmamCfg::BM == 0 && a.vec_ok && a.N % 8 == 0 && a.nsplit % 8 == 0 && !a.amax && a.res_rows == 0 && !a.ln_out &&
+                    (!a.res || a.res_dtype == DT_BF16);
+  if (lean && in_dt == DT_FP8 && out_dt == DT_BF16) return launch_dmam<DT_FP8, DT_BF16, 1>(a, st);
+  if (lean && in_dt == DT_FP8 && out_dt == DT_FP8) return launch_dmam<DT_FP8, DT_FP8, 1>(a, st);
+  if (lean && in_dt == DT_BF16 && out_dt == DT_BF16) return launch_dmam<DT_BF16, DT_BF16, 1>(a, st);
   if (in_dt == DT_FP8) {
     switch (out_dt) {
       case DT_BF16: return launch_dmam<DT_FP8, DT_BF16>(a, st);

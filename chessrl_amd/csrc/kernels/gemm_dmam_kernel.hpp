@@ -29,7 +29,8 @@ struct DmamCfg {
 // operation, i.e. for the slabs that are meant to stay in flight).
 __device__ __forceinline__ void dmam_barrier() { asm volatile("s_barrier" ::: "memory"); }
 
-template <int IN_DT, int OUT_DT>
+// LEAN: the epilogue without its edge and type guards (gemm_epilogue's LEAN = 1; the launcher says when).
+template <int IN_DT, int OUT_DT, int LEAN = 0>
 __global__ void __launch_bounds__(DmamCfg::NT) gemm_dmam_kernel(const GemmArgs a, const DmafWalk wk) {
   typedef DmamCfg Cfg;
   constexpr int ESZ = IN_DT == DT_FP8 ? 1 : 2;                      // bytes per operand element
@@ -156,12 +157,12 @@ __global__ void __launch_bounds__(DmamCfg::NT) gemm_dmam_kernel(const GemmArgs a
   wait_vmcnt<0>();
   dmam_barrier();  // every wave is done with the ring, and the empty loads past the end of K have retired
 
-  gemm_epilogue<Cfg::WM, Cfg::WN, OUT_DT, 0>(a, acc, reinterpret_cast<float*>(smem) + wave * (32 * Cfg::WN),
+  gemm_epilogue<Cfg::WM, Cfg::WN, OUT_DT, 0, LEAN>(a, acc, reinterpret_cast<float*>(smem) + wave * (32 * Cfg::WN),
                                               m0 + wm * Cfg::WM, n0 + wn * Cfg::WN, lane, nullptr,
                                               reinterpret_cast<const float*>(smem + Cfg::COLS_OFF) + wave * (3 * Cfg::WN));
 }
 
-template <int IN_DT, int OUT_DT>
+template <int IN_DT, int OUT_DT, int LEAN = 0>
 static hipError_t launch_dmam(const GemmArgs& a, hipStream_t st) {
   static std::atomic<bool> attr_set[16] = {};
   hipError_t e = hipSuccess;
@@ -170,7 +171,7 @@ static hipError_t launch_dmam(const GemmArgs& a, hipStream_t st) {
     return hipErrorInvalidValue;
   int dev = 0;
   (void)hipGetDevice(&dev);
-  auto kern = gemm_dmam_kernel<IN_DT, OUT_DT>;
+  auto kern = gemm_dmam_kernel<IN_DT, OUT_DT, LEAN>;
   if (!attr_set[dev]) {
     e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, DmamCfg::LDS_BYTES);
     if (e != hipSuccess) return e;

@@ -257,6 +257,10 @@ def test_gemm_guardless_epilogue_instances_equal_general_kernel(cuda, M, N, K):
             assert (a8 != b8).float().mean().item() < 1e-4 and torch.allclose(a8, b8, rtol=2 ** -3, atol=2 ** -9)
         else:
             assert torch.equal(lean, general), (M, N, K, kw["out_dt"], sorted(args))
+        # the 128x128 tile has such an instance too (tile 11, where M is whole 128-row tiles) against its register-staged
+        # twin with the general epilogue (tile 12)
+        if M <= 16384:
+            assert torch.equal(run_gemm(A, W, kw["out_dt"], tile=11, **args), run_gemm(A, W, kw["out_dt"], tile=12, **args)), (M, N, K, sorted(args))
 
 
 @pytest.mark.parametrize("M,N,K", [(128, 128, 64), (128, 128, 256), (4096, 1024, 1024), (4096, 1536, 1024), (4096, 1024, 1536), (2048, 4096, 256),
