@@ -86,9 +86,11 @@ __device__ __forceinline__ uint4 nt_load16(const char* p) {
 template <int OUT_DT, int NT = 0>
 __device__ __forceinline__ void store8(void* base, long off, const float v[8]) {
   // The hint is written as an instruction: __builtin_nontemporal_store beside a plain store of the same value in the
-  // other arm of a branch is merged with it by the compiler, and the hint is dropped.
+  // other arm of a branch is merged with it by the compiler, and the hint is dropped. The idle cycles behind it keep the
+  // next writer of the data registers away: a 16-byte store reads them some cycles after it issues, and the compiler,
+  // which knows that of its own stores, cannot see this one.
   auto put = [](i32x4_t* p, i32x4_t x) {
-    if constexpr (NT) asm volatile("global_store_dwordx4 %0, %1, off nt" ::"v"(p), "v"(x) : "memory");
+    if constexpr (NT) asm volatile("global_store_dwordx4 %0, %1, off nt\n\ts_nop 7" ::"v"(p), "v"(x) : "memory");
     else *p = x;
   };
   if constexpr (OUT_DT == DT_F32) {
