@@ -135,6 +135,75 @@ __global__ void __launch_bounds__(256) layernorm_kernel(const LayerNormArgs a) {
   }
 }
 
+// The trunk's norm: bf16 rows of exactly 1024 elements, LayerNorm with offset, outputs bf16 and/or e4m3. Same arithmetic per
+// row as layernorm_kernel (same order of additions, same roundings), but with everything about the call fixed at compile
+// time and all of a wave's loads (RPW rows, then scale and offset, which RPW rows share) issued before the first
+// reduction, so that a wave waits for memory once instead of three times.
+template <bool OUT16, bool OUT8, int RPW>
+__global__ void __launch_bounds__(256) layernorm_trunk_kernel(const LayerNormArgs a) {
+  const int lane = threadIdx.x & 63;
+  const long row0 = ((long)blockIdx.x * 4 + (threadIdx.x >> 6)) * RPW;
+  if (row0 >= a.rows) return;
+  float x[RPW][2][8], g[2][8], b[2][8];
+#pragma unroll
+  for (int i = 0; i < 2; ++i) {
+    load8<DT_F32>(a.gamma, (i * 64 + lane) * 8, g[i]);
+    load8<DT_F32>(a.beta, (i * 64 + lane) * 8, b[i]);
+  }
+#pragma unroll
+  for (int r = 0; r < RPW; ++r) {
+#pragma unroll
+    for (int i = 0; i < 2; ++i) load8<DT_BF16>(a.x, (row0 + r) * a.ldx + (i * 64 + lane) * 8, x[r][i]);
+  }
+  __builtin_amdgcn_sched_barrier(0);   // (no use of a loaded value, and so no wait, moves up between the loads)
+  const float inv_c = fast_rcp(1024.f);
+  float am = 0.f;
+#pragma unroll
+  for (int r = 0; r < RPW; ++r) {
+    float s = 0.f;
+#pragma unroll
+    for (int i = 0; i < 2; ++i) {
+#pragma unroll
+      for (int e = 0; e < 8; ++e) s += x[r][i][e];
+    }
+    const float mean = wave_sum(s) * inv_c;
+    float q = 0.f;
+#pragma unroll
+    for (int i = 0; i < 2; ++i) {
+#pragma unroll
+      for (int e = 0; e < 8; ++e) { const float d = x[r][i][e] - mean; q += d * d; }
+    }
+    const float rstd = rsqrtf(wave_sum(q) * inv_c + a.eps);
+    if (a.stats && lane == 0) *reinterpret_cast<float2*>(a.stats + 2 * (row0 + r)) = make_float2(rstd, -mean * rstd);
+#pragma unroll
+    for (int i = 0; i < 2; ++i) {
+      float y[8];
+#pragma unroll
+      for (int e = 0; e < 8; ++e) y[e] = (x[r][i][e] - mean) * rstd * g[i][e] + b[i][e];
+      const long off = (row0 + r) * a.ldo + (i * 64 + lane) * 8;
+      if constexpr (OUT16) store8(a.out, off, y, DT_BF16);
+      if constexpr (OUT8) store8_fp8(a.out_fp8, off, y, a.fp8_scale);
+      if (a.amax) {
+#pragma unroll
+        for (int e = 0; e < 8; ++e) am = fmaxf(am, fabsf(y[e]));
+      }
+    }
+  }
+  if (a.amax) {
+    am = wave_max(am);
+    if (lane == 0) atomic_amax(a.amax, am);
+  }
+}
+
+template <int RPW>
+static bool launch_ln_trunk(const LayerNormArgs& a, hipStream_t st) {
+  const dim3 grid((a.rows / RPW + 3) / 4), block(256);
+  if (a.out && a.out_fp8) hipLaunchKernelGGL((layernorm_trunk_kernel<true, true, RPW>), grid, block, 0, st, a);
+  else if (a.out) hipLaunchKernelGGL((layernorm_trunk_kernel<true, false, RPW>), grid, block, 0, st, a);
+  else hipLaunchKernelGGL((layernorm_trunk_kernel<false, true, RPW>), grid, block, 0, st, a);
+  return true;
+}
+
 // Rows longer than 2048 elements (the 8192-wide norm of the bias generator): the four waves of a workgroup share one
 // row, 8 elements per thread and step of 2048, and meet through LDS for the two reductions (wave sums added in wave
 // order). Chosen by the row length alone, so a row's result does not depend on how many rows the call has; with one
@@ -203,6 +272,14 @@ template <int IN_DT>
 static hipError_t launch_ln_dt(const LayerNormArgs& a, hipStream_t st) {
   const dim3 grid((a.rows + 3) / 4), block(256);
   const int vecs = (a.C / 8 + 63) / 64;
+  if constexpr (IN_DT == DT_BF16) {
+    if (a.C == 1024 && !a.rms && a.beta && !a.out_b && (a.out || a.out_fp8) && (!a.out || a.out_dtype == DT_BF16)) {
+      // (two rows per wave: 18 % faster than one at 262144 rows, and no slower than four; per-row arithmetic is the same)
+      if (a.rows % 2 == 0) launch_ln_trunk<2>(a, st);
+      else launch_ln_trunk<1>(a, st);
+      return hipGetLastError();
+    }
+  }
   if (vecs <= 1) hipLaunchKernelGGL((layernorm_kernel<IN_DT, 1>), grid, block, 0, st, a);
   else if (a.C == 1024) hipLaunchKernelGGL((layernorm_kernel<IN_DT, 2, true>), grid, block, 0, st, a);   // (the trunk's width: no column guards)
   else if (vecs <= 2) hipLaunchKernelGGL((layernorm_kernel<IN_DT, 2>), grid, block, 0, st, a);

@@ -357,6 +357,39 @@ def test_layernorm(cuda, C_, in_dt):
     assert abs(amax.item() - ref.abs().max().item()) < 1e-3 * ref.abs().max().item()
 
 
+@pytest.mark.parametrize("rows", [77, 4098])
+def test_layernorm_trunk_width_instance_equals_general_kernel(cuda, rows):
+    """bf16 rows of 1024 elements take an instance of their own (all loads issued up front, one or two rows per wave by
+    the parity of the row count) unless the 16-bit output is f16: the e4m3 copy, the maximum and, across row counts, the
+    bf16 output must carry the same bits either way."""
+    torch.manual_seed(rows)
+    C_ = 1024
+    x = (torch.randn(rows, C_, device=cuda) * (torch.rand(rows, 1, device=cuda) * 4) + torch.randn(rows, 1, device=cuda)).bfloat16()
+    g = torch.randn(C_, device=cuda)
+    b = torch.randn(C_, device=cuda)
+
+    def run(n, out_dt, want16=True, want8=True):
+        out = torch.zeros(n, C_, dtype=TORCH_DT[out_dt], device=cuda) if want16 else None
+        out8 = torch.zeros(n, C_, dtype=torch.uint8, device=cuda) if want8 else None
+        amax = torch.zeros(1, device=cuda)
+        check(lib().crl_layernorm(p(x), C_, _lib.BF16, p(g), p(b), p(out), out_dt, p(out8), 0.7, C_, n, C_, 1e-5, p(amax), stream()), "ln")
+        torch.cuda.synchronize()
+        return out, out8, amax.item()
+
+    o_t, o8_t, am_t = run(rows, _lib.BF16)           # the instance for this width
+    o_g, o8_g, am_g = run(rows, _lib.F16)            # the general kernel
+    assert torch.equal(o8_t, o8_g) and am_t == am_g
+    assert torch.allclose(o_t.float(), o_g.float(), rtol=2 ** -8, atol=2 ** -8)
+    _, o8_only, am_only = run(rows, _lib.BF16, want16=False)
+    assert torch.equal(o8_only, o8_t) and am_only == am_t
+    o_16, _, _ = run(rows, _lib.BF16, want8=False)
+    assert torch.equal(o_16, o_t)
+    o_less, o8_less, _ = run(rows - 1, _lib.BF16)    # the other parity: the other number of rows per wave
+    assert torch.equal(o_less, o_t[:rows - 1]) and torch.equal(o8_less, o8_t[:rows - 1])
+    ref = F.layer_norm(x.float(), (C_,), g, b, 1e-5)
+    assert torch.allclose(o_t.float(), ref, rtol=2 ** -8, atol=2 ** -8)
+
+
 def make_qkv(B, H, hs, device, seed, dtype=torch.bfloat16):
     torch.manual_seed(seed)
     Cm = H * hs
