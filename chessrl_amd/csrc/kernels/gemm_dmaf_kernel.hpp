@@ -236,11 +236,13 @@ __global__ void __launch_bounds__(DmafCfg::NT, 2) gemm_dmaf_kernel(const GemmArg
         constexpr int i = decltype(ic)::value;
         constexpr int tn = i / TM, tm = i % TM;
         acc[tn][tm] = mfma_frag<IN_DT>(wf[tn], xf[tm], acc[tn][tm]);
-        // With e4m3 operands the next slab's loads go out one at a time, after every second MFMA, held in place by
-        // scheduling barriers.
-        if constexpr (SPREAD && (i & 1) == 1) {
+        // With e4m3 operands the next slab's loads go out one at a time, one behind each of the slab's first eight MFMAs,
+        // held in place by scheduling barriers: the last of them then has the other eight MFMAs in which to land before
+        // the wave waits for it (spread over all sixteen, one behind every second MFMA, the products of a large pass
+        // take 3.8 % longer; starting one MFMA earlier or two later, or two loads behind each of four MFMAs, 1 %).
+        if constexpr (SPREAD && ks == 0) {
           __builtin_amdgcn_sched_barrier(0);
-          issue_one(slab + 1, rnext, std::integral_constant<int, ks * 4 + (i >> 1)>{});
+          issue_one(slab + 1, rnext, std::integral_constant<int, i>{});
           __builtin_amdgcn_sched_barrier(0);
         }
       });
