@@ -51,6 +51,7 @@ SIGNATURES = {
     "crl_perft": (C.c_uint64, [_cp, _i]),
     "crl_random_positions": (_i, [C.c_uint64, _i, _i, C.c_double, _i, _vp, _vp, _vp, _vp]),
     "crl_gemm": (_i, [_vp, _i64, _vp, _i64, _vp, _i64, _i, _i, _i, _i, _i, _vp, _i, _f, _f, _vp, _i64, _i, _f, _vp, _i, _vp]),
+    "crl_gemm_split": (_i, [_vp, _i64, _vp, _i64, _vp, _i64, _vp, _i64, _i, _i, _i, _i, _i, _i, _vp, _f, _i, _vp]),
     "crl_gemm_static_scratch": (_i, [_vp, _i64, _vp, _i64, _vp, _i64, _i, _i, _i, _i, _i, _vp, _i, _f, _f, _vp, _i64, _i, _f, _vp, _vp]),
     "crl_gemm_static_scratch_bytes": (_i64, []),
     "crl_shutdown": (None, []),

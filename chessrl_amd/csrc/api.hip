@@ -223,6 +223,22 @@ int crl_gemm(const void* A, int64_t lda, const void* W, int64_t ldw, void* C, in
   return e == hipSuccess ? CRL_OK : hip_fail("crl_gemm", e);
 }
 
+int crl_gemm_split(const void* A, int64_t lda, const void* W, int64_t ldw, void* C, int64_t ldc, void* C2, int64_t ldc2, int nsplit,
+                   int M, int N, int K, int in_dtype, int out_dtype, const float* bias, float descale, int tile, void* stream) {
+  if (!A || !W || !C || !C2 || M < 0 || N < 0 || K <= 0) return arg_fail("crl_gemm_split: bad arguments");
+  if (nsplit <= 0 || nsplit >= N || nsplit % 8 != 0) return arg_fail("crl_gemm_split: nsplit must be a multiple of 8 inside (0, N)");
+  if (in_dtype != DT_BF16 && in_dtype != DT_F16 && in_dtype != DT_FP8) return arg_fail("crl_gemm_split: in_dtype must be bf16, f16 or fp8");
+  if (out_dtype < 0 || out_dtype > 3 || (tile != 0 && tile != 3 && tile != 7 && tile != 10)) return arg_fail("crl_gemm_split: bad out_dtype or tile");
+  GemmArgs g;
+  std::memset(&g, 0, sizeof(g));
+  g.A = A; g.lda = lda; g.W = W; g.ldw = ldw; g.C = C; g.ldc = ldc; g.C2 = C2; g.ldc2 = ldc2; g.M = M; g.N = N; g.K = K; g.nsplit = nsplit;
+  g.bias = bias; g.descale = descale; g.alpha = 1.f; g.out_scale = 1.f;
+  hipError_t e = launch_gemm(g, in_dtype, out_dtype, tile, (hipStream_t)stream);
+  if (e == hipErrorInvalidValue)
+    return arg_fail("crl_gemm_split: operands must be 16-byte aligned with K*elem_size a multiple of 16");
+  return e == hipSuccess ? CRL_OK : hip_fail("crl_gemm_split", e);
+}
+
 int crl_gemm_static_scratch(const void* A, int64_t lda, const void* W, int64_t ldw, void* C, int64_t ldc, int M, int N, int K, int in_dtype,
                             int out_dtype, const float* bias, int act, float descale, float alpha, const void* res, int64_t ldr,
                             int res_dtype, float out_scale, float* amax, void* stream) {

@@ -25,7 +25,9 @@ hipError_t launch_gemm_dmaf(const GemmArgs& a, int in_dt, int out_dt, hipStream_
   const int lean = dmaf_lean_level(a, out_dt, false);
   if (in_dt == DT_FP8) {
     switch (out_dt) {
-      case DT_BF16: return lean == 2 ? launch_dmaf<DT_FP8, DT_BF16, 0, 2>(a, st) : lean == 1 ? launch_dmaf<DT_FP8, DT_BF16, 0, 1>(a, st) : launch_dmaf<DT_FP8, DT_BF16, 0>(a, st);
+      case DT_BF16:
+        if (lean == 2 && dmaf_xtra_ok(a)) return launch_dmaf<DT_FP8, DT_BF16, 0, 2, 1>(a, st);
+        return lean == 2 ? launch_dmaf<DT_FP8, DT_BF16, 0, 2>(a, st) : lean == 1 ? launch_dmaf<DT_FP8, DT_BF16, 0, 1>(a, st) : launch_dmaf<DT_FP8, DT_BF16, 0>(a, st);
       case DT_F16: return launch_dmaf<DT_FP8, DT_F16, 0>(a, st);
       case DT_FP8: return lean == 2 ? launch_dmaf<DT_FP8, DT_FP8, 0, 2>(a, st) : lean == 1 ? launch_dmaf<DT_FP8, DT_FP8, 0, 1>(a, st) : launch_dmaf<DT_FP8, DT_FP8, 0>(a, st);
     }

@@ -23,6 +23,11 @@ struct DmafCfg {
   static constexpr int STATS_OFF = RING_BYTES + 256;        // behind the landing strip of the L2 touches
   static constexpr int COLS_OFF = STATS_OFF + NW * 2 * WM * 4;   // per-column epilogue constants: [wave][bias, gain, offset][WN]
   static constexpr int LDS_BYTES = COLS_OFF + NW * 3 * WN * 4;
+  // XTRA instances: up to 32 weight rows beyond the last tile column, two stages of 4 KB on an 8 KB boundary (a stage is
+  // bit 12 of an address there).
+  static constexpr int XTRA_OFF = (LDS_BYTES + 8191) / 8192 * 8192;
+  static constexpr int LDS_BYTES_XTRA = XTRA_OFF + 8192;
+  static_assert(LDS_BYTES_XTRA <= 160 * 1024, "LDS of a CU");
 };
 
 // The tile walk's constants, worked out once on the host: the walk divides a workgroup index by six launch constants,
@@ -51,7 +56,12 @@ inline DmafWalk dmaf_walk(int M, int N, bool fp8) {
 }
 
 // LEAN: the epilogue without its edge and type guards (gemm_epilogue's LEAN; dmaf_lean_ok says when).
-template <int IN_DT, int OUT_DT, int RES_NORM = 0, int LEAN = 0>
+// XTRA: the tile columns cover the first nsplit columns only (nsplit a multiple of 256), and the workgroups of the last
+// tile column also compute the up to 32 columns behind them (the second output of a column split): every wave one more
+// 32x32 MFMA tile per K step, rows [32 wn, +32) of its 128, on weight rows that four more loads per slab bring in. Same
+// operands in the same K order as a tile column of their own would use (bit-equal), without that column's second pass
+// over the activations.
+template <int IN_DT, int OUT_DT, int RES_NORM = 0, int LEAN = 0, int XTRA = 0>
 __global__ void __launch_bounds__(DmafCfg::NT, 2) gemm_dmaf_kernel(const GemmArgs a, const int pf, const DmafWalk wk) {
   typedef DmafCfg Cfg;
   constexpr int ESZ = IN_DT == DT_FP8 ? 1 : 2;                      // bytes per operand element
@@ -116,8 +126,31 @@ __global__ void __launch_bounds__(DmafCfg::NT, 2) gemm_dmaf_kernel(const GemmArg
     __builtin_amdgcn_raw_ptr_buffer_load_lds(r, (__attribute__((address_space(3))) void*)(smem + (lds_load0 ^ ((slab & 1) << 15)) + i * 1024), 16,
                                              (int)voff[i], slab * Cfg::ROWB, 0, 0);
   };
+  // XTRA: waves 0-3 bring in eight of the extra weight rows each.
+  const bool extra = XTRA != 0 && tile_n == tiles_n - 1;
+  const int n_x = n0 + BN;   // first extra column
+  uint32_t voff_x = 0;
+  __amdgpu_buffer_rsrc_t rsrc_xw = rsrc_none;
+  if constexpr (XTRA != 0) {
+    if (extra && !loads_a) {
+      const int rows_x = a.N - n_x < 32 ? a.N - n_x : 32;
+      int r = 8 * wave + (lane >> 3);
+      r = r < rows_x ? r : rows_x - 1;
+      voff_x = (uint32_t)r * (uint32_t)ld + (((lane & 7) ^ (lane >> 3) ^ wave) << 4);
+      rsrc_xw = make_rsrc(reinterpret_cast<const uint8_t*>(a.W) + (long)n_x * a.ldw * ESZ, rows_x, (long)a.ldw * ESZ);
+    }
+  }
+  auto issue_extra = [&](int slab, bool live) {
+    if constexpr (XTRA != 0) {
+      if (extra && !loads_a)
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(live ? rsrc_xw : rsrc_none,
+                                                 (__attribute__((address_space(3))) void*)(smem + Cfg::XTRA_OFF + ((slab & 1) << 12) + wave * 1024), 16,
+                                                 (int)voff_x, slab * Cfg::ROWB, 0, 0);
+    }
+  };
   // The first slab is requested as early as its addresses exist; everything else the prologue sets up follows.
   static_for<0, LOADS>([&](auto ic) { issue_one(0, rsrc_mine, ic); });
+  issue_extra(0, true);
   __builtin_amdgcn_sched_barrier(0);
 
   // The per-column constants of the epilogue (bias; gain and offset of a residual normalised on the fly) for this wave's
@@ -202,6 +235,20 @@ __global__ void __launch_bounds__(DmafCfg::NT, 2) gemm_dmaf_kernel(const GemmArg
     return *reinterpret_cast<const __attribute__((address_space(3))) i32x4_t*>((is_w ? wb[k] : xb[k]) + t * 32 * Cfg::ROWB);
   };
 
+  // XTRA: fragment addresses of the extra weight rows (row lr of 32) and of this wave's rows [32 wn, +32) of its activation block.
+  uint32_t eb[4] = {0, 0, 0, 0};
+  f32x16_t accx;
+#pragma unroll
+  for (int r = 0; r < 16; ++r) accx[r] = 0.f;
+  const uint32_t xrow_off = (uint32_t)wn * 32 * Cfg::ROWB;
+  if constexpr (XTRA != 0) {
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+      const int kc = (k & 1) | ((k >> 1) << 2);
+      eb[k] = lds0 + Cfg::XTRA_OFF + lr * Cfg::ROWB + ((kc ^ L0) << 4);
+    }
+  }
+
   // A wave whose 128x64 part lies wholly outside C still takes its share of the loads and every barrier.
   const bool wave_active = (m0 + wm * Cfg::WM < a.M) && (n0 + wn * Cfg::WN < a.N);
 
@@ -215,6 +262,7 @@ __global__ void __launch_bounds__(DmafCfg::NT, 2) gemm_dmaf_kernel(const GemmArg
     prefetch(slab + 1 + pf);
     if (!wave_active) {
       static_for<0, LOADS>([&](auto ic) { issue_one(slab + 1, rnext, ic); });
+      issue_extra(slab + 1, slab + 1 < nslab);
       continue;
     }
     constexpr bool SPREAD = IN_DT == DT_FP8;   // 16-bit operands measure 2-3 % slower with their loads spread out
@@ -243,10 +291,28 @@ __global__ void __launch_bounds__(DmafCfg::NT, 2) gemm_dmaf_kernel(const GemmArg
         if constexpr (SPREAD && ks == 0) {
           __builtin_amdgcn_sched_barrier(0);
           issue_one(slab + 1, rnext, std::integral_constant<int, i>{});
+          if constexpr (i == TN * TM - 1) issue_extra(slab + 1, slab + 1 < nslab);
           __builtin_amdgcn_sched_barrier(0);
         }
       });
+      if constexpr (XTRA != 0 && IN_DT == DT_FP8) {
+        if (extra) {
+          constexpr int k0 = (4 * ks) & 1 | (((4 * ks) >> 2) << 1), k1 = ((4 * ks + 1) & 1) | (((4 * ks + 1) >> 2) << 1);
+          Frag<IN_DT> wfx, xfx;
+          wfx.lo = *reinterpret_cast<const __attribute__((address_space(3))) i32x4_t*>(eb[k0]);
+          wfx.hi = *reinterpret_cast<const __attribute__((address_space(3))) i32x4_t*>(eb[k1]);
+          // (rows 32 t + lr of a block carry the swizzle of lr with bit 2 flipped for odd t: the other pair of lane addresses)
+          const uint32_t xa0 = ((wn & 1) ? xb[k0 ^ 2] : xb[k0]) + xrow_off, xa1 = ((wn & 1) ? xb[k1 ^ 2] : xb[k1]) + xrow_off;
+          xfx.lo = *reinterpret_cast<const __attribute__((address_space(3))) i32x4_t*>(xa0);
+          xfx.hi = *reinterpret_cast<const __attribute__((address_space(3))) i32x4_t*>(xa1);
+          accx = mfma_frag<IN_DT>(wfx, xfx, accx);
+        }
+      }
     });
+    if constexpr (XTRA != 0) {
+#pragma unroll
+      for (int k = 0; k < 4; ++k) eb[k] ^= 4096u;
+    }
     // The address registers follow the ring to the other stage.
 #pragma unroll
     for (int k = 0; k < 4; ++k) { wb[k] ^= 32768u; xb[k] ^= 32768u; }
@@ -259,6 +325,16 @@ __global__ void __launch_bounds__(DmafCfg::NT, 2) gemm_dmaf_kernel(const GemmArg
                                                      m0 + wm * Cfg::WM, n0 + wn * Cfg::WN, lane,
                                                      reinterpret_cast<float*>(smem + Cfg::STATS_OFF) + wave * (2 * Cfg::WM),
                                                      reinterpret_cast<const float*>(smem + Cfg::COLS_OFF) + wave * (3 * Cfg::WN));
+  if constexpr (XTRA != 0) {
+    if (extra) {
+      // The extra columns' 32x32 tile of this wave, through the same patch (its bias comes from global memory).
+      f32x16_t ax[1][1];
+      ax[0][0] = accx;
+      wave_lds_fence();
+      gemm_epilogue<32, 32, OUT_DT, 0, LEAN>(a, ax, reinterpret_cast<float*>(smem) + wave * (32 * Cfg::WN),
+                                             m0 + wm * Cfg::WM + wn * 32, n_x, lane);
+    }
+  }
 }
 
 // 0: the general epilogue; 1: without edge, alignment and type guards; 2: with the call's shape fixed at compile time as well
@@ -277,7 +353,12 @@ inline int dmaf_lean_level(const GemmArgs& a, int out_dt, bool res_norm) {
   return a.act == (out_dt == DT_FP8 ? ACT_MISH : ACT_NONE) ? 2 : 1;
 }
 
-template <int IN_DT, int OUT_DT, int RES_NORM = 0, int LEAN = 0>
+// Whether the XTRA instance serves this call: a column split at a multiple of 256 with at most 32 columns behind it.
+inline bool dmaf_xtra_ok(const GemmArgs& a) {
+  return a.C2 != nullptr && a.nsplit >= 256 && a.nsplit % 256 == 0 && a.N > a.nsplit && a.N - a.nsplit <= 32;
+}
+
+template <int IN_DT, int OUT_DT, int RES_NORM = 0, int LEAN = 0, int XTRA = 0>
 static hipError_t launch_dmaf(const GemmArgs& a, hipStream_t st) {
   static std::atomic<bool> attr_set[16] = {};
   hipError_t e = hipSuccess;
@@ -286,18 +367,20 @@ static hipError_t launch_dmaf(const GemmArgs& a, hipStream_t st) {
   if ((a.K * ESZ) % DmafCfg::ROWB != 0 || a.K <= 0 || (long)a.lda * ESZ * 256 >= (1L << 31) || (long)a.ldw * ESZ * 256 >= (1L << 31)) return hipErrorInvalidValue;
   int dev = 0;
   (void)hipGetDevice(&dev);
-  auto kern = gemm_dmaf_kernel<IN_DT, OUT_DT, RES_NORM, LEAN>;
+  auto kern = gemm_dmaf_kernel<IN_DT, OUT_DT, RES_NORM, LEAN, XTRA>;
+  constexpr int LDS = XTRA ? DmafCfg::LDS_BYTES_XTRA : DmafCfg::LDS_BYTES;
   if (!attr_set[dev]) {
-    e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, DmafCfg::LDS_BYTES);
+    e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, LDS);
     if (e != hipSuccess) return e;
     attr_set[dev] = true;
   }
-  const int tiles_n = (a.N + DmafCfg::BN - 1) / DmafCfg::BN;
+  const int Nt = XTRA ? a.nsplit : a.N;   // columns the tile columns cover
+  const int tiles_n = (Nt + DmafCfg::BN - 1) / DmafCfg::BN;
   const int tiles = ((a.M + DmafCfg::BM - 1) / DmafCfg::BM) * tiles_n;
   // (the L2 touches pay for e4m3 operands only: the 16-bit instances lose 2-6 % with them)
   const int pf = (IN_DT == DT_FP8 && tiles_n % 4 == 0 && (long)a.K >= 8 * DmafCfg::ROWB) ? 2 : 0;
   if (tiles >= 65536) return hipErrorInvalidValue;   // (the walk's divisions are exact below that; the caller has another kernel)
-  hipLaunchKernelGGL(kern, dim3(tiles), dim3(DmafCfg::NT), DmafCfg::LDS_BYTES, st, a, pf, dmaf_walk(a.M, a.N, IN_DT == DT_FP8));
+  hipLaunchKernelGGL(kern, dim3(tiles), dim3(DmafCfg::NT), LDS, st, a, pf, dmaf_walk(a.M, Nt, IN_DT == DT_FP8));
   return hipGetLastError();
 }
 

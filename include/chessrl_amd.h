@@ -128,6 +128,16 @@ int crl_gemm(const void* A, int64_t lda, const void* W, int64_t ldw, void* C, in
              const float* bias, int act, float descale, float alpha,
              const void* res, int64_t ldr, int res_dtype, float out_scale, float* amax,
              int tile, void* stream);
+/* crl_gemm with its columns split over two outputs: columns [0, nsplit) go to C, columns [nsplit, N) to C2 (row stride
+ * ldc2, column n at n - nsplit), both of out_dtype; epilogue descale * acc + bias. This is how the BT4-class layer runs the
+ * q, k, v projections and the 32-column compression of the attention-bias generator as one product over one
+ * concatenated weight (the reference's layers call one nn.Linear per projection, new_paradigm/attn.py:501-503; the
+ * generator follows lc0's smolgen, which the reference does not contain). tile: 0 = automatic, or 3, 7, 10 as in crl_gemm
+ * (same sums and result bits in every case). With e4m3 operands, a 16-bit output of more than 64 MB, M in whole 256-row
+ * tiles, nsplit a multiple of 256 and at most 32 columns behind it, the 256x256 kernel's last tile column computes the
+ * columns of C2 as well instead of a tile column of their own. */
+int crl_gemm_split(const void* A, int64_t lda, const void* W, int64_t ldw, void* C, int64_t ldc, void* C2, int64_t ldc2, int nsplit,
+                   int M, int N, int K, int in_dtype, int out_dtype, const float* bias, float descale, int tile, void* stream);
 /* No counterpart in the reference: crl_gemm with tile = 4 (K cut into slices, a second kernel adds them) for callers that
  * cannot allocate device memory, i.e. code under HIP graph capture, serving loops and harnesses that forbid hipMalloc.
  * The partial sums of the slices go to a fixed array of crl_gemm_static_scratch_bytes() = 8 MB inside the library's

@@ -263,6 +263,42 @@ def test_gemm_guardless_epilogue_instances_equal_general_kernel(cuda, M, N, K):
             assert torch.equal(run_gemm(A, W, kw["out_dt"], tile=11, **args), run_gemm(A, W, kw["out_dt"], tile=12, **args)), (M, N, K, sorted(args))
 
 
+@pytest.mark.parametrize("M,nsplit,extra,K", [(16384, 3072, 32, 1024), (12288, 3072, 16, 1536), (1024, 512, 32, 256), (16640, 3072, 32, 1024), (16384, 3072, 40, 1024)])
+def test_gemm_split_output_last_tile_column_carries_the_columns_behind_it(cuda, M, nsplit, extra, K):
+    """crl_gemm_split: columns [0, nsplit) into C, the rest into C2. Where the 16-bit output passes 64 MB, M is whole tiles
+    and at most 32 columns lie behind a split at a multiple of 256, tile 10 computes them in the workgroups of the last
+    tile column (no tile column of their own); the general kernel (tile 7) and the cases outside those conditions (a small
+    output, 40 columns, a ragged M) give them a tile column. Same sums either way: both outputs bit-equal, and equal to the
+    unsplit product."""
+    torch.manual_seed(M + nsplit + extra + K)
+    N = nsplit + extra
+    A = (torch.randn(M, K, device=cuda) * 30).to(torch.float8_e4m3fn)
+    W = (torch.randn(N, K, device=cuda) * 30).to(torch.float8_e4m3fn)
+    bias = torch.randn(N, device=cuda)
+    ldc2 = 40
+
+    def run(tile, with_bias):
+        C = torch.zeros(M, nsplit, dtype=torch.bfloat16, device=cuda)
+        C2 = torch.full((M, ldc2), 7.0, dtype=torch.bfloat16, device=cuda)
+        check(lib().crl_gemm_split(p(A), K, p(W), K, p(C), nsplit, p(C2), ldc2, nsplit, M, N, K, _lib.FP8, _lib.BF16,
+                                   p(bias) if with_bias else p(None), 1e-3, tile, stream()), "crl_gemm_split")
+        torch.cuda.synchronize()
+        return C, C2
+
+    for with_bias in (False, True):
+        c10, d10 = run(10, with_bias)
+        c7, d7 = run(7, with_bias)
+        c0, d0 = run(0, with_bias)
+        assert torch.equal(c10, c7) and torch.equal(d10, d7), (M, N, K, with_bias, (d10.float() - d7.float()).abs().max().item())
+        assert torch.equal(c0, c7) and torch.equal(d0, d7)
+        assert (d10[:, extra:] == 7.0).all()              # nothing written past the extra columns
+        whole = run_gemm(A, W, _lib.BF16, bias=bias if with_bias else None, descale=1e-3, tile=7)
+        assert torch.equal(whole[:, :nsplit], c10) and torch.equal(whole[:, nsplit:], d10[:, :extra])
+    ref = (A[:512].float() @ W.float().t()) * 1e-3
+    got = torch.cat([c10[:512].float(), d10[:512, :extra].float()], dim=1) - bias
+    assert torch.allclose(got, ref, rtol=2 ** -6, atol=2 ** -6 * ref.abs().max().item())
+
+
 @pytest.mark.parametrize("M,N,K", [(128, 128, 64), (128, 128, 256), (4096, 1024, 1024), (4096, 1536, 1024), (4096, 1024, 1536), (2048, 4096, 256),
                                    (300, 700, 512), (1000, 3104, 1024), (4096, 200, 192), (130, 129, 128), (640, 3104, 1088)])
 @pytest.mark.parametrize("dt", ["bf16", "fp8"])
