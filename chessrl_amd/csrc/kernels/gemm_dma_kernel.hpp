@@ -239,12 +239,10 @@ __global__ void __launch_bounds__(Cfg::NT, 2) gemm_dma_kernel(const GemmArgs a, 
     else wait_vmcnt<0>();
     __syncthreads();
     const bool more = slab + NSTAGE - 1 < nslab;
-    constexpr bool SPREAD = IN_DT == DT_FP8;   // 16-bit operands measure 2-3 % slower with their loads spread out
-    if (!SPREAD && more) issue(slab + NSTAGE - 1);
     prefetch(slab + NSTAGE - 1 + pf);
     const uint8_t* st = smem + (slab % NSTAGE) * Cfg::STAGE_BYTES;
     if (!wave_active) {   // no MFMAs to put the loads between
-      if (SPREAD && more) issue(slab + NSTAGE - 1);
+      if (more) issue(slab + NSTAGE - 1);
       continue;
     }
 #pragma unroll
@@ -256,16 +254,14 @@ __global__ void __launch_bounds__(Cfg::NT, 2) gemm_dma_kernel(const GemmArgs a, 
 #pragma unroll
         for (int tm = 0; tm < TM; ++tm) {
           acc[tn][tm] = mfma_frag<IN_DT>(wf[tn], xf[tm], acc[tn][tm]);
-          // With e4m3 operands the next slab's loads go out one at a time between the MFMAs (after every second one),
-          // held in place by scheduling barriers, instead of eight in a row behind the barrier: a
-          // wave stalls at a load until the memory pipeline takes it, and spread out those stalls fall under MFMAs that
-          // are already executing (measured 1-4 % per GEMM).
-          const int i = tn * TM + tm;
-          constexpr int PER = (TN * TM * KSTEPS) / LOADS >= 1 ? (TN * TM * KSTEPS) / LOADS : 1;
-          if constexpr (SPREAD) if ((i % PER) == PER - 1) {
-            const int j = (ks * TN * TM + i) / PER;
+          // The loads of the slab that follows the ring go out one at a time, one behind each of this slab's first MFMAs,
+          // held in place by scheduling barriers, instead of all in a row behind the barrier (a wave stalls at a load
+          // until the memory pipeline takes it, and spread out those stalls fall under MFMAs that are already
+          // executing) and early enough for the last of them to land under the slab's other MFMAs.
+          const int j = ks * TN * TM + tn * TM + tm;
+          if (j < LOADS) {
             __builtin_amdgcn_sched_barrier(0);
-            if (SPREAD && more && j < LOADS) issue_one(slab + NSTAGE - 1, j);
+            if (more) issue_one(slab + NSTAGE - 1, j);
             __builtin_amdgcn_sched_barrier(0);
           }
         }

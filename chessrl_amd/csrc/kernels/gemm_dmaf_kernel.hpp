@@ -265,8 +265,6 @@ __global__ void __launch_bounds__(DmafCfg::NT, 2) gemm_dmaf_kernel(const GemmArg
       issue_extra(slab + 1, slab + 1 < nslab);
       continue;
     }
-    constexpr bool SPREAD = IN_DT == DT_FP8;   // 16-bit operands measure 2-3 % slower with their loads spread out
-    if constexpr (!SPREAD) static_for<0, LOADS>([&](auto ic) { issue_one(slab + 1, rnext, ic); });
     static_for<0, KSTEPS>([&](auto ksc) {
       constexpr int ks = decltype(ksc)::value;
       Frag<IN_DT> wf[TN], xf[TM];
@@ -284,11 +282,12 @@ __global__ void __launch_bounds__(DmafCfg::NT, 2) gemm_dmaf_kernel(const GemmArg
         constexpr int i = decltype(ic)::value;
         constexpr int tn = i / TM, tm = i % TM;
         acc[tn][tm] = mfma_frag<IN_DT>(wf[tn], xf[tm], acc[tn][tm]);
-        // With e4m3 operands the next slab's loads go out one at a time, one behind each of the slab's first eight MFMAs,
-        // held in place by scheduling barriers: the last of them then has the other eight MFMAs in which to land before
-        // the wave waits for it (spread over all sixteen, one behind every second MFMA, the products of a large pass
-        // take 3.8 % longer; starting one MFMA earlier or two later, or two loads behind each of four MFMAs, 1 %).
-        if constexpr (SPREAD && ks == 0) {
+        // The next slab's loads go out one at a time, one behind each of the slab's first eight MFMAs, held in place by
+        // scheduling barriers: the last of them then has the rest of the slab's MFMAs in which to land before the wave
+        // waits for it. Measured on the products of a large pass, e4m3: spread over all sixteen MFMAs (one behind every
+        // second) +3.8 %, starting one MFMA earlier or two later, or two loads behind each of four MFMAs, +1 %; 16-bit
+        // operands (32 MFMAs per slab): all eight at the head of the slab +2.6 %, behind every second of the first sixteen +2.6 %.
+        if constexpr (ks == 0) {
           __builtin_amdgcn_sched_barrier(0);
           issue_one(slab + 1, rnext, std::integral_constant<int, i>{});
           if constexpr (i == TN * TM - 1) issue_extra(slab + 1, slab + 1 < nslab);
