@@ -14,57 +14,105 @@
 namespace crl {
 
 
+// One workgroup per position, four waves. Each wave takes a quarter of the channels and forms its partial 64x64 product
+// from rows it alone reads (a row's 512 bytes of that quarter are four whole lines; with the channels shared and the
+// output split over the waves instead, every row was fetched by two waves in 32-byte pieces: 2.4 TB/s); the partial
+// tiles meet in LDS and are added in a fixed order, (w0 + w2) + (w1 + w3).
+constexpr int PQK_STRIDE = 68;   // floats per row of a partial tile: 16 lanes' 16-byte stores cover 64 banks
 template <int IN_DT>
 __global__ void __launch_bounds__(256) policy_qk_kernel(const PolicyQKArgs a) {
-  __shared__ float s_a[64 * 65];
+  __shared__ __align__(16) float s_part[2][64 * PQK_STRIDE];
   __shared__ float s_off[8][4];
+  float* const s_a = s_part[0];   // after the sum: the scaled 64x64 tile, row stride 65 (the gather's bank spread)
   const int b = blockIdx.x;
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
   const int lr = lane & 31, g = lane >> 5;
-  const int it = wave & 1, jt = wave >> 1;
-  const uint16_t* qp = reinterpret_cast<const uint16_t*>(a.q) + ((long)b * 64 + 32 * it + lr) * a.ldq + 8 * g;
-  const uint16_t* kp = reinterpret_cast<const uint16_t*>(a.k) + ((long)b * 64 + 32 * jt + lr) * a.ldk + 8 * g;
+  const int kq = a.C / 4;   // channels per wave (the launcher checks C % 64 == 0)
+  const uint16_t* qp = reinterpret_cast<const uint16_t*>(a.q) + ((long)b * 64 + lr) * a.ldq + wave * kq + 8 * g;
+  const uint16_t* kp = reinterpret_cast<const uint16_t*>(a.k) + ((long)b * 64 + lr) * a.ldk + wave * kq + 8 * g;
+  const long q32 = 32 * a.ldq, k32 = 32 * a.ldk;
 
-  f32x16_t acc;
+  f32x16_t acc[2][2];   // [jt][it]
 #pragma unroll
-  for (int r = 0; r < 16; ++r) acc[r] = 0.f;
-  const int steps = a.C / 16;
-#pragma unroll 8
+  for (int jt = 0; jt < 2; ++jt)
+#pragma unroll
+    for (int it = 0; it < 2; ++it)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) acc[jt][it][r] = 0.f;
+  const int steps = kq / 16;
+#pragma unroll 4
   for (int s = 0; s < steps; ++s) {
-    const uint4 qv = *reinterpret_cast<const uint4*>(qp + 16 * s);
-    const uint4 kv = *reinterpret_cast<const uint4*>(kp + 16 * s);
-    if constexpr (IN_DT == DT_BF16)
-      acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, kv), __builtin_bit_cast(bf16x8_t, qv), acc, 0, 0, 0);
-    else
-      acc = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8_t, kv), __builtin_bit_cast(f16x8_t, qv), acc, 0, 0, 0);
+    uint4 qv[2], kv[2];
+#pragma unroll
+    for (int t = 0; t < 2; ++t) {
+      qv[t] = *reinterpret_cast<const uint4*>(qp + t * q32 + 16 * s);
+      kv[t] = *reinterpret_cast<const uint4*>(kp + t * k32 + 16 * s);
+    }
+#pragma unroll
+    for (int jt = 0; jt < 2; ++jt)
+#pragma unroll
+      for (int it = 0; it < 2; ++it) {
+        if constexpr (IN_DT == DT_BF16)
+          acc[jt][it] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, kv[jt]), __builtin_bit_cast(bf16x8_t, qv[it]), acc[jt][it], 0, 0, 0);
+        else
+          acc[jt][it] = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8_t, kv[jt]), __builtin_bit_cast(f16x8_t, qv[it]), acc[jt][it], 0, 0, 0);
+      }
   }
-  // acc[r]: key j = 32jt + 8(r/4) + 4g + r%4, query i = 32it + lr.
-  const int i = 32 * it + lr;
-  if (a.dense) {
+  // acc[jt][it][r]: key j = 32jt + 8(r/4) + 4g + r%4, query i = 32it + lr.
+  // Waves 0 and 1 lay their tiles down, waves 2 and 3 add theirs on top (same lane, same element).
 #pragma unroll
-    for (int rq = 0; rq < 4; ++rq) {
-      const int j = 32 * jt + 8 * rq + 4 * g;
-      float v[4];
+  for (int pass = 0; pass < 2; ++pass) {
+    if ((wave >> 1) == pass) {
 #pragma unroll
-      for (int e = 0; e < 4; ++e) v[e] = acc[4 * rq + e] * a.scale;
-      const long off = (long)b * a.ldd + i * 64 + j;
+      for (int jt = 0; jt < 2; ++jt)
+#pragma unroll
+        for (int it = 0; it < 2; ++it)
+#pragma unroll
+          for (int rq = 0; rq < 4; ++rq) {
+            f32x4_t v4 = {acc[jt][it][4 * rq], acc[jt][it][4 * rq + 1], acc[jt][it][4 * rq + 2], acc[jt][it][4 * rq + 3]};
+            f32x4_t* slot = reinterpret_cast<f32x4_t*>(&s_part[wave & 1][(32 * it + lr) * PQK_STRIDE + 32 * jt + 8 * rq + 4 * g]);
+            if (pass == 1) v4 = *slot + v4;
+            *slot = v4;
+          }
+    }
+    __syncthreads();
+  }
+  // Thread t adds the two sums of row t / 4, columns [16 (t % 4), +16).
+  float tot[16];
+  {
+    const int i = threadIdx.x >> 2, j0 = (threadIdx.x & 3) * 16;
+#pragma unroll
+    for (int c = 0; c < 4; ++c) {
+      const f32x4_t p0 = *reinterpret_cast<const f32x4_t*>(&s_part[0][i * PQK_STRIDE + j0 + 4 * c]);
+      const f32x4_t p1 = *reinterpret_cast<const f32x4_t*>(&s_part[1][i * PQK_STRIDE + j0 + 4 * c]);
+#pragma unroll
+      for (int e = 0; e < 4; ++e) tot[4 * c + e] = (p0[e] + p1[e]) * a.scale;
+    }
+    if (a.dense) {
+      const long off = (long)b * a.ldd + i * 64 + j0;
       if (a.dense_dtype == DT_F32) {
-        *reinterpret_cast<float4*>(reinterpret_cast<float*>(a.dense) + off) = make_float4(v[0], v[1], v[2], v[3]);
-      } else if (a.dense_dtype == DT_BF16) {
-        *reinterpret_cast<uint2*>(reinterpret_cast<uint16_t*>(a.dense) + off) = make_uint2(pack_bf16x2(v[0], v[1]), pack_bf16x2(v[2], v[3]));
+#pragma unroll
+        for (int c = 0; c < 4; ++c)
+          *reinterpret_cast<float4*>(reinterpret_cast<float*>(a.dense) + off + 4 * c) = make_float4(tot[4 * c], tot[4 * c + 1], tot[4 * c + 2], tot[4 * c + 3]);
       } else {
-        *reinterpret_cast<uint2*>(reinterpret_cast<uint16_t*>(a.dense) + off) =
-            make_uint2((uint32_t)f32_to_f16_bits(v[0]) | ((uint32_t)f32_to_f16_bits(v[1]) << 16),
-                       (uint32_t)f32_to_f16_bits(v[2]) | ((uint32_t)f32_to_f16_bits(v[3]) << 16));
+        uint32_t w[8];
+#pragma unroll
+        for (int e = 0; e < 8; ++e)
+          w[e] = a.dense_dtype == DT_BF16 ? pack_bf16x2(tot[2 * e], tot[2 * e + 1])
+                                          : ((uint32_t)f32_to_f16_bits(tot[2 * e]) | ((uint32_t)f32_to_f16_bits(tot[2 * e + 1]) << 16));
+        uint4* dp = reinterpret_cast<uint4*>(reinterpret_cast<uint16_t*>(a.dense) + off);
+        dp[0] = make_uint4(w[0], w[1], w[2], w[3]);
+        dp[1] = make_uint4(w[4], w[5], w[6], w[7]);
       }
     }
   }
   if (!a.logits) return;  // uniform across the workgroup
 
+  __syncthreads();   // every thread has read its partials: their first tile becomes the summed one
+  {
+    const int i = threadIdx.x >> 2, j0 = (threadIdx.x & 3) * 16;
 #pragma unroll
-  for (int r = 0; r < 16; ++r) {
-    const int j = 32 * jt + 8 * (r >> 2) + 4 * g + (r & 3);
-    s_a[i * 65 + j] = acc[r] * a.scale;
+    for (int e = 0; e < 16; ++e) s_a[i * 65 + j0 + e] = tot[e];
   }
   // Promotion offsets from the keys of the promotion rank: tokens 0..7 when white is
   // to move, 56..63 (rank 1) when black is. 32 dot products, 8 threads each.
@@ -77,9 +125,17 @@ __global__ void __launch_bounds__(256) policy_qk_kernel(const PolicyQKArgs a) {
     const float* wrow = a.wpromo + (long)piece * a.C;
     float sum = 0.f;
     if (a.wpromo) {
-      for (int c = part; c < a.C; c += 8) {
-        const float kv = (IN_DT == DT_BF16) ? bf16_bits_to_f32(krow[c]) : f16_bits_to_f32(krow[c]);
-        sum = fmaf(kv, wrow[c], sum);
+      // (eight channels per thread and step: a 16-byte piece of the key row against two vectors of the weight row)
+      for (int c = part * 8; c < a.C; c += 64) {
+        const uint4 kraw = *reinterpret_cast<const uint4*>(krow + c);
+        const float4 w0 = *reinterpret_cast<const float4*>(wrow + c), w1 = *reinterpret_cast<const float4*>(wrow + c + 4);
+        const uint32_t kw[4] = {kraw.x, kraw.y, kraw.z, kraw.w};
+        const float wv[8] = {w0.x, w0.y, w0.z, w0.w, w1.x, w1.y, w1.z, w1.w};
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+          const uint16_t bits = (uint16_t)((e & 1) ? (kw[e >> 1] >> 16) : (kw[e >> 1] & 0xffff));
+          sum = fmaf((IN_DT == DT_BF16) ? bf16_bits_to_f32(bits) : f16_bits_to_f32(bits), wv[e], sum);
+        }
       }
     }
     sum += __shfl_xor(sum, 1, 64);
@@ -100,10 +156,11 @@ __global__ void __launch_bounds__(256) policy_qk_kernel(const PolicyQKArgs a) {
 
 hipError_t launch_policy_qk(const PolicyQKArgs& a, hipStream_t st) {
   if (a.B <= 0) return hipSuccess;
-  if (a.C % 16 || a.ldq % 8 || a.ldk % 8 || (reinterpret_cast<uintptr_t>(a.q) & 15) || (reinterpret_cast<uintptr_t>(a.k) & 15))
+  if (a.C % 64 || a.ldq % 8 || a.ldk % 8 || (reinterpret_cast<uintptr_t>(a.q) & 15) || (reinterpret_cast<uintptr_t>(a.k) & 15))
     return hipErrorInvalidValue;
-  if (a.dense && (a.ldd % 4)) return hipErrorInvalidValue;
+  if (a.dense && ((a.ldd % 8) || (reinterpret_cast<uintptr_t>(a.dense) & 15))) return hipErrorInvalidValue;
   if (a.logits && (!a.gidx || !a.gpromo)) return hipErrorInvalidValue;
+  if (a.wpromo && (reinterpret_cast<uintptr_t>(a.wpromo) & 15)) return hipErrorInvalidValue;
   if (a.in_dtype == DT_BF16) hipLaunchKernelGGL((policy_qk_kernel<DT_BF16>), dim3(a.B), dim3(256), 0, st, a);
   else if (a.in_dtype == DT_F16) hipLaunchKernelGGL((policy_qk_kernel<DT_F16>), dim3(a.B), dim3(256), 0, st, a);
   else return hipErrorInvalidValue;
