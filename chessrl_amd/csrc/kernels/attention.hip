@@ -61,9 +61,12 @@ __device__ __forceinline__ typename H::vec add_bias_h(typename H::vec q, const f
 }
 
 // Waves per workgroup: the relative-shift mode needs a 16.6 KB score patch per wave,
-// so it runs two waves per workgroup to stay inside 64 KB of static LDS.
+// so it runs two waves per workgroup to stay inside 64 KB of static LDS. With a generated bias a workgroup takes eight
+// heads of a position (eight waves): per token row it then reads 512 contiguous bytes of each of q, k and v, its bias is
+// 2 KB pieces of the blocked layout and its e4m3 output rows are two whole lines (measured 9.07 -> 8.53 ms per
+// 4096-position forward against four waves; sixteen waves, one workgroup per CU, 9.71 ms).
 template <int MODE>
-struct AttnWaves { static constexpr int N = MODE == ATTN_RELSHIFT ? 2 : 4; };
+struct AttnWaves { static constexpr int N = MODE == ATTN_RELSHIFT ? 2 : MODE == ATTN_BIAS ? 8 : 4; };
 
 // Waves per SIMD the register allocation is held to (0: the compiler's own choice). The kernel is a chain of load,
 // compute and store phases, so resident waves are what hides its memory latency: at head size 32 with a generated
@@ -83,18 +86,24 @@ __global__ void __launch_bounds__(64 * AttnWaves<MODE>::N, (AttnMinWaves<HS, MOD
   constexpr int NW = AttnWaves<MODE>::N;
   __shared__ __align__(16) uint16_t s_vt[NW][HS * VT_STRIDE];
   __shared__ float s_sp[MODE == ATTN_RELSHIFT ? NW : 1][MODE == ATTN_RELSHIFT ? 64 * SP_STRIDE : 1];
-  // Output tile of the workgroup's NW heads (head size 32, four waves): 64 rows of NW * HS elements, 16 bytes of padding
+  // Output tile of the workgroup's NW heads (head size 32): 64 rows of NW * HS elements, 16 bytes of padding
   // per row. A wave's own output is 64 row pieces of 32 (e4m3) or 64 bytes, which it would have to store 16 bytes per
   // lane and row, a quarter or an eighth of a line at a time; gathered here, the workgroup stores whole lines (measured
   // on 4096 positions x 32 heads in e4m3: the stores were 9 % of the kernel's bytes and 21 % of its time).
-  static_assert(!COOP || (HS == 32 && NW == 4), "the output tile is laid out for four waves of head size 32");
+  static_assert(!COOP || (HS == 32 && (NW == 4 || NW == 8 || NW == 16)), "the output tile is laid out for head size 32");
   constexpr int OSZ = OUT_FP8 ? 1 : 2;
   constexpr int OROW = NW * HS * OSZ, OSTRIDE = OROW + 16;
   __shared__ __align__(16) uint8_t s_out[COOP ? 64 * OSTRIDE : 16];
 
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
   const int lr = lane & 31, g = lane >> 5;
-  const int unit = blockIdx.x * NW + wave;
+  // (workgroup indices go round the eight XCDs: renumbered so that each XCD walks a contiguous range of units)
+  int bid = blockIdx.x;
+  {
+    const int per = gridDim.x >> 3;
+    if (bid < (per << 3)) bid = (bid & 7) * per + (bid >> 3);
+  }
+  const int unit = bid * NW + wave;
   if (unit >= a.B * a.H) return;
   const int b = unit / a.H, h = unit - b * a.H;
   constexpr bool coop = COOP != 0;
@@ -604,7 +613,7 @@ template <int HS, int MODE, int IN_DT>
 static hipError_t launch_attn_dt(const AttnArgs& a, hipStream_t st) {
   constexpr int NW = AttnWaves<MODE>::N;
   const dim3 grid((a.B * a.H + NW - 1) / NW), block(64 * NW);
-  if constexpr (HS == 32 && NW == 4) {
+  if constexpr (HS == 32 && (NW == 4 || NW == 8 || NW == 16)) {
     // Whole workgroups only: H a multiple of 4 puts four heads of one position in every workgroup and leaves none partly
     // filled; 16-byte stores need rows and base aligned to that.
     const int osz = a.out_dtype == DT_FP8 ? 1 : 2;
