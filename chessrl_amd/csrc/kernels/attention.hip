@@ -95,6 +95,9 @@ __global__ void __launch_bounds__(64 * AttnWaves<MODE>::N, (AttnMinWaves<HS, MOD
   constexpr int OROW = NW * HS * OSZ, OSTRIDE = OROW + 16;
   __shared__ __align__(16) uint8_t s_out[COOP ? 64 * OSTRIDE : 16];
 
+  // A wave that starts gets its loads out ahead of its neighbours' arithmetic: raised priority until the score product
+  // begins (which also keeps every load above that point: 8.49 -> 8.31 ms per 4096-position forward).
+  if constexpr (MODE == ATTN_BIAS) __builtin_amdgcn_s_setprio(3);
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
   const int lr = lane & 31, g = lane >> 5;
   // (workgroup indices go round the eight XCDs: renumbered so that each XCD walks a contiguous range of units)
@@ -172,6 +175,7 @@ __global__ void __launch_bounds__(64 * AttnWaves<MODE>::N, (AttnMinWaves<HS, MOD
       kf[t][ks] = *reinterpret_cast<const hvec*>(kp + (long)(32 * t + lr) * a.ldk + 16 * ks + 8 * g);
     }
 
+  if constexpr (MODE == ATTN_BIAS) __builtin_amdgcn_s_setprio(0);
   f32x16_t s[2][2];  // [jt][it]
 #pragma unroll
   for (int jt = 0; jt < 2; ++jt)
