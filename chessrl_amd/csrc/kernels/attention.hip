@@ -115,29 +115,6 @@ __global__ void __launch_bounds__(64 * AttnWaves<MODE>::N, (AttnMinWaves<HS, MOD
   const uint16_t* kp = reinterpret_cast<const uint16_t*>(a.k) + (long)b * 64 * a.ldk + h * HS;
   const uint16_t* vp = reinterpret_cast<const uint16_t*>(a.v) + (long)b * 64 * a.ldv + h * HS;
 
-  // The bias tile is the largest operand (8 KB per wave): request it first so it travels while V is
-  // transposed and the scores are formed.
-  uint4 braw[2][2][2];
-  if constexpr (MODE == ATTN_BIAS) {
-    // Element k = 512 L + 8 lane + e of the unit's 4096 (L = (it, jt, rh)): row-major, or in blocks of 256 units x 128
-    // elements (the layout the bias generator's GEMM writes fastest), where a load of 1 KB is four pieces of 256 bytes.
-    const uint16_t* bp = reinterpret_cast<const uint16_t*>(a.bias);
-    long lstride = 512;
-    if (a.bias_blocked) {
-      bp += (long)(unit >> 8) * (256 * 4096) + ((long)(lane >> 4) * 256 + (unit & 255)) * 128 + ((lane & 15) << 3);
-      lstride = 4 * 256 * 128;
-    } else {
-      bp += (long)unit * 4096 + (lane << 3);
-    }
-#pragma unroll
-    for (int it = 0; it < 2; ++it)
-#pragma unroll
-      for (int jt = 0; jt < 2; ++jt)
-#pragma unroll
-        for (int rh = 0; rh < 2; ++rh)
-          braw[it][jt][rh] = *reinterpret_cast<const uint4*>(bp + ((it * 2 + jt) * 2 + rh) * lstride);
-  }
-
   // ---- V -> V^T in LDS ------------------------------------------------------------
   uint16_t* vt = s_vt[wave];
   {
@@ -174,6 +151,29 @@ __global__ void __launch_bounds__(64 * AttnWaves<MODE>::N, (AttnMinWaves<HS, MOD
       qf[t][ks] = *reinterpret_cast<const hvec*>(qp + (long)(32 * t + lr) * a.ldq + 16 * ks + 8 * g);
       kf[t][ks] = *reinterpret_cast<const hvec*>(kp + (long)(32 * t + lr) * a.ldk + 16 * ks + 8 * g);
     }
+
+  // The bias tile (8 KB per wave), requested behind V, q and k: loads return in the order of their issue, which is now
+  // the order of their use, and all twenty are out before the first of them is waited for.
+  uint4 braw[2][2][2];
+  if constexpr (MODE == ATTN_BIAS) {
+    // Element k = 512 L + 8 lane + e of the unit's 4096 (L = (it, jt, rh)): row-major, or in blocks of 256 units x 128
+    // elements (the layout the bias generator's GEMM writes fastest), where a load of 1 KB is four pieces of 256 bytes.
+    const uint16_t* bp = reinterpret_cast<const uint16_t*>(a.bias);
+    long lstride = 512;
+    if (a.bias_blocked) {
+      bp += (long)(unit >> 8) * (256 * 4096) + ((long)(lane >> 4) * 256 + (unit & 255)) * 128 + ((lane & 15) << 3);
+      lstride = 4 * 256 * 128;
+    } else {
+      bp += (long)unit * 4096 + (lane << 3);
+    }
+#pragma unroll
+    for (int it = 0; it < 2; ++it)
+#pragma unroll
+      for (int jt = 0; jt < 2; ++jt)
+#pragma unroll
+        for (int rh = 0; rh < 2; ++rh)
+          braw[it][jt][rh] = *reinterpret_cast<const uint4*>(bp + ((it * 2 + jt) * 2 + rh) * lstride);
+  }
 
   if constexpr (MODE == ATTN_BIAS) __builtin_amdgcn_s_setprio(0);
   f32x16_t s[2][2];  // [jt][it]
