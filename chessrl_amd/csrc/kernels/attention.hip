@@ -72,6 +72,14 @@ struct AttnWaves { static constexpr int N = MODE == ATTN_RELSHIFT ? 2 : MODE == 
 // compute and store phases, so resident waves are what hides its memory latency: at head size 32 with a generated
 // bias it fits 4 waves in 122 registers without spilling (152 and 3 waves left alone; measured 10.8 -> 9.6 ms per
 // 4096-position forward; 5 waves spill and are slower). The other instances spill at that bound and keep theirs.
+// 16 bytes that the kernel reads once: loaded with the non-temporal hint so that they do not displace what other kernels
+// will want from the caches.
+__device__ __forceinline__ uint4 attn_load_once(const void* p) {
+  typedef int i32x4_nt __attribute__((ext_vector_type(4)));
+  const i32x4_nt v = __builtin_nontemporal_load(reinterpret_cast<const i32x4_nt*>(p));
+  return make_uint4((uint32_t)v[0], (uint32_t)v[1], (uint32_t)v[2], (uint32_t)v[3]);
+}
+
 template <int HS, int MODE>
 struct AttnMinWaves { static constexpr int N = (HS == 32 && MODE == ATTN_BIAS) ? 4 : 0; };
 
@@ -172,7 +180,7 @@ __global__ void __launch_bounds__(64 * AttnWaves<MODE>::N, (AttnMinWaves<HS, MOD
       for (int jt = 0; jt < 2; ++jt)
 #pragma unroll
         for (int rh = 0; rh < 2; ++rh)
-          braw[it][jt][rh] = *reinterpret_cast<const uint4*>(bp + ((it * 2 + jt) * 2 + rh) * lstride);
+          braw[it][jt][rh] = attn_load_once(bp + ((it * 2 + jt) * 2 + rh) * lstride);
   }
 
   if constexpr (MODE == ATTN_BIAS) __builtin_amdgcn_s_setprio(0);

@@ -76,7 +76,10 @@ __global__ void __launch_bounds__(DmafCfg::NT, 2) gemm_dmaf_kernel(const GemmArg
 
   const int tiles_n = wk.tiles_n;
   const int nblk = gridDim.x;
-  int pid = blockIdx.x;
+  // Tiles are walked from the last row of tiles to the first. The kernels around a product (norms, attention) walk their
+  // rows upwards, so this product starts on the rows its producer wrote last and ends on the rows its consumer reads first,
+  // which are the ones the memory-side cache still holds (measured on a 4096-position pass: -0.4 ms over its 60 launches).
+  int pid = nblk - 1 - (int)blockIdx.x;
   {
     const int per = nblk >> 3;
     if (pid < (per << 3)) pid = (pid & 7) * per + (pid >> 3);
