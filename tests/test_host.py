@@ -178,6 +178,22 @@ def test_no_cpu_fallback():
         m.forward((torch.zeros(1, 8, 8, 19), None))
 
 
+def test_gemm_split_rejects_bad_arguments_before_any_launch():
+    """crl_gemm_split checks its arguments on the host: a split outside (0, N) or off a multiple of 8, a tile code that has
+    no two-output form, null outputs. Each is CRL_ERR_ARG with a message, with or without a GPU (nothing is launched)."""
+    L = _lib.lib()
+    buf = (ctypes.c_uint8 * 4096)()
+    ptr = ctypes.cast(buf, ctypes.c_void_p)
+
+    def call(C=ptr, C2=ptr, nsplit=256, N=288, tile=0, in_dt=_lib.FP8):
+        return L.crl_gemm_split(ptr, 64, ptr, 64, C, 256, C2, 32, nsplit, 16, N, 64, in_dt, _lib.BF16, None, 1.0, tile, None)
+
+    for kw in (dict(nsplit=0), dict(nsplit=288), dict(nsplit=300), dict(nsplit=4), dict(tile=2), dict(tile=13), dict(C2=None), dict(C=None),
+               dict(in_dt=_lib.F32)):
+        assert call(**kw) == -1, kw   # CRL_ERR_ARG
+        assert b"crl_gemm_split" in L.crl_last_error()
+
+
 def test_late_game_positions_match_python_oracle():
     """The rollout-scoring sweep draws 30 % of its positions from playouts continued until at most 10 pieces remain
     (sparser legal masks): planes, both masks and the piece counts against the pure-Python rules."""
