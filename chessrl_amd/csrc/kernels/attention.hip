@@ -119,13 +119,39 @@ __global__ void __launch_bounds__(64 * AttnWaves<MODE>::N, (AttnMinWaves<HS, MOD
   const int b = unit / a.H, h = unit - b * a.H;
   constexpr bool coop = COOP != 0;
 
-  const uint16_t* qp = reinterpret_cast<const uint16_t*>(a.q) + (long)b * 64 * a.ldq + h * HS;
-  const uint16_t* kp = reinterpret_cast<const uint16_t*>(a.k) + (long)b * 64 * a.ldk + h * HS;
+  const int qk_hst = a.qk_hstride ? a.qk_hstride : HS;
+  const bool qk_once = a.qk_hstride != 0;   // q and k of a head share lines with nobody else
+  const uint16_t* qp = reinterpret_cast<const uint16_t*>(a.q) + (long)b * 64 * a.ldq + h * qk_hst;
+  const uint16_t* kp = reinterpret_cast<const uint16_t*>(a.k) + (long)b * 64 * a.ldk + h * qk_hst;
   const uint16_t* vp = reinterpret_cast<const uint16_t*>(a.v) + (long)b * 64 * a.ldv + h * HS;
 
   // ---- V -> V^T in LDS ------------------------------------------------------------
   uint16_t* vt = s_vt[wave];
-  {
+  // VPAIR: the two waves of a pair of neighbouring heads (a token's V rows of the two are one whole 128-byte line) take
+  // half the tokens each, for both heads: every line is read by one wave, once, with the non-temporal hint, and lands
+  // transposed in the patch of the head it belongs to; the workgroup meets at a barrier before the second product.
+  constexpr bool VPAIR = COOP != 0 && MODE == ATTN_BIAS && HS == 32 && NW % 2 == 0;
+  if constexpr (VPAIR) {
+    const int half = wave & 1;
+    const uint16_t* vp2 = vp - half * HS;
+    const int dc8 = lane & 7, jq8 = lane >> 3;
+    uint4 rows[4];
+#pragma unroll
+    for (int t = 0; t < 4; ++t) rows[t] = attn_load_once(vp2 + (long)(32 * half + 4 * jq8 + t) * a.ldv + 8 * dc8);
+    uint16_t* vt2 = s_vt[(wave & ~1) + (dc8 >> 2)];
+    const int dc = dc8 & 3, jq = 8 * half + jq8;
+    const uint32_t* w0 = reinterpret_cast<const uint32_t*>(&rows[0]);
+    const uint32_t* w1 = reinterpret_cast<const uint32_t*>(&rows[1]);
+    const uint32_t* w2 = reinterpret_cast<const uint32_t*>(&rows[2]);
+    const uint32_t* w3 = reinterpret_cast<const uint32_t*>(&rows[3]);
+#pragma unroll
+    for (int e2 = 0; e2 < 4; ++e2) {
+      uint2 lo = make_uint2((w0[e2] & 0xffffu) | (w1[e2] << 16), (w2[e2] & 0xffffu) | (w3[e2] << 16));
+      uint2 hi = make_uint2((w0[e2] >> 16) | (w1[e2] & 0xffff0000u), (w2[e2] >> 16) | (w3[e2] & 0xffff0000u));
+      *reinterpret_cast<uint2*>(vt2 + (8 * dc + 2 * e2) * VT_STRIDE + 4 * jq) = lo;
+      *reinterpret_cast<uint2*>(vt2 + (8 * dc + 2 * e2 + 1) * VT_STRIDE + 4 * jq) = hi;
+    }
+  } else {
     constexpr int DC = HS / 8;            // 16-byte chunks per V row
     constexpr int PASSES = (16 * DC) / 64;
 #pragma unroll
@@ -156,8 +182,15 @@ __global__ void __launch_bounds__(64 * AttnWaves<MODE>::N, (AttnMinWaves<HS, MOD
   for (int t = 0; t < 2; ++t)
 #pragma unroll
     for (int ks = 0; ks < KS; ++ks) {
-      qf[t][ks] = *reinterpret_cast<const hvec*>(qp + (long)(32 * t + lr) * a.ldq + 16 * ks + 8 * g);
-      kf[t][ks] = *reinterpret_cast<const hvec*>(kp + (long)(32 * t + lr) * a.ldk + 16 * ks + 8 * g);
+      const uint16_t* qa = qp + (long)(32 * t + lr) * a.ldq + 16 * ks + 8 * g;
+      const uint16_t* ka = kp + (long)(32 * t + lr) * a.ldk + 16 * ks + 8 * g;
+      if (qk_once) {
+        qf[t][ks] = __builtin_bit_cast(hvec, attn_load_once(qa));
+        kf[t][ks] = __builtin_bit_cast(hvec, attn_load_once(ka));
+      } else {
+        qf[t][ks] = *reinterpret_cast<const hvec*>(qa);
+        kf[t][ks] = *reinterpret_cast<const hvec*>(ka);
+      }
     }
 
   // The bias tile (8 KB per wave), requested behind V, q and k: loads return in the order of their issue, which is now
@@ -320,9 +353,13 @@ __global__ void __launch_bounds__(64 * AttnWaves<MODE>::N, (AttnMinWaves<HS, MOD
   }
 
   // ---- O^T = V^T · P^T ------------------------------------------------------------------
-  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-  __builtin_amdgcn_wave_barrier();
-  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+  if constexpr (VPAIR) {
+    __syncthreads();   // (the other wave of the pair wrote half of this head's V^T)
+  } else {
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+  }
   f32x16_t o[DT_TILES][2];
 #pragma unroll
   for (int dt = 0; dt < DT_TILES; ++dt)
@@ -663,7 +700,7 @@ static hipError_t launch_attn_hs(const AttnArgs& a, hipStream_t st) {
 hipError_t launch_attention(const AttnArgs& a, int head_dim, hipStream_t st) {
   if (a.B <= 0) return hipSuccess;
   // 16-byte row-segment loads: strides and bases must be multiples of 8 elements.
-  if (a.ldq % 8 || a.ldk % 8 || a.ldv % 8 || a.ldo % 4 ||
+  if (a.ldq % 8 || a.ldk % 8 || a.ldv % 8 || a.ldo % 4 || a.qk_hstride % 8 || (a.qk_hstride && (a.qk_hstride < head_dim || (a.T != 0 && a.T != 64))) ||
       (reinterpret_cast<uintptr_t>(a.q) & 15) || (reinterpret_cast<uintptr_t>(a.k) & 15) || (reinterpret_cast<uintptr_t>(a.v) & 15))
     return hipErrorInvalidValue;
   if (a.mode == ATTN_BIAS && !a.bias) return hipErrorInvalidValue;

@@ -209,8 +209,10 @@ struct TokenEmbedArgs {
 enum AttnMode : int { ATTN_PLAIN = 0, ATTN_CAUSAL = 1, ATTN_BIAS = 2, ATTN_RELSHIFT = 3 };
 
 struct AttnArgs {
-  const void* q; const void* k; const void* v;  // bf16 or f16, [B*64, ld*] with head h at column h*HS
+  const void* q; const void* k; const void* v;  // bf16 or f16, [B*64, ld*] with head h at column h*HS (q, k: h*qk_hstride if set)
   long ldq, ldk, ldv;
+  int qk_hstride;       // elements between consecutive heads in q and in k; 0 = the head size. 2*HS with k = q + HS: [q_h | k_h] pairs,
+                        // one whole 128-byte line per token and head at head size 32, which the kernel then reads with the non-temporal hint
   const void* bias;     // ATTN_BIAS: bf16 [B,H,4096] in the kernel's register order
   int bias_blocked;     // 1: the [B*H, 4096] bias matrix is stored in blocks of 256 rows x 128 columns (GemmArgs::c_blocked); B*H % 256 == 0
   const void* pos;      // ATTN_RELSHIFT: bf16 [64, H*HS] projected positional table

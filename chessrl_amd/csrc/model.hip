@@ -241,6 +241,19 @@ int Model::finalize() {
       std::vector<float> wq = cat({&w(p + "attention.query_proj.weight"), &w(p + "attention.key_proj.weight"), &w(p + "attention.value_proj.weight")});
       std::vector<float> bq = cat({&w(p + "attention.query_proj.bias"), &w(p + "attention.key_proj.bias"), &w(p + "attention.value_proj.bias")});
       int nq = 3 * C;
+      if (qk_paired()) {
+        // Output columns [q_0 | k_0 | q_1 | k_1 | ...] then v: a head's q and k of one token are one whole 128-byte line.
+        const int hsz = C / cfg.n_head;
+        std::vector<float> wp(wq), bp(bq);
+        for (int h = 0; h < cfg.n_head; ++h)
+          for (int part = 0; part < 2; ++part)
+            for (int r = 0; r < hsz; ++r) {
+              const size_t src = (size_t)part * C + (size_t)h * hsz + r, dst = ((size_t)h * 2 + part) * hsz + r;
+              std::copy(wq.begin() + src * C, wq.begin() + (src + 1) * C, wp.begin() + dst * C);
+              bp[dst] = bq[src];
+            }
+        wq.swap(wp); bq.swap(bp);
+      }
       if (cfg.arch == CRL_ARCH_BT4CLASS) {
         const auto& cw = w(p + "smolgen.compress.weight");
         wq.insert(wq.end(), cw.begin(), cw.end());
@@ -602,7 +615,9 @@ int Model::forward_chunk(const float* planes, const uint8_t* ids, const uint8_t*
       AttnArgs a;
       std::memset(&a, 0, sizeof(a));
       const uint16_t* base = reinterpret_cast<const uint16_t*>(ws.qkv);
-      a.q = base; a.k = base + C; a.v = base + 2 * C; a.ldq = a.ldk = a.ldv = 3 * C;
+      if (!gpt && qk_paired()) { a.q = base; a.k = base + hs; a.qk_hstride = 2 * hs; }
+      else { a.q = base; a.k = base + C; }
+      a.v = base + 2 * C; a.ldq = a.ldk = a.ldv = 3 * C;
       a.bias = bias_tile; a.bias_blocked = bias_blocked ? 1 : 0; a.pos = ly.pos; a.u_bias = ly.u_bias; a.v_bias = ly.v_bias;
       a.out = f8 ? (void*)ws.ao8 : (void*)ws.ao; a.ldo = C; a.out_dtype = f8 ? DT_FP8 : ad;
       a.out_scale = f8 ? act_scale(l, 1) : 1.f; a.amax = am(l, 1);

@@ -48,6 +48,8 @@ struct Workspace {
 struct GOpt;
 
 struct Model {
+  // q and k columns of the concatenated q|k|v weight paired head by head (BT4-class with 64-byte head rows)
+  bool qk_paired() const { return cfg.arch == CRL_ARCH_BT4CLASS && cfg.d_model / cfg.n_head == 32; }
   crl_model_config cfg;
   int vocab = 0;
   bool finalized = false;
