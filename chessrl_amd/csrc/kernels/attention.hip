@@ -17,7 +17,8 @@
 
 namespace crl {
 
-constexpr int VT_STRIDE = 72;   // bf16 elements per V^T row (64 keys + 8 padding)
+constexpr int VT_STRIDE = 68;   // bf16 elements per V^T row (64 keys + 4 padding: rows 8 apart land 16 banks apart, so the transposing
+                                // 8-byte writes and the fragment reads of a wave touch every bank twice, the minimum; with 72 it was eight and four times)
 constexpr int SP_STRIDE = 65;   // floats per row of the positional score patch
 
 // Storage order of a 64x64 bias tile so that each lane reads its accumulator
