@@ -71,6 +71,8 @@ SIGNATURES = {
     "crl_model_set_amax": (_i, [_vp, _vp, _i]),
     "crl_model_forward": (_i, [_vp, _vp, _i, _vp, _vp, _vp]),
     "crl_model_forward_compact": (_i, [_vp, _vp, _vp, _i, _vp, _vp, _vp]),
+    "crl_model_run_layers": (_i, [_vp, _vp, _i, _i, _i, _vp, _vp]),
+    "crl_model_read_tensor": (_i, [_vp, _cp, _vp, _i64, _vp]),
     "crl_model_vocab": (_i, [_vp]),
     "crl_model_flops_per_position": (C.c_double, [_vp]),
     "crl_model_set_profiling": (_i, [_vp, _i]),

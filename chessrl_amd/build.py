@@ -18,8 +18,6 @@ SOURCES = [
     "kernels/gemm.hip",
     "kernels/gemm_dma.hip",
     "kernels/gemm_dma_resnorm.hip",
-    "kernels/gemm_pp.hip",
-    "kernels/gemm_sp.hip",
     "kernels/gemm_sp2.hip",
     "kernels/gemm_dmaf.hip",
     "kernels/gemm_dmam.hip",

@@ -211,7 +211,7 @@ int crl_gemm(const void* A, int64_t lda, const void* W, int64_t ldw, void* C, in
              float out_scale, float* amax, int tile, void* stream) {
   if (!A || !W || !C || M < 0 || N < 0 || K <= 0) return arg_fail("crl_gemm: bad arguments");
   if (in_dtype != DT_BF16 && in_dtype != DT_F16 && in_dtype != DT_FP8) return arg_fail("crl_gemm: in_dtype must be bf16, f16 or fp8");
-  if (out_dtype < 0 || out_dtype > 3 || tile < 0 || tile > 14) return arg_fail("crl_gemm: bad out_dtype or tile");
+  if (out_dtype < 0 || out_dtype > 3 || tile < 0 || tile > 14 || tile == 6 || tile == 8) return arg_fail("crl_gemm: bad out_dtype or tile");
   GemmArgs g;
   std::memset(&g, 0, sizeof(g));
   g.A = A; g.lda = lda; g.W = W; g.ldw = ldw; g.C = C; g.ldc = ldc; g.M = M; g.N = N; g.K = K; g.nsplit = N;
@@ -464,6 +464,8 @@ int crl_model_create(const crl_model_config* cfg, crl_model** out) {
   const int hs = cfg->d_model / cfg->n_head;
   if (hs != 32 && hs != 64) return arg_fail("crl_model_create: head dimension must be 32 or 64");
   if (cfg->d_model % 16 || cfg->d_model > 2048 || cfg->d_ff % 8) return arg_fail("crl_model_create: d_model must be a multiple of 16 up to 2048, d_ff a multiple of 8");
+  if (cfg->arch != CRL_ARCH_GPT64 && cfg->d_model % 64)
+    return arg_fail("crl_model_create: d_model must be a multiple of 64 for CRL_ARCH_BT4 and CRL_ARCH_BT4CLASS (the policy head's product splits the channels over four waves in steps of 16)");
   if (cfg->arch == CRL_ARCH_BT4CLASS) {
     const int sg = cfg->smolgen_gen ? cfg->smolgen_gen : 256, sc = cfg->smolgen_compress ? cfg->smolgen_compress : 32;
     const int sh = cfg->smolgen_hidden ? cfg->smolgen_hidden : 256;
@@ -700,6 +702,14 @@ int crl_model_search_1ply(crl_model* m, const char* const* fens, int n, int chun
     if (best_uci6) put_str(best_uci6 + (size_t)i * 6, 6, move_uci(moves[i][(size_t)pick]));
   }
   return CRL_OK;
+}
+int crl_model_run_layers(crl_model* m, const float* x_in, int B, int first, int last, float* x_out, void* stream) {
+  if (!m) return arg_fail("crl_model_run_layers: null model");
+  return m->impl.run_layers(x_in, B, first, last, x_out, (hipStream_t)stream);
+}
+int crl_model_read_tensor(crl_model* m, const char* name, void* out, int64_t bytes, void* stream) {
+  if (!m) return arg_fail("crl_model_read_tensor: null model");
+  return m->impl.debug_read(name, out, (long)bytes, (hipStream_t)stream);
 }
 int crl_model_vocab(const crl_model* m) { return m ? m->impl.vocab : 0; }
 double crl_model_flops_per_position(const crl_model* m) { return m ? m->impl.flops_per_position() : 0.0; }

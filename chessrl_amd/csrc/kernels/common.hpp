@@ -318,6 +318,8 @@ hipError_t launch_leela_to_rl(const ScatterArgs& a, hipStream_t st);
 hipError_t launch_extract_stm(const float* planes, const uint8_t* flags, uint8_t* white_to_move, int B, hipStream_t st);
 hipError_t launch_fill_f32(float* p, float v, long n, hipStream_t st);
 hipError_t launch_convert(const float* src, void* dst, long n, int dt, float scale, hipStream_t st);
+// {f32, bf16, f16} -> f32
+hipError_t launch_widen(const void* src, int dt, float* dst, long n, hipStream_t st);
 hipError_t launch_kv_store(const void* qkv, void* cache, int B, int T, int Tmax, int C, hipStream_t st);
 // dyn_k (optional, device): the kernels take the token index k from it instead of from their arguments, so one captured
 // graph serves every step: position = 64 + k, keys = 65 + k.

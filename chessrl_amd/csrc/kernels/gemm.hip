@@ -602,14 +602,7 @@ static hipError_t launch_in_out(const GemmArgs& a, int tile, hipStream_t st) {
       if (ks > 1) return launch_splitk<CfgSmallK4, IN_DT, OUT_DT>(a, ks, per, st);
     }
   }
-  if (tile == 6) {
-    if constexpr (IN_DT == DT_FP8 && (OUT_DT == DT_BF16 || OUT_DT == DT_FP8)) return launch_gemm_pp(a, OUT_DT, st);
-    else return hipErrorInvalidValue;
-  }
-  if (tile == 8) {
-    if constexpr (IN_DT == DT_FP8 && (OUT_DT == DT_BF16 || OUT_DT == DT_FP8)) return launch_gemm_sp(a, OUT_DT, st);
-    else return hipErrorInvalidValue;
-  }
+  if (tile == 6 || tile == 8) return hipErrorInvalidValue;   // codes of two retired kernels
   // The 256x256 tile has three kernels. Eight waves in step (gemm_dma_kernel.hpp, tile 7): every operand type, any K. The
   // same with its address arithmetic out of the main loop (gemm_dmaf_kernel.hpp, tile 10): K in whole 128-byte slabs;
   // bit-equal and faster (the GEMMs of a 4096-position e4m3 forward: -4.9 %), so tile 3 means this one where it exists.

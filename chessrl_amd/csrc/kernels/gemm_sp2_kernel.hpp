@@ -30,7 +30,6 @@
 // the loads go through a descriptor of zero length: they move nothing and keep the counts the waits rely on.
 #pragma once
 #include "gemm_dma_kernel.hpp"
-#include "gemm_sp_kernel.hpp"
 
 namespace crl {
 
@@ -45,6 +44,8 @@ struct Sp2Cfg {
   static constexpr int LDS_BYTES = STATS_OFF + NW * 2 * WM * 4;
   static_assert(EPI_BYTES <= RING_BYTES, "the epilogue patches reuse the ring");
 };
+
+__device__ __forceinline__ void sp_barrier() { asm volatile("s_barrier" ::: "memory"); }
 
 // Slot in which fragment f (0..7 = W[f], 8..15 = X[f - 8]) is refilled: for the next slab; slots 0 and 1: for the slab
 // that has just begun.
@@ -175,7 +176,7 @@ __global__ void __launch_bounds__(Sp2Cfg::NT) gemm_sp2_kernel(const GemmArgs a) 
     i32x8_t& dst = is_w ? wf[idx] : xf[idx];
     dst = i32x8_t{lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
   };
-  // The accumulators are pinned to the accumulation registers by the operand constraint (see gemm_sp_kernel.hpp). The
+  // The accumulators are pinned to the accumulation registers by the operand constraint of the inline-assembly MFMAs. The
   // instruction is the e4m3 x e4m3 form (no format modifiers).
   auto mfma = [&](f32x4_t& c, const i32x8_t& w, const i32x8_t& x) {
     asm volatile("v_mfma_f32_16x16x128_f8f6f4 %0, %1, %2, %0" : "+a"(c) : "v"(w), "v"(x));

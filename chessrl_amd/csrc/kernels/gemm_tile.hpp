@@ -519,10 +519,6 @@ hipError_t launch_gemm_dma(const GemmArgs& a, int in_dt, int out_dt, hipStream_t
 // One 256-byte block of zeros per device (gemm.hip): the source of K-tail chunks for the direct-to-LDS loads.
 const uint8_t* device_zeros(hipError_t* err);
 hipError_t launch_gemm_dma_resnorm(const GemmArgs& a, hipStream_t st);   // gemm_dma_resnorm.hip
-// The same tile with the two waves of a SIMD out of step (gemm_pp.hip): e4m3 operands, bf16 or e4m3 output.
-hipError_t launch_gemm_pp(const GemmArgs& a, int out_dt, hipStream_t st);
-// The same tile on four waves of 128x128, software-pipelined inside the wave (gemm_sp.hip): e4m3 operands, bf16 or e4m3 output.
-hipError_t launch_gemm_sp(const GemmArgs& a, int out_dt, hipStream_t st);
 // gemm_dmaf.hip: the eight-wave in-step tile with address arithmetic kept out of the main loop (K in whole 128-byte slabs).
 bool gemm_dmaf_has(int in_dt, int out_dt, bool res_norm);
 hipError_t launch_gemm_dmaf(const GemmArgs& a, int in_dt, int out_dt, hipStream_t st);

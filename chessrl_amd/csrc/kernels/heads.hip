@@ -388,6 +388,20 @@ hipError_t launch_convert(const float* src, void* dst, long n, int dt, float sca
   return hipGetLastError();
 }
 
+__global__ void widen_kernel(const void* src, int dt, float* dst, long n) {
+  const long i = (long)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= n) return;
+  dst[i] = dt == DT_F32 ? reinterpret_cast<const float*>(src)[i]
+         : dt == DT_BF16 ? bf16_bits_to_f32(reinterpret_cast<const uint16_t*>(src)[i])
+                         : f16_bits_to_f32(reinterpret_cast<const uint16_t*>(src)[i]);
+}
+hipError_t launch_widen(const void* src, int dt, float* dst, long n, hipStream_t st) {
+  if (n <= 0) return hipSuccess;
+  if (dt != DT_F32 && dt != DT_BF16 && dt != DT_F16) return hipErrorInvalidValue;
+  hipLaunchKernelGGL(widen_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, st, src, dt, dst, n);
+  return hipGetLastError();
+}
+
 __global__ void fill_f32_kernel(float* p, float v, long n) {
   const long i = (long)blockIdx.x * blockDim.x + threadIdx.x;
   if (i < n) p[i] = v;

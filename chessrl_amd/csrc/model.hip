@@ -520,8 +520,11 @@ int Model::forward_tokens(const float* planes, const uint8_t* ids, const uint8_t
 }
 
 int Model::forward_chunk(const float* planes, const uint8_t* ids, const uint8_t* flags, const int64_t* idx, int t, int mb,
-                         float* policy, float* all_logits, float* wdl, bool calibrate, hipStream_t st) {
+                         float* policy, float* all_logits, float* wdl, bool calibrate, hipStream_t st, const LayerWindow* win) {
   const int C = cfg.d_model, F = cfg.d_ff, H = cfg.n_head, L = cfg.n_layer, hs = C / H;
+  // Layers [l0, l1) of this call: the whole trunk, or the window of run_layers (its input comes from the caller instead of
+  // the embedding, its first layer reads that input as a plain residual and its last one writes the 16-bit output).
+  const int l0 = win ? win->first : 0, l1 = win ? win->last : L;
   const int T = 64 + t;          // tokens per position: the board, then t move tokens (CRL_ARCH_GPT64 only)
   const int M = mb * T;
   const bool f8 = cfg.fp8 && !calibrate && !force_16bit;
@@ -537,7 +540,12 @@ int Model::forward_chunk(const float* planes, const uint8_t* ids, const uint8_t*
 #define RUN(call) do { rc = (call); if (rc) return rc; } while (0)
 
   // ---- embedding
-  {
+  if (win) {
+    const long n = (long)M * C;
+    HIPCHK(launch_convert(win->x_in, ws.x, n, xdt, 1.f, st));
+    if (f8 && !gpt) HIPCHK(launch_convert(win->x_in, ws.x8, n, DT_FP8, act_scale(l0, 0), st));
+    if (sf32p && !f8) HIPCHK(launch_convert(win->x_in, ws.x16, n, ad, 1.f, st));
+  } else {
     EmbedArgs e;
     std::memset(&e, 0, sizeof(e));
     e.planes = planes; e.ids = ids; e.flags = flags;
@@ -561,7 +569,7 @@ int Model::forward_chunk(const float* planes, const uint8_t* ids, const uint8_t*
       HIPCHK(he);
     }
   }
-  if (cfg.arch == CRL_ARCH_BT4CLASS) {
+  if (cfg.arch == CRL_ARCH_BT4CLASS && !win) {
     HIPCHK(launch_extract_stm(planes, flags, ws.stm, mb, st));
   }
 
@@ -574,9 +582,9 @@ int Model::forward_chunk(const float* planes, const uint8_t* ids, const uint8_t*
   const float attn_scale = cfg.arch == CRL_ARCH_BT4 ? 1.0f / std::sqrt((float)C) : 1.0f / std::sqrt((float)hs);
   const float alpha = cfg.arch == CRL_ARCH_BT4CLASS ? std::pow(2.0f * (float)L, -0.25f) : 1.0f;
 
-  for (int l = 0; l < L; ++l) {
+  for (int l = l0; l < l1; ++l) {
     const Layer& ly = layers[l];
-    const bool last = l + 1 == L;
+    const bool last = l + 1 == l1;
     const void* a_in; int a_dt; float a_sc = 1.f;
     if (gpt) {
       // h = LN1(x)
@@ -645,7 +653,7 @@ int Model::forward_chunk(const float* planes, const uint8_t* ids, const uint8_t*
       // takes x or h as its residual re-normalises the un-normalised tensor t in its epilogue, writing in place.
       // With an fp32 stream x, t and h are fp32 and every norm also writes the 16-bit operand copy (x16, h16).
       { GOpt o; o.res = ws.x; o.ldr = C; o.res_dt = xdt; o.alpha = alpha; o.a_scale = f8 ? act_scale(l, 1) : 1.f;
-        if (fold && l > 0) { o.res = ws.t; o.res_stats = ws.st2; o.res_g = layers[l - 1].ln2_g; o.res_b = layers[l - 1].ln2_b; }
+        if (fold && l > l0) { o.res = ws.t; o.res_stats = ws.st2; o.res_g = layers[l - 1].ln2_g; o.res_b = layers[l - 1].ln2_b; }
         RUN(gemm(ly.proj, ao_in, C, ao_dt, ws.t, C, xdt, M, o, st)); }
       RUN(lnorm(ws.t, C, xdt, ly.ln1_g, ly.ln1_b, fold ? nullptr : ws.h, xdt, f8 ? ws.h8 : nullptr, f8 ? act_scale(l, 2) : 1.f, C, M, C, am(l, 2), st,
                 fold ? ws.st1 : nullptr, (sf32p && !f8) ? ws.h16 : nullptr, ad));
@@ -670,22 +678,32 @@ int Model::forward_chunk(const float* planes, const uint8_t* ids, const uint8_t*
     }
   }
 
+  if (win) {
+    HIPCHK(launch_widen(ws.x, gpt ? xdt : hd, win->x_out, (long)M * C, st));
+    return CRL_OK;
+  }
+
   // ---- heads
   if (gpt) {
     // lm_head takes e4m3 operands too in the fp8 model (model_fp8.py:140); its input scale is the first entry of the
     // amax table's last row.
-    const bool f8h = f8 && lm_head.w8 != nullptr;
+    // An uncalibrated head row (a legacy n_layer*5 table was loaded) keeps lm_head on its 16-bit copy.
+    const bool f8h = f8 && lm_head.w8 != nullptr && amax_host[(size_t)L * AMAX_SLOTS] > 0.f;
     const float hsc = f8h ? act_scale(L, 0) : 1.f;
+    // Calibration takes the head's input amax over EVERY token of ln_f: forward_tokens(all_logits) quantises all of them
+    // with this one scale (model_bis.py:189-192), not just the last token that the policy-only forward reads.
+    const bool cal_all = calibrate && !all_logits;
+    if (cal_all) RUN(lnorm(ws.x, C, xdt, lnf_g, lnf_b, ws.h, hd, nullptr, 1.f, C, M, C, am(L, 0), st));
     if (all_logits) {
       // ln_f and lm_head on every token (model_bis.py:189-192, compute_loss=True).
-      RUN(lnorm(ws.x, C, xdt, lnf_g, lnf_b, f8h ? nullptr : ws.h, hd, f8h ? ws.h8 : nullptr, hsc, C, M, C, policy ? nullptr : am(L, 0), st));
+      RUN(lnorm(ws.x, C, xdt, lnf_g, lnf_b, f8h ? nullptr : ws.h, hd, f8h ? ws.h8 : nullptr, hsc, C, M, C, am(L, 0), st));
       GOpt o; o.a_scale = hsc;
       RUN(gemm(lm_head, f8h ? (const void*)ws.h8 : (const void*)ws.h, C, f8h ? DT_FP8 : hd, all_logits, VOCAB_RL, DT_F32, M, o, st));
     }
     if (policy) {
       // ln_f and lm_head on the last token only (model_bis.py:195-196, 369-370).
       const char* last_tok = reinterpret_cast<const char*>(ws.x) + (size_t)(T - 1) * C * dtype_size(xdt);
-      RUN(lnorm(last_tok, (long)T * C, xdt, lnf_g, lnf_b, f8h ? nullptr : ws.hl, hd, f8h ? ws.hl8 : nullptr, hsc, C, mb, C, am(L, 0), st));
+      RUN(lnorm(last_tok, (long)T * C, xdt, lnf_g, lnf_b, f8h ? nullptr : ws.hl, hd, f8h ? ws.hl8 : nullptr, hsc, C, mb, C, nullptr, st));
       GOpt o; o.a_scale = hsc;
       RUN(gemm(lm_head, f8h ? (const void*)ws.hl8 : (const void*)ws.hl, C, f8h ? DT_FP8 : hd, policy, VOCAB_RL, DT_F32, mb, o, st));
     }
@@ -718,6 +736,34 @@ int Model::forward_chunk(const float* planes, const uint8_t* ids, const uint8_t*
   }
   if (cfg.arch == CRL_ARCH_BT4) { GOpt o; RUN(gemm(pol_head, ws.dense, 4096, hd, policy, VOCAB_RL, DT_F32, mb, o, st)); }
 #undef RUN
+  return CRL_OK;
+}
+
+int Model::run_layers(const float* x_in, int B, int first, int last, float* x_out, hipStream_t st) {
+  if (!finalized) { set_error("run_layers: call crl_model_finalize first"); return CRL_ERR_STATE; }
+  if (!x_in || !x_out || B <= 0 || first < 0 || last > cfg.n_layer || first >= last) { set_error("run_layers: bad arguments (0 <= first < last <= n_layer)"); return CRL_ERR_ARG; }
+  if (B > cfg.micro_batch) { set_error("run_layers: at most one micro-batch of positions"); return CRL_ERR_ARG; }
+  int rc = ensure_ws(B);
+  if (rc) return rc;
+  LayerWindow w{first, last, x_in, x_out};
+  float dummy_policy;   // never written: the window returns before the heads
+  return forward_chunk(nullptr, nullptr, nullptr, nullptr, 0, B, &dummy_policy, nullptr, nullptr, false, st, &w);
+}
+
+int Model::debug_read(const char* name, void* out, long bytes, hipStream_t st) {
+  if (!name || !out || bytes < 0 || ws_mb == 0) { set_error("debug_read: bad arguments, or no forward has run yet"); return CRL_ERR_ARG; }
+  const size_t M = (size_t)ws_mb * 64, C = cfg.d_model, F = cfg.d_ff;
+  const std::string n = name;
+  const void* src = nullptr;
+  size_t cap = 0;
+  if (n == "x8") { src = ws.x8; cap = M * C; }
+  else if (n == "h8") { src = ws.h8; cap = M * C; }
+  else if (n == "ao8") { src = ws.ao8; cap = M * C; }
+  else if (n == "f8") { src = ws.f8; cap = M * F; }
+  else if (n == "t") { src = ws.t; cap = M * C * ((cfg.arch != CRL_ARCH_GPT64 && cfg.stream_f32 > 0) ? 4 : 2); }
+  else { set_error("debug_read: unknown tensor " + n); return CRL_ERR_ARG; }
+  if ((size_t)bytes > cap) { set_error("debug_read: " + n + " holds " + std::to_string(cap) + " bytes"); return CRL_ERR_ARG; }
+  HIPCHK(hipMemcpyAsync(out, src, (size_t)bytes, hipMemcpyDeviceToDevice, st));
   return CRL_OK;
 }
 

@@ -47,6 +47,13 @@ struct Workspace {
 
 struct GOpt;
 
+// A run of consecutive encoder layers on a caller-supplied input (Model::run_layers).
+struct LayerWindow {
+  int first, last;
+  const float* x_in;   // device f32 [positions*64, d_model]: input of layer `first`
+  float* x_out;        // device f32, same shape: output of layer `last - 1`
+};
+
 struct Model {
   // q and k columns of the concatenated q|k|v weight paired head by head (BT4-class with 64-byte head rows)
   bool qk_paired() const { return cfg.arch == CRL_ARCH_BT4CLASS && cfg.d_model / cfg.n_head == 32; }
@@ -104,6 +111,12 @@ struct Model {
   int forward_tokens(const float* planes, const uint8_t* ids, const uint8_t* flags, const int64_t* idx, int t, int B, float* policy,
                      float* all_logits, float* wdl, bool calibrate, hipStream_t st);
   int calibrate(const float* planes, int B, hipStream_t st);
+  // Layers [first, last) on x_in (device f32 [B*64, d_model]); x_out receives the output of layer last-1 widened to f32.
+  // The window's first layer takes x_in as its residual as layer 0 takes the embedding, its last layer writes its
+  // normalised output in the 16-bit type as the trunk's last layer does; everything between runs as in forward().
+  int run_layers(const float* x_in, int B, int first, int last, float* x_out, hipStream_t st);
+  // Copies a workspace tensor as the last call left it ("x8", "h8", "ao8", "f8": the e4m3 operand copies; "t") to `out`.
+  int debug_read(const char* name, void* out, long bytes, hipStream_t st);
   // Sequence generation with cached keys/values (model_bis.py:213-263 with rules, 266-311 without): seq [B, steps+1]
   // receives <thinking> and then `steps` sampled tokens; step_out [B, steps, V] (optional) the probabilities of
   // every step, or its logits when out_logits. Runs in the 16-bit element type whatever cfg.fp8 says.
@@ -118,7 +131,7 @@ struct Model {
   int make_lin(Lin& L, const std::vector<float>& W, const std::vector<float>* bias, int N, int K, int dt16, bool fp8, float amax_all = -1.f);
   int ensure_ws(int mb);
   int forward_chunk(const float* planes, const uint8_t* ids, const uint8_t* flags, const int64_t* idx, int t, int mb, float* policy,
-                    float* all_logits, float* wdl, bool calibrate, hipStream_t st);
+                    float* all_logits, float* wdl, bool calibrate, hipStream_t st, const LayerWindow* win = nullptr);
   int gemm(const Lin& L, const void* A, long lda, int in_dt, void* C, long ldc, int out_dt, int M, const GOpt& o, hipStream_t st);
   int lnorm(const void* x, long ldx, int in_dt, const float* g, const float* b, void* out, int out_dt, uint8_t* out8, float scale8,
             long ldo, int rows, int C, float* amax, hipStream_t st, float* stats = nullptr, void* out_b = nullptr, int out_b_dt = DT_BF16,

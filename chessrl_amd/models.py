@@ -220,9 +220,12 @@ class _Engine:
         planes = _as_planes(planes)
         check(lib().crl_model_calibrate(self.handle, _ptr(planes), planes.shape[0], _stream_ptr()), "crl_model_calibrate")
 
-    def get_amax(self, head=False):
+    def get_amax(self, head=None):
         """Activation amax table [n_layer, 5]; with head=True [n_layer + 1, 5], whose last row starts with the amax
-        of lm_head's input."""
+        of lm_head's input. head=None picks the full table for GPT64 (whose lm_head runs in e4m3 and needs that row:
+        a model that receives the short table keeps lm_head in 16 bits) and the short one for the encoders."""
+        if head is None:
+            head = self.cfg.arch == _lib.ARCH_GPT64
         rows = self.n_layer + (1 if head else 0)
         a = np.zeros(rows * 5, np.float32)
         check(lib().crl_model_get_amax(self.handle, a.ctypes.data, a.size), "crl_model_get_amax")
@@ -320,6 +323,24 @@ class _Engine:
             per_root.append(([mraw[6 * (o + c):6 * (o + c) + 6].split(b"\0")[0].decode() for c in range(k)], vals[o:o + k].clone()))
             o += k
         return moves, per_root
+
+    def run_layers(self, x_in, first, last):
+        """Encoder layers [first, last) on a caller-supplied layer input (cuda float32 [B,64,C]) -> output of layer
+        last-1 (cuda float32 [B,64,C])."""
+        if not self.ready:
+            self.finalize()
+        x_in = x_in.to(torch.float32).contiguous()
+        out = torch.empty_like(x_in)
+        check(lib().crl_model_run_layers(self.handle, _ptr(x_in), x_in.shape[0], int(first), int(last), _ptr(out), _stream_ptr()),
+              "crl_model_run_layers")
+        return out
+
+    def read_tensor(self, name, shape, dtype=torch.uint8, device="cuda"):
+        """A workspace tensor as the last call left it (see crl_model_read_tensor)."""
+        out = torch.empty(shape, dtype=dtype, device=device)
+        check(lib().crl_model_read_tensor(self.handle, name.encode(), _ptr(out), out.numel() * out.element_size(), _stream_ptr()),
+              "crl_model_read_tensor")
+        return out
 
     def flops_per_position(self):
         return lib().crl_model_flops_per_position(self.handle)

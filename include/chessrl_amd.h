@@ -55,7 +55,8 @@ const char* crl_last_error(void);
 const char* crl_version(void);
 /* Frees the device memory the library keeps outside any model handle: the 64 MB K-slice workspaces crl_gemm allocates per
  * stream, a 256-byte block of zeros per device and the move maps of crl_leela_to_rl. Call it with no library work in
- * flight; later calls allocate again on demand. Models are freed by crl_model_destroy. */
+ * flight; later calls allocate again on demand. Models are freed by crl_model_destroy. A HIP graph captured from
+ * library calls has those device addresses baked in: destroy or re-capture such graphs after crl_shutdown. */
 void crl_shutdown(void);
 
 /* ------------------------------------------------------------------ host: vocabulary */
@@ -109,13 +110,12 @@ int crl_random_positions(uint64_t seed, int n, int max_plies, double late_fracti
  * LDS. Both are deterministic from launch to launch but differ from 1-3 in summation order. With tile 0, outputs of at
  * most 256 columns whose K is 4 KB or more per row are always K-sliced the same way (a function of N and K alone), so
  * the row-count independence holds for them too. The first K-sliced launch on a stream allocates that stream's
- * workspace: issue it once outside any graph capture. 6-10 name the 256x256 kernels explicitly: 7 = eight waves in
+ * workspace: issue it once outside any graph capture. 7, 9 and 10 name the 256x256 kernels explicitly: 7 = eight waves in
  * step (any K, any operand type), 10 = the same with its address arithmetic kept out of the main loop (K in whole
  * 128-byte slabs; 3 runs this one where it applies), both with the sums and result bits of 1-3; 9 = four
  * software-pipelined waves with 16x16x128 MFMAs (e4m3 operands, whole slabs; what 3 runs from K = 4096 on; these MFMAs
- * add 128 products per instruction instead of 64, so a sum can differ from the others' in its last fp32 bits); 6 = the
- * two waves of a SIMD out of step and 8 = four software-pipelined waves fed in 64-byte pieces (e4m3 operands, bit-equal
- * to 7) exist for measurement and are slower. 9 and 10 fall back to 7 where K is not whole slabs. 11 and 12 name the two
+ * add 128 products per instruction instead of 64, so a sum can differ from the others' in its last fp32 bits); 6 and 8
+ * are not assigned (CRL_ERR_ARG). 9 and 10 fall back to 7 where K is not whole slabs. 11 and 12 name the two
  * 128x128 kernels (same sums and bits as 2): 11 = fed by direct-to-LDS loads through a four-stage ring (whole slabs; what 2
  * runs for at most one tile per CU), 12 = register-staged (any K; 11 hands over to it where K is not whole slabs).
  * 13 and 14 name the kernel for K = 256 e4m3 elements whose workgroups keep 256 rows of A in registers and walk N (the
@@ -220,7 +220,9 @@ int crl_model_finalize(crl_model* m);
 int crl_model_calibrate(crl_model* m, const float* planes, int B, void* stream);
 /* Read / overwrite the activation amax table, float[n_layer*5]: per layer the input of q|k|v, the attention output,
  * the inputs of the two FFN linears and the input of the shared attention-bias generator (BT4-class only, else 0).
- * With n = (n_layer+1)*5 the table carries one more row whose first entry is the amax of lm_head's input (GPT64). */
+ * With n = (n_layer+1)*5 the table carries one more row whose first entry is the amax of lm_head's input (GPT64), taken
+ * by crl_model_calibrate over every token of ln_f. While that entry is 0 (never calibrated, or only the short table was
+ * set) lm_head runs on its 16-bit copy. */
 int crl_model_get_amax(crl_model* m, float* out, int n);
 int crl_model_set_amax(crl_model* m, const float* in, int n);
 /* The forward pass. planes: device f32 [B,64,19] (GPT.forward batch[0] / BT4.forward inp[0]).
@@ -281,6 +283,19 @@ int crl_model_evaluate_fens(crl_model* m, const char* const* fens, int n, int ch
  * sum(n_moves[0..i)) onwards in move-generation order, total <= capacity or the call fails. Not for CRL_ARCH_GPT64. */
 int crl_model_search_1ply(crl_model* m, const char* const* fens, int n, int chunk, float temperature, uint64_t seed,
                           char* best_uci6, int32_t* n_moves, char* moves_uci6, float* values, int64_t capacity, int threads);
+/* Verification hooks with no counterpart in the reference (its layers are nn.Modules one can call one at a time:
+ * new_paradigm/value.py:58-75 EncoderLayer.forward, model_bis.py:110-113 Block.forward). crl_model_run_layers runs encoder
+ * layers [first, last) on a caller-supplied layer input x_in (device f32 [B*64, d_model], at most one micro-batch) and
+ * writes the output of layer last-1 to x_out (device f32, same shape). The window's first layer treats x_in as layer 0
+ * treats the embedding (stored in the model's activation type; for an fp8 model its e4m3 copy is quantised from x_in
+ * directly with that layer's scale), its last layer writes its output in the 16-bit type as the trunk's last layer does,
+ * the layers between run exactly as inside crl_model_forward. A parity test can so hand every layer the oracle's own
+ * input and hold its output to a per-layer bar. crl_model_read_tensor copies one of the workspace tensors the last call
+ * left behind to `out` (device): "x8", "h8", "ao8" (e4m3 [tokens, d_model]: the inputs of q|k|v, of FFN-1 and of the
+ * out-projection), "f8" (e4m3 [tokens, d_ff]: the input of FFN-2), "t" (the un-normalised residual sum in the stream's
+ * type); only the e4m3 copies an fp8 model writes are meaningful. */
+int crl_model_run_layers(crl_model* m, const float* x_in, int B, int first, int last, float* x_out, void* stream);
+int crl_model_read_tensor(crl_model* m, const char* name, void* out, int64_t bytes, void* stream);
 int crl_model_vocab(const crl_model* m);
 /* 2*MAC count of one position through this model (for roofline accounting). */
 double crl_model_flops_per_position(const crl_model* m);

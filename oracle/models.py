@@ -74,6 +74,7 @@ class Fp8Plan:
         self.amax = torch.zeros(n_layer, 5)
         self.head_amax = torch.zeros(1)     # input of lm_head (model_fp8.py:140); addressed as layer == n_layer, slot 0
         self.recording = False
+        self.capture = None                 # a dict collects the e4m3 codes (uint8) of every quantised input by (layer, slot)
 
     def lin(self, x, layer, slot, weight, bias, weight_amax=None):
         """weight_amax: amax of the whole weight tensor when `weight` is a slice of it (padded vocabulary rows)."""
@@ -83,6 +84,8 @@ class Fp8Plan:
             return F.linear(x, weight, bias)
         sx = amax_scale(cell.item())
         sw = amax_scale(weight.abs().max().item() if weight_amax is None else weight_amax)
+        if self.capture is not None:
+            self.capture[(layer, slot)] = (x * sx).clamp(-FP8_MAX, FP8_MAX).to(torch.float8_e4m3fn).view(torch.uint8)
         return F.linear(fp8_quant_dequant(x, sx), fp8_quant_dequant(weight, sw), bias)
 
     def table(self, head=False):
@@ -98,6 +101,38 @@ def _lin(plan, x, layer, slot, mod):
     if plan is None:
         return mod(x)
     return plan.lin(x, layer, slot, mod.weight, mod.bias)
+
+
+class Storage:
+    """Emulation of an implementation that keeps the tensors between its kernels in a 16-bit type while every
+    product accumulates in fp32: each named site is rounded to `dtype` and widened again. Sites of BT4ClassOracle:
+    'w' (every weight matrix), 'stem' (embedding output), 'qkv' (q, k, v and the compression columns), 'smolgen' (the
+    bias generator's hidden tensors and the generated bias), 'probs' (softmax output, the operand of P.V),
+    'attn_out', 'resid' (the un-normalised sums x + alpha*f(x)), 'ln_out' (both norms' outputs), 'ffn_hidden',
+    'heads' (the tensors between the head linears). `sites=None` rounds all of them. Used by the tests to measure what
+    a faithful 16-bit implementation can reach against the fp32 oracle and which site carries the error."""
+
+    SITES = ("w", "stem", "qkv", "smolgen", "probs", "attn_out", "resid", "ln_out", "ffn_hidden", "heads")
+
+    def __init__(self, dtype=torch.bfloat16, sites=None):
+        self.dtype = dtype
+        self.sites = set(self.SITES if sites is None else sites)
+        assert self.sites <= set(self.SITES)
+
+    def __call__(self, site, x):
+        return x.to(self.dtype).to(torch.float32) if site in self.sites else x
+
+    def linear(self, x, mod):
+        """mod(x) with the weight matrix stored in the 16-bit type (the bias stays fp32)."""
+        return F.linear(x, self("w", mod.weight), mod.bias)
+
+
+def _st(store, site, x):
+    return x if store is None else store(site, x)
+
+
+def _slin(store, x, mod):
+    return mod(x) if store is None else store.linear(x, mod)
 
 
 # ------------------------------------------------------------------ shared pieces
@@ -230,21 +265,25 @@ class GPTOracle(nn.Module):
     def forward_last(self, planes, plan=None):
         """planes [B,8,8,19] -> logits [B,1929] of token 63 (model_bis.py:360-370)."""
         x = self._trunk(self.FenEncoder(planes) + self.pe[:64], plan)
+        if plan is not None and plan.recording:
+            # the head's input scale has to cover every token: the per-token logits of forward_tokens (model_bis.py:189-192)
+            # go through the same e4m3 lm_head
+            plan.head_amax[0] = max(plan.head_amax[0].item(), x.abs().max().item())
         return self._head(x[:, -1, :], plan)
 
     @torch.no_grad()
-    def forward_tokens(self, planes, idx, compute_loss=False):
+    def forward_tokens(self, planes, idx, compute_loss=False, plan=None):
         """(planes [B,8,8,19], idx [B,t]) -> (logits, loss, targets) of model_bis.py:171-199."""
         position = self.FenEncoder(planes)
         B, t = idx.shape
         targets = torch.cat((torch.full((B, 64), 1928, dtype=torch.int64), idx), dim=1).roll(-1, dims=1)
         x = torch.cat((position, self.transformer.wte(idx)), dim=1) + self.pe[:64 + t]
-        x = self._trunk(x)
+        x = self._trunk(x, plan)
         if compute_loss:
-            logits = self.lm_head(x)
+            logits = self._head(x, plan)
             loss = F.cross_entropy(logits.view(-1, logits.size(-1)), targets.view(-1), ignore_index=1928)
             return logits, loss, targets
-        return self.lm_head(x[:, [-1], :]), None, targets
+        return self._head(x[:, [-1], :], plan), None, targets
 
 
 def apply_generation_rules(raw):
@@ -432,38 +471,74 @@ class BT4ClassOracle(nn.Module):
         self.value_head = _ValueHead(d_model)
         self.tables = leela_gather_tables(policy_leela)
 
-    @torch.no_grad()
-    def forward_pv(self, planes, plan=None):
-        """planes [B,8,8,19] -> (policy logits [B,1858] in the side-to-move frame, wdl logits [B,3])."""
+    def embed(self, planes):
+        """planes [B,8,8,19] -> x [B,64,C], the input of the first layer."""
         planes = planes.reshape(-1, 64, 19)
-        white = planes[:, 0, 12] > 0.5
-        x = self.ma_gating(self.layernorm1(F.gelu(self.linear1(planes))))
+        return self.ma_gating(self.layernorm1(F.gelu(self.linear1(planes))))
+
+    def layer(self, li, x, plan=None, store=None):
+        """One encoder layer on x [B,64,C] (fp32). plan: the e4m3 emulation; store: the 16-bit storage emulation."""
+        ly = self.layers[li]
         B, T, C = x.shape
         H = self.num_heads
         hs = C // H
         alpha = (2.0 * self.num_layers) ** -0.25 if self.num_layers else 1.0
-        for li, ly in enumerate(self.layers):
-            at, sm = ly.attention, ly.smolgen
-            if plan is None:
-                q, k, v, comp = at.query_proj(x), at.key_proj(x), at.value_proj(x), sm.compress(x)
-            else:
-                # one fused linear over [q;k;v;compress] with a single weight scale
-                w = torch.cat([at.query_proj.weight, at.key_proj.weight, at.value_proj.weight, sm.compress.weight])
-                b = torch.cat([at.query_proj.bias, at.key_proj.bias, at.value_proj.bias, torch.zeros(sm.compress.weight.shape[0])])
-                out = plan.lin(x, li, 0, w, b)
-                q, k, v, comp = out.split([C, C, C, sm.compress.weight.shape[0]], dim=-1)
-            hid = sm.hidden_ln(F.silu(sm.hidden(comp.reshape(B, -1))))
-            gen = sm.gen_from_ln(F.silu(sm.gen_from(hid))).view(B, H, -1)
-            bias = _lin(plan, gen, li, 4, self.smol_weight_gen).view(B, H, 64, 64)
-            q, k, v = (t.view(B, T, H, hs).transpose(1, 2) for t in (q, k, v))
-            score = torch.matmul(q, k.transpose(-2, -1)) / math.sqrt(hs) + bias
-            ctx = torch.matmul(F.softmax(score, -1), v).transpose(1, 2).reshape(B, T, C)
-            x = _norm(ly.norm1, x + alpha * _lin(plan, ctx, li, 1, at.out_proj), self.rms)
-            f = F.mish(_lin(plan, x, li, 2, ly.ff1))
-            x = _norm(ly.norm2, x + alpha * _lin(plan, f, li, 3, ly.ff2), self.rms)
-        wdl = self.value_head(x, F.mish)
-        tok = F.mish(self.policy_tokens_lin(x))
-        qp, kp = self.queries_pol(tok), self.keys_pol(tok)
+        at, sm = ly.attention, ly.smolgen
+        if plan is None:
+            q, k, v, comp = (_slin(store, x, m) for m in (at.query_proj, at.key_proj, at.value_proj, sm.compress))
+        else:
+            # one fused linear over [q;k;v;compress] with a single weight scale
+            w = torch.cat([at.query_proj.weight, at.key_proj.weight, at.value_proj.weight, sm.compress.weight])
+            b = torch.cat([at.query_proj.bias, at.key_proj.bias, at.value_proj.bias, torch.zeros(sm.compress.weight.shape[0])])
+            out = plan.lin(x, li, 0, w, b)
+            q, k, v, comp = out.split([C, C, C, sm.compress.weight.shape[0]], dim=-1)
+        q, k, v, comp = (_st(store, "qkv", t) for t in (q, k, v, comp))
+        hid = _st(store, "smolgen", F.silu(_slin(store, comp.reshape(B, -1), sm.hidden)))
+        hid = _st(store, "smolgen", sm.hidden_ln(hid))
+        gen = _st(store, "smolgen", F.silu(_slin(store, hid, sm.gen_from)))
+        gen = _st(store, "smolgen", sm.gen_from_ln(gen)).view(B, H, -1)
+        if plan is None:
+            bias = _slin(store, gen, self.smol_weight_gen)
+        else:
+            bias = _lin(plan, gen, li, 4, self.smol_weight_gen)
+        bias = _st(store, "smolgen", bias).view(B, H, 64, 64)
+        q, k, v = (t.view(B, T, H, hs).transpose(1, 2) for t in (q, k, v))
+        score = torch.matmul(q, k.transpose(-2, -1)) / math.sqrt(hs) + bias
+        ctx = torch.matmul(_st(store, "probs", F.softmax(score, -1)), v).transpose(1, 2).reshape(B, T, C)
+        ctx = _st(store, "attn_out", ctx)
+        proj = _lin(plan, ctx, li, 1, at.out_proj) if plan is not None else _slin(store, ctx, at.out_proj)
+        x = _st(store, "ln_out", _norm(ly.norm1, _st(store, "resid", x + alpha * proj), self.rms))
+        f = _lin(plan, x, li, 2, ly.ff1) if plan is not None else _slin(store, x, ly.ff1)
+        f = _st(store, "ffn_hidden", F.mish(f))
+        f2 = _lin(plan, f, li, 3, ly.ff2) if plan is not None else _slin(store, f, ly.ff2)
+        return _st(store, "ln_out", _norm(ly.norm2, _st(store, "resid", x + alpha * f2), self.rms))
+
+    @torch.no_grad()
+    def forward_layers(self, x, first, last, plan=None, store=None):
+        """Layers [first, last) on x [B,64,C]."""
+        for li in range(first, last):
+            x = self.layer(li, x, plan, store)
+        return x
+
+    @torch.no_grad()
+    def forward_pv(self, planes, plan=None, store=None):
+        """planes [B,8,8,19] -> (policy logits [B,1858] in the side-to-move frame, wdl logits [B,3])."""
+        planes = planes.reshape(-1, 64, 19)
+        white = planes[:, 0, 12] > 0.5
+        x = _st(store, "stem", self.embed(planes))
+        B, T, C = x.shape
+        x = self.forward_layers(x, 0, self.num_layers, plan, store)
+        return self.heads(x, white, store)
+
+    @torch.no_grad()
+    def heads(self, x, white, store=None):
+        """Trunk output x [B,64,C] and the side to move -> (policy logits [B,1858], wdl logits [B,3])."""
+        B, T, C = x.shape
+        vh = self.value_head
+        v1 = _st(store, "heads", F.mish(_slin(store, x, vh.dense1))).reshape(B, -1)
+        wdl = _slin(store, _st(store, "heads", F.mish(_slin(store, v1, vh.dense2))), vh.dense3)
+        tok = _st(store, "heads", F.mish(_slin(store, x, self.policy_tokens_lin)))
+        qp, kp = _st(store, "heads", _slin(store, tok, self.queries_pol)), _st(store, "heads", _slin(store, tok, self.keys_pol))
         a = torch.matmul(qp, kp.transpose(-2, -1)) / math.sqrt(C)       # [B, from, to]
         w_from, w_to, b_from, b_to, promo = self.tables
         wl = white.unsqueeze(1)

@@ -162,6 +162,11 @@ def test_state_dict_tables_match_library():
         assert set(shapes) - set(exp) <= {"transformer.wte.weight"}
     with pytest.raises(_lib.CrlError):
         models._Engine(_lib.ARCH_GPT64, 2, 250, 8, 1000)      # head dim must be 32 or 64
+    # the attention-policy head of BT4 / BT4-class needs d_model in whole 64s; GPT64 (no such head) takes 96
+    for arch in (_lib.ARCH_BT4, _lib.ARCH_BT4CLASS):
+        with pytest.raises(_lib.CrlError, match="multiple of 64"):
+            models._Engine(arch, 2, 96, 3, 256)
+    models._Engine(_lib.ARCH_GPT64, 1, 96, 3, 384)
     e = models._Engine(_lib.ARCH_GPT64, 1, 256, 8, 1024)
     with pytest.raises(_lib.CrlError):
         _lib.check(_lib.lib().crl_model_set_weight(e.handle, b"nope", None, 0))
