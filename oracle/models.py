@@ -114,10 +114,13 @@ class Storage:
 
     SITES = ("w", "stem", "qkv", "smolgen", "probs", "attn_out", "resid", "ln_out", "ffn_hidden", "heads")
 
-    def __init__(self, dtype=torch.bfloat16, sites=None):
+    def __init__(self, dtype=torch.bfloat16, sites=None, probs_unnormalised=False):
         self.dtype = dtype
         self.sites = set(self.SITES if sites is None else sites)
         assert self.sites <= set(self.SITES)
+        # True: the 'probs' site rounds exp(score - row max) and divides by the fp32 row sum after the product with V
+        # (what a kernel does that normalises its output instead of its probabilities); False: rounds softmax(score).
+        self.probs_unnormalised = probs_unnormalised
 
     def __call__(self, site, x):
         return x.to(self.dtype).to(torch.float32) if site in self.sites else x
@@ -504,7 +507,12 @@ class BT4ClassOracle(nn.Module):
         bias = _st(store, "smolgen", bias).view(B, H, 64, 64)
         q, k, v = (t.view(B, T, H, hs).transpose(1, 2) for t in (q, k, v))
         score = torch.matmul(q, k.transpose(-2, -1)) / math.sqrt(hs) + bias
-        ctx = torch.matmul(_st(store, "probs", F.softmax(score, -1)), v).transpose(1, 2).reshape(B, T, C)
+        if store is not None and store.probs_unnormalised:
+            e = torch.exp(score - score.max(-1, keepdim=True).values)
+            ctx = torch.matmul(_st(store, "probs", e), v) / e.sum(-1, keepdim=True)
+        else:
+            ctx = torch.matmul(_st(store, "probs", F.softmax(score, -1)), v)
+        ctx = ctx.transpose(1, 2).reshape(B, T, C)
         ctx = _st(store, "attn_out", ctx)
         proj = _lin(plan, ctx, li, 1, at.out_proj) if plan is not None else _slin(store, ctx, at.out_proj)
         x = _st(store, "ln_out", _norm(ly.norm1, _st(store, "resid", x + alpha * proj), self.rms))

@@ -716,3 +716,21 @@ def test_fp8_conversion_matches_torch_bit_for_bit(cuda):
     torch.cuda.synchronize()
     assert torch.equal(out8, (out * 5.0).clamp(-448, 448).to(torch.float8_e4m3fn).view(torch.uint8))
     assert (out.abs() * 5.0 > 448).any()          # the sweep reaches the saturating range
+
+
+def test_shutdown_releases_and_later_calls_allocate_again(cuda):
+    """crl_shutdown frees the per-stream K-slice workspaces and the per-device block of zeros (the K-tail source of the
+    256x256 kernels); the next calls allocate them again and give the same bits."""
+    torch.manual_seed(5)
+    A = torch.randn(64, 8192, device=cuda).bfloat16()
+    W = (torch.randn(128, 8192, device=cuda) * 0.05).bfloat16()
+    A2 = (torch.randn(512, 1000, device=cuda) * 20).to(torch.float8_e4m3fn)      # K tail: 1000 is not whole 128-byte slabs
+    W2 = (torch.randn(512, 1000, device=cuda) * 20).to(torch.float8_e4m3fn)
+    before = run_gemm(A, W, _lib.F32, tile=4).clone(), run_gemm(A2, W2, _lib.BF16, descale=1e-3, tile=7).clone()
+    torch.cuda.synchronize()
+    lib().crl_shutdown()
+    after = run_gemm(A, W, _lib.F32, tile=4), run_gemm(A2, W2, _lib.BF16, descale=1e-3, tile=7)
+    assert torch.equal(before[0], after[0]) and torch.equal(before[1], after[1])
+    lib().crl_shutdown()
+    lib().crl_shutdown()      # idempotent
+    assert torch.equal(run_gemm(A, W, _lib.F32, tile=4), before[0])

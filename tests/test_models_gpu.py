@@ -1,6 +1,8 @@
 """Whole-model parity: the HIP forward (through the C ABI) against the CPU fp32 oracle on the same
 seeded positions and weights. Tolerances: WDL max-abs <= 1e-2 and top-1 move agreement >= 99.5 %
-(the benchmark's bf16 bar); logits are also compared as a relative RMS error."""
+(the benchmark's bf16 bar); logits are also compared as a relative RMS error. The full-size 16-bit
+comparisons against torch's own bf16 / f16 forward, the teacher-forced e4m3 layers and the large-batch
+sweep live in test_bt4class_parity_gpu.py."""
 import numpy as np
 import pytest
 import torch
@@ -198,42 +200,6 @@ def full_size_reference():
     return _FULL
 
 
-@pytest.mark.parametrize("act,stream_f32", [("bf16", False), ("f16", False), ("bf16", True), ("f16", True)])
-def test_bt4class_full_size(cuda, act, stream_f32):
-    """The benchmark model at its real size (15 layers, d=1024, 32 heads, FFN 1536) and its benchmark
-    initialisation (normal(0, 0.02), zero biases), 256 positions, with the residual stream in the 16-bit type
-    (default) and in fp32.
-
-    WDL meets the 1e-2 bar everywhere. On THIS initialisation the reference's top-1/top-2 logit gap has a median
-    near 1e-3 against a logit standard deviation of 0.07, so agreement of the arg-max measures rounding noise against
-    near-ties; the test pins the logit error itself, that every position whose reference gap exceeds twice the
-    largest logit error picks the same move, and the agreement each variant reaches."""
-    L, Cm, Fm, H = 15, 1024, 1536, 32
-    ref = full_size_reference()
-    planes, mask, rpol, rwdl = ref["planes"], ref["mask"], ref["rpol"], ref["rwdl"]
-    m = models.BT4Class(L, Cm, Fm, H, act_dtype=act, stream_f32=stream_f32)
-    m.load_state_dict(ref["oracle"].state_dict())
-    pol, wdl = m(planes.to(cuda))
-    pol, wdl = pol.cpu(), wdl.cpu()
-    report("bt4class full size %s stream %s" % (act, "fp32" if stream_f32 else "16-bit"), pol, rpol, mask, wdl, rwdl)
-    neg = (1.0 - mask.float()) * -999.0
-    top2 = (rpol + neg).topk(2, -1).values
-    gap = top2[:, 0] - top2[:, 1]
-    err = (pol - rpol).abs().max().item()
-    same = (pol + neg).argmax(-1) == (rpol + neg).argmax(-1)
-    decisive = gap > 2 * err
-    print("   logit std %.3e, median gap %.3e, max logit error %.3e, decisive positions %d of %d, agreement on them %.4f, overall %.4f"
-          % (rpol.std().item(), gap.median().item(), err, int(decisive.sum()), len(gap),
-             same[decisive].float().mean().item() if decisive.any() else 1.0, same.float().mean().item()))
-    # measured: rel-rms 2.1e-2 / 2.7e-3 / 6.4e-3 / 8.7e-4, WDL 6.2e-3 / 7.8e-4 / 2.0e-3 / 2.3e-4, top-1 74 / 94 / 88 / 98 %
-    bars = {("bf16", False): (3e-2, 1e-2, 0.70), ("f16", False): (4e-3, 2e-3, 0.91),
-            ("bf16", True): (1e-2, 4e-3, 0.85), ("f16", True): (1.5e-3, 1e-3, 0.96)}[(act, stream_f32)]
-    assert rel_rms(pol, rpol) < bars[0]
-    assert (wdl - rwdl).abs().max() <= bars[1]
-    assert bool(same[decisive].all())
-    assert same.float().mean() >= bars[2]
-
-
 @pytest.mark.parametrize("act", ["bf16", "f16"])
 def test_bt4class_heads_only_error(cuda, act):
     """Where the full-size error comes from: the same stem and heads (d=1024, benchmark initialisation) with no trunk
@@ -248,33 +214,6 @@ def test_bt4class_heads_only_error(cuda, act):
     report("bt4class stem + heads only, %s" % act, pol.cpu(), rpol, mask, wdl.cpu(), rwdl)
     assert rel_rms(pol.cpu(), rpol) < (6e-3 if act == "bf16" else 8e-4)
     assert (wdl.cpu() - rwdl).abs().max() <= (4e-3 if act == "bf16" else 5e-4)
-
-
-def test_bt4class_full_size_top1_bar(cuda):
-    """The benchmark's literal bar, top-1 move agreement >= 99.5 % and WDL max-abs <= 1e-2, on the full-size model with
-    weights whose policies are not near-ties: every parameter non-trivial (biases, norm gains, per-square gating), so
-    the tokens differ by square and the reference's top-1/top-2 gap has a median of 5e-3 instead of 8e-4. f16 operands
-    meet the bar with either residual stream; bf16 operands (8 significant bits in every GEMM input) reach 97 % with
-    the fp32 stream and 89 % without, which is what their measured logit error against these gaps gives. Scaling the
-    policy head (logit standard deviation 0.05 -> 6) scales errors and gaps alike and changes none of these figures."""
-    L, Cm, Fm, H = 15, 1024, 1536, 32
-    oracle = om.test_init_(om.BT4ClassOracle(policy_leela, L, Cm, Fm, H), seed=0)
-    planes, mask = positions(256, seed=1, leela=True)
-    rpol, rwdl = oracle.forward_pv(planes)
-    got = {}
-    for act, sf in (("f16", True), ("f16", False), ("bf16", True), ("bf16", False)):
-        m = models.BT4Class(L, Cm, Fm, H, act_dtype=act, stream_f32=sf)
-        m.load_state_dict(oracle.state_dict())
-        pol, wdl = m(planes.to(cuda))
-        pol, wdl = pol.cpu(), wdl.cpu()
-        report("bt4class full size, test weights, %s stream %s" % (act, "fp32" if sf else "16-bit"), pol, rpol, mask, wdl, rwdl)
-        got[(act, sf)] = (top1_agreement(pol, rpol, mask), (wdl - rwdl).abs().max().item())
-        del m
-    assert got[("f16", True)][0] >= 0.995 and got[("f16", True)][1] <= 1e-2        # the literal bar
-    assert got[("f16", False)][0] >= 0.98 and got[("f16", False)][1] <= 1e-2
-    assert got[("bf16", True)][0] >= 0.95 and got[("bf16", True)][1] <= 1e-2
-    assert got[("bf16", False)][0] >= 0.85 and got[("bf16", False)][1] <= 1e-2
-    assert got[("bf16", True)][0] > got[("bf16", False)][0]
 
 
 @pytest.mark.parametrize("B", [1, 8, 64, 256])

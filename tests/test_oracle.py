@@ -410,3 +410,43 @@ def test_rms_norm_matches_library():
         blk.ln_1.bias.data += 1.0
     assert torch.equal(g.forward_last(planes), base)
     assert not torch.allclose(base, om.test_init_(om.GPTOracle(2, 8, 256), 2).forward_last(planes))
+
+
+def test_storage_emulation_sites_and_refactored_layers():
+    """Storage rounds exactly the named sites to the 16-bit type and leaves the rest alone; forward_pv is embed ->
+    forward_layers -> heads; and on a small model the two sites that carry a bf16 implementation's error are the
+    residual sums and the norm outputs (the tensors an fp32 residual stream keeps wide). With
+    CRL_FULL_ATTRIBUTION=1 the same table is printed for the 15 x 1024 benchmark model on 256 positions (minutes)."""
+    import copy
+    import os
+    from chessrl_amd import board
+    x = torch.randn(3, 7) * 5
+    st = om.Storage(torch.bfloat16, ["resid"])
+    assert torch.equal(st("resid", x), x.bfloat16().float()) and st("ln_out", x) is x
+    with pytest.raises(AssertionError):
+        om.Storage(torch.bfloat16, ["nope"])
+    full = os.environ.get("CRL_FULL_ATTRIBUTION") == "1"
+    cfg, n = ((15, 1024, 1536, 32), 256) if full else ((4, 256, 384, 8), 48)
+    o = om.test_init_(om.BT4ClassOracle(policy_leela, *cfg), seed=0)
+    r = board.random_positions(1, n, masks_leela=True)
+    planes, mask = torch.from_numpy(r["planes"]), torch.from_numpy(r["masks_leela"])
+    pol, wdl = o.forward_pv(planes)
+    # the pieces compose to the whole
+    white = planes.reshape(-1, 64, 19)[:, 0, 12] > 0.5
+    p2, w2 = o.heads(o.forward_layers(o.embed(planes), 0, cfg[0]), white)
+    assert torch.equal(p2, pol) and torch.equal(w2, wdl)
+    rel = lambda a, b: ((a - b).pow(2).mean().sqrt() / b.pow(2).mean().sqrt()).item()
+    neg = (1.0 - mask.float()) * -999.0
+    top1 = lambda a: ((a + neg).argmax(-1) == (pol + neg).argmax(-1)).float().mean().item()
+    lit = copy.deepcopy(o).to(torch.bfloat16).forward_pv(planes.bfloat16())[0].float()
+    every = o.forward_pv(planes, store=om.Storage(torch.bfloat16))[0]
+    print("torch.bfloat16 forward: rel-rms %.3e top-1 %.4f; every site rounded: %.3e %.4f" % (rel(lit, pol), top1(lit), rel(every, pol), top1(every)))
+    assert 0.5 * rel(lit, pol) < rel(every, pol) < 1.5 * rel(lit, pol)
+    only = {}
+    for s in om.Storage.SITES:
+        q, w = o.forward_pv(planes, store=om.Storage(torch.bfloat16, [s]))
+        only[s] = rel(q, pol)
+        print("only %-10s rel-rms %.3e  top-1 %.4f  wdl max-abs %.3e" % (s, only[s], top1(q), (w - wdl).abs().max().item()))
+    order = sorted(only, key=only.get, reverse=True)
+    assert set(order[:2]) == {"resid", "ln_out"}
+    assert only["smolgen"] < 0.1 * only["resid"] and only["probs"] < 0.2 * only["resid"]
