@@ -42,6 +42,7 @@ def parse():
     ap.add_argument("--no-latency", action="store_true", help="skip the batch-64 latency leg")
     ap.add_argument("--no-pipeline", action="store_true", help="skip the FEN-strings-to-host-results leg")
     ap.add_argument("--no-bf16-leg", action="store_true", help="skip the bf16 batch-1024 side measurement of the default workload")
+    ap.add_argument("--fp8-heads", action="store_true", help="fp8 workloads: the three per-token head linears in e4m3 as well (off by default)")
     ap.add_argument("--stream-f32", action="store_true", help="keep the residual stream in fp32 (16-bit GEMM operands)")
     ap.add_argument("--act-dtype", default="bf16", choices=["bf16", "f16"], help="16-bit element type of activations and weights")
     ap.add_argument("--calibrate-copy", action="store_true",
@@ -170,6 +171,21 @@ def grpo_rollout(a, torch, models, board, dev):
                       "roofline": None, "cpu_baseline": None}))
 
 
+def host_cpu_counts():
+    """Physical and logical CPU counts of the host as lscpu reports them, plus the CPUs this process may run on."""
+    info = {"usable_by_this_process": len(os.sched_getaffinity(0)) if hasattr(os, "sched_getaffinity") else None}
+    try:
+        import subprocess
+        txt = subprocess.run(["lscpu"], capture_output=True, text=True, timeout=10).stdout
+        field = lambda name: next((l.split(":", 1)[1].strip() for l in txt.splitlines() if l.startswith(name + ":")), None)
+        sockets, cores, threads = field("Socket(s)"), field("Core(s) per socket"), field("Thread(s) per core")
+        info.update(model=field("Model name"), logical=int(field("CPU(s)")) if field("CPU(s)") else None,
+                    physical=int(sockets) * int(cores) if sockets and cores else None, threads_per_core=int(threads) if threads else None)
+    except Exception as e:      # lscpu missing: the counts stay absent rather than guessed
+        info["error"] = str(e)
+    return info
+
+
 def main():
     a = parse()
     if a.gpus != 1:
@@ -196,7 +212,7 @@ def main():
     L, C, F, H = a.layers, 1024, 1536, 32
 
     model = models.BT4Class(L, C, F, H, fp8=fp8, micro_batch=a.micro_batch, act_dtype=a.act_dtype, seed=0,
-                            stream_f32=True if a.stream_f32 else None)
+                            stream_f32=True if a.stream_f32 else None, fp8_heads=True if (fp8 and a.fp8_heads) else None)
     planes = torch.from_numpy(board.random_positions(1, B, late_fraction=late)["planes"]).to(dev)
     if fp8:
         calib = torch.from_numpy(board.random_positions(2, 512)["planes"]).to(dev)
@@ -360,7 +376,7 @@ def main():
         cdt = time.perf_counter() - t1
         cpu = {"value": round(nb * reps / cdt, 2), "unit": "positions/s", "cores": torch.get_num_threads(), "kind": "port",
                "sample": "%d passes of %d positions through the fp32 torch restatement of the same model (oracle/models.py)" % (reps, nb),
-               "logical_cpus": os.cpu_count()}
+               "logical_cpus": os.cpu_count(), "host": host_cpu_counts()}
         # The outputs the timed run left behind (its last step), first 32 positions, against that oracle pass; for the
         # e4m3 model also against the quantise->dequantise oracle with the model's own scale table.
         rr = lambda x, y: float(((x - y).pow(2).mean().sqrt() / y.pow(2).mean().sqrt()).item())
@@ -369,7 +385,9 @@ def main():
                   "wdl_max_abs": round(float((hw - rwdl).abs().max().item()), 5), "finite": bool(torch.isfinite(pol).all() and torch.isfinite(wdl).all())}
         if fp8:
             plan = om.Fp8Plan(L)
-            plan.amax = torch.from_numpy(eng.get_amax().copy())
+            table = torch.from_numpy(eng.get_amax(head=True).copy())
+            plan.amax, plan.head_amax = table[:L].clone(), table[L].clone()
+            plan.heads = bool(table[L, 0] > 0 and table[L, 1] > 0)      # the head linears run in e4m3 exactly when their row is calibrated
             epol, ewdl = oracle.forward_pv(cp, plan)
             parity["vs_fp8_emulation"] = {"policy_rel_rms": round(rr(hp, epol), 5), "wdl_max_abs": round(float((hw - ewdl).abs().max().item()), 5),
                                           "emulation_vs_fp32_policy_rel_rms": round(rr(epol, rpol), 5)}
@@ -392,7 +410,7 @@ def main():
         "ms_per_step": round(ms_per_step, 3), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "fp8" if fp8 else a.act_dtype, "data": "synthetic",
         "config": {"workload": a.workload, "layers": L, "d_model": C, "heads": H, "ffn": F, "batch": B,
-                   "micro_batch": eng.cfg.micro_batch or 4096, "act_dtype": a.act_dtype, "residual_stream": "fp32" if a.stream_f32 else "16-bit", "positions": "seeded random playouts 0-80 plies",
+                   "micro_batch": eng.cfg.micro_batch or 4096, "act_dtype": a.act_dtype, "residual_stream": "fp32" if a.stream_f32 else "16-bit", "head_linears": "e4m3" if (fp8 and a.fp8_heads) else "16-bit", "positions": "seeded random playouts 0-80 plies",
                    "weights": "normal(0,0.02) seed 0", "fp8_calibration_positions": 512 if fp8 else 0},
         "roofline": roofline, "cpu_baseline": cpu, "parity_check": parity, "latency_b64": latency, "fen_pipeline": pipeline,
         "bf16_b1024": bf16_leg,

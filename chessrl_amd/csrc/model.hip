@@ -49,7 +49,7 @@ Model::Model(const crl_model_config& c) : cfg(c) {
   // tri-state switches: 0 picks the default
   if (cfg.stream_f32 == 0) cfg.stream_f32 = cfg.arch == CRL_ARCH_GPT64 ? 1 : -1;
   if (cfg.ln_fold == 0) cfg.ln_fold = 1;
-  if (cfg.fp8_lm_head == 0) cfg.fp8_lm_head = 1;
+  if (cfg.fp8_lm_head == 0) cfg.fp8_lm_head = cfg.arch == CRL_ARCH_GPT64 ? 1 : -1;
   cfg.norm_rms = cfg.norm_rms ? 1 : 0;
   vocab = cfg.arch == CRL_ARCH_BT4CLASS ? VOCAB_LEELA : VOCAB_RL;
   const long C = cfg.d_model, F = cfg.d_ff, L = cfg.n_layer, H = cfg.n_head;
@@ -287,11 +287,17 @@ int Model::finalize() {
         UP(w(p + "smolgen.gen_from_ln.weight"), DT_F32, ly.sm_ln2_g); UP(w(p + "smolgen.gen_from_ln.bias"), DT_F32, ly.sm_ln2_b);
       }
     }
-    LIN(pol_tok, w("policy_tokens_lin.weight"), &w("policy_tokens_lin.bias"), C, C, hd, false);
+    // The reference's fp8 recipe turns every nn.Linear of the model into a te.Linear, the output head included
+    // (model_fp8.py:43,45,90,92,140): in the e4m3 BT4-class model the three head linears that run on every token
+    // (policy_tokens_lin, queries_pol|keys_pol, value_head.dense1) get e4m3 copies too. dense2 and dense3 (one row per
+    // position) stay 16-bit. Off unless asked for (cfg.fp8_lm_head = 1): on the benchmark model it takes 0.6 ms off a
+    // 49 ms pass and adds half again to the policy error against fp32.
+    const bool f8heads = f8 && cfg.arch == CRL_ARCH_BT4CLASS && cfg.fp8_lm_head > 0;
+    LIN(pol_tok, w("policy_tokens_lin.weight"), &w("policy_tokens_lin.bias"), C, C, hd, f8heads);
     {
       std::vector<float> wqk = cat({&w("queries_pol.weight"), &w("keys_pol.weight")});
       std::vector<float> bqk = cat({&w("queries_pol.bias"), &w("keys_pol.bias")});
-      LIN(pol_qk, wqk, &bqk, 2 * C, C, hd, false);
+      LIN(pol_qk, wqk, &bqk, 2 * C, C, hd, f8heads);
     }
     if (cfg.arch == CRL_ARCH_BT4) {
       LIN(pol_head, w("policy_head.weight"), nullptr, VOCAB_RL, 4096, hd, false);
@@ -323,7 +329,7 @@ int Model::finalize() {
       HIPCHK(hipMemcpy(gidx, gi.data(), gi.size() * 2, hipMemcpyHostToDevice));
       HIPCHK(hipMemcpy(gpromo, gp.data(), gp.size(), hipMemcpyHostToDevice));
     }
-    LIN(val1, w("value_head.dense1.weight"), &w("value_head.dense1.bias"), 128, C, hd, false);
+    LIN(val1, w("value_head.dense1.weight"), &w("value_head.dense1.bias"), 128, C, hd, f8heads);
     LIN(val2, w("value_head.dense2.weight"), &w("value_head.dense2.bias"), 128, 8192, hd, false);
     LIN(val3, w("value_head.dense3.weight"), &w("value_head.dense3.bias"), 3, 128, hd, false);
   }
@@ -576,6 +582,12 @@ int Model::forward_chunk(const float* planes, const uint8_t* ids, const uint8_t*
   // BT4-class in e4m3 with bf16 activations: the normalised activations are not written in 16 bits at all (every
   // tile size has the residual-normalising epilogue, so this does not depend on the batch).
   const bool fold = cfg.ln_fold > 0 && f8 && cfg.arch == CRL_ARCH_BT4CLASS && ad == DT_BF16 && !sf32;
+  // e4m3 head linears (BT4-class): the trunk's last norm writes the e4m3 copy the policy-token and value linears read
+  // (scale from the first entry of the amax table's last row), the policy-token linear writes its output in e4m3 for
+  // the query|key linear (second entry). Rows that were never calibrated keep the heads on their 16-bit copies.
+  const bool f8h = f8 && !win && cfg.arch == CRL_ARCH_BT4CLASS && L > 0 && pol_tok.w8 != nullptr && amax_host[(size_t)L * AMAX_SLOTS] > 0.f &&
+                   amax_host[(size_t)L * AMAX_SLOTS + 1] > 0.f;
+  const bool cal_heads = calibrate && cfg.arch == CRL_ARCH_BT4CLASS && L > 0;
   // 16-bit operand copies of x and h (the tensors themselves when the stream is 16-bit)
   void* const x_op = sf32p ? ws.x16 : ws.x;
   void* const h_op = sf32p ? ws.h16 : ws.h;
@@ -671,9 +683,10 @@ int Model::forward_chunk(const float* planes, const uint8_t* ids, const uint8_t*
           if (fold) { o.res = ws.t; o.res_stats = ws.st1; o.res_g = ly.ln1_g; o.res_b = ly.ln1_b; }
           RUN(gemm(ly.ff2, f8 ? (const void*)ws.f8 : (const void*)ws.f, F, ao_dt, ws.t, C, xdt, M, o, st)); }
       }
-      // x = LN2(t); the last layer's output feeds only the heads.
-      RUN(lnorm(ws.t, C, xdt, ly.ln2_g, ly.ln2_b, (fold && !last) ? nullptr : ws.x, last ? hd : xdt, (f8 && !last) ? ws.x8 : nullptr,
-                (f8 && !last) ? act_scale(l + 1, 0) : 1.f, C, M, C, last ? nullptr : am(l + 1, 0), st, (fold && !last) ? ws.st2 : nullptr,
+      // x = LN2(t); the last layer's output feeds only the heads (as an e4m3 copy alone when they run in e4m3).
+      const bool x8_out = f8 && (!last || f8h);
+      RUN(lnorm(ws.t, C, xdt, ly.ln2_g, ly.ln2_b, ((fold && !last) || (last && f8h)) ? nullptr : ws.x, last ? hd : xdt, x8_out ? ws.x8 : nullptr,
+                x8_out ? act_scale(l + 1, 0) : 1.f, C, M, C, (last && !cal_heads) ? nullptr : am(l + 1, 0), st, (fold && !last) ? ws.st2 : nullptr,
                 (sf32p && !f8 && !last) ? ws.x16 : nullptr, ad));
     }
   }
@@ -710,17 +723,25 @@ int Model::forward_chunk(const float* planes, const uint8_t* ids, const uint8_t*
     return CRL_OK;
   }
   const int hact = cfg.arch == CRL_ARCH_BT4 ? ACT_GELU : ACT_MISH;
+  const void* x_head = f8h ? (const void*)ws.x8 : (const void*)ws.x;
+  const int xh_dt = f8h ? DT_FP8 : hd;
+  const float xh_sc = f8h ? act_scale(L, 0) : 1.f;
   if (wdl) {
-    { GOpt o; o.act = hact; RUN(gemm(val1, ws.x, C, hd, ws.v1, 128, hd, M, o, st)); }
+    { GOpt o; o.act = hact; o.a_scale = xh_sc; RUN(gemm(val1, x_head, C, xh_dt, ws.v1, 128, hd, M, o, st)); }
     { GOpt o; o.act = hact; RUN(gemm(val2, ws.v1, 8192, hd, ws.v2, 128, hd, mb, o, st)); }
     { GOpt o; RUN(gemm(val3, ws.v2, 128, hd, wdl, 3, DT_F32, mb, o, st)); }
   }
   {
     GOpt o; o.act = hact;
     if (cfg.arch == CRL_ARCH_BT4) { o.res = pe_head; o.ldr = C; o.res_dt = hd; o.res_rows = 64; }
-    RUN(gemm(pol_tok, ws.x, C, hd, ws.tok, C, hd, M, o, st));
+    o.a_scale = xh_sc;
+    if (f8h) o.out_scale = act_scale(L, 1);
+    if (cal_heads) o.amax = am(L, 1);
+    // (the e4m3 policy tokens take the place of h8, which nothing reads after the trunk)
+    RUN(gemm(pol_tok, x_head, C, xh_dt, f8h ? (void*)ws.h8 : ws.tok, C, f8h ? DT_FP8 : hd, M, o, st));
   }
-  { GOpt o; RUN(gemm(pol_qk, ws.tok, C, hd, ws.pqk, 2 * C, hd, M, o, st)); }
+  { GOpt o; o.a_scale = f8h ? act_scale(L, 1) : 1.f;
+    RUN(gemm(pol_qk, f8h ? (const void*)ws.h8 : (const void*)ws.tok, C, xh_dt, ws.pqk, 2 * C, hd, M, o, st)); }
   {
     PolicyQKArgs p;
     std::memset(&p, 0, sizeof(p));

@@ -222,10 +222,11 @@ class _Engine:
 
     def get_amax(self, head=None):
         """Activation amax table [n_layer, 5]; with head=True [n_layer + 1, 5], whose last row starts with the amax
-        of lm_head's input. head=None picks the full table for GPT64 (whose lm_head runs in e4m3 and needs that row:
-        a model that receives the short table keeps lm_head in 16 bits) and the short one for the encoders."""
+        of lm_head's input (GPT64) or with the amax of the trunk output and of the policy tokens (BT4-class: the inputs
+        of its e4m3 head linears). head=None picks the full table for the models whose heads run in e4m3 (a model that
+        receives the short table keeps its heads in 16 bits) and the short one otherwise."""
         if head is None:
-            head = self.cfg.arch == _lib.ARCH_GPT64
+            head = self.fp8 and (self.cfg.arch == _lib.ARCH_GPT64 or (self.cfg.arch == _lib.ARCH_BT4CLASS and self.cfg.fp8_lm_head > 0))
         rows = self.n_layer + (1 if head else 0)
         a = np.zeros(rows * 5, np.float32)
         check(lib().crl_model_get_amax(self.handle, a.ctypes.data, a.size), "crl_model_get_amax")
@@ -700,13 +701,14 @@ class BT4Class(_ModelBase):
 
     def __init__(self, num_layers=15, d_model=1024, d_ff=1536, num_heads=32, fp8=False, micro_batch=0,
                  head_dtype=None, act_dtype="bf16", compress=32, hidden=256, gen=256, seed=0, stream_f32=None, ln_fold=None,
-                 norm_rms=False):
+                 norm_rms=False, fp8_heads=None):
+        """fp8_heads: with fp8, run policy_tokens_lin, queries_pol|keys_pol and value dense1 in e4m3 too (off by default)."""
         self.num_layers, self.d_model = num_layers, d_model
         self._shapes = bt4_shapes(num_layers, d_model, d_ff, num_heads, True, compress, hidden, gen)
         self._sd = _default_init(self._shapes, seed)
         self._engine = _Engine(_lib.ARCH_BT4CLASS, num_layers, d_model, num_heads, d_ff, fp8=fp8, micro_batch=micro_batch,
                                head_dtype=head_dtype, act_dtype=act_dtype, compress=compress, hidden=hidden, gen=gen,
-                               stream_f32=stream_f32, ln_fold=ln_fold, norm_rms=norm_rms)
+                               stream_f32=stream_f32, ln_fold=ln_fold, norm_rms=norm_rms, fp8_lm_head=fp8_heads)
         self._engine.load(self._sd)
 
     @torch.no_grad()

@@ -201,7 +201,11 @@ typedef struct crl_model_config {
                              in its epilogue. 0 = default (on), -1 = off (every norm writes its 16-bit output). */
   int32_t norm_rms;       /* 1: the norms of the trunk (and GPT64's ln_f) are RMSNorm, x/sqrt(mean(x^2)+eps)*weight; their
                              .bias entries are accepted and ignored. 0 = LayerNorm as in the reference. */
-  int32_t fp8_lm_head;    /* GPT64 with fp8: lm_head runs in e4m3 as well (model_fp8.py:140). 0 = default (on), -1 = 16-bit. */
+  int32_t fp8_lm_head;    /* fp8 models: the output heads run in e4m3 as well, as the reference's recipe quantises every
+                             nn.Linear (model_fp8.py:43,45,90,92,140): lm_head for GPT64; policy_tokens_lin, queries_pol|keys_pol
+                             and value_head.dense1 for BT4-class. 1 = e4m3 heads, -1 = 16-bit heads, 0 = default: on for GPT64
+                             (the reference's fp8 model), off for BT4-class (whose policy is a product of two quantised
+                             projections: its error against fp32 grows by half for about one percent of the pass). */
 } crl_model_config;
 
 /* GPT(config) / BT4(...) constructors (model_bis.py:127-157, new_paradigm/value.py:122-152). */
@@ -220,9 +224,11 @@ int crl_model_finalize(crl_model* m);
 int crl_model_calibrate(crl_model* m, const float* planes, int B, void* stream);
 /* Read / overwrite the activation amax table, float[n_layer*5]: per layer the input of q|k|v, the attention output,
  * the inputs of the two FFN linears and the input of the shared attention-bias generator (BT4-class only, else 0).
- * With n = (n_layer+1)*5 the table carries one more row whose first entry is the amax of lm_head's input (GPT64), taken
- * by crl_model_calibrate over every token of ln_f. While that entry is 0 (never calibrated, or only the short table was
- * set) lm_head runs on its 16-bit copy. */
+ * With n = (n_layer+1)*5 the table carries one more row for the e4m3 head linears: its first entry is the amax of lm_head's
+ * input (GPT64; taken by crl_model_calibrate over every token of ln_f) or of the trunk output that policy_tokens_lin and
+ * value_head.dense1 read (BT4-class), its second entry the amax of the policy tokens that queries_pol|keys_pol read
+ * (BT4-class). While the entries a model needs are 0 (never calibrated, or only the short table was set) its heads run on
+ * their 16-bit copies. */
 int crl_model_get_amax(crl_model* m, float* out, int n);
 int crl_model_set_amax(crl_model* m, const float* in, int n);
 /* The forward pass. planes: device f32 [B,64,19] (GPT.forward batch[0] / BT4.forward inp[0]).

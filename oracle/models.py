@@ -67,18 +67,21 @@ def amax_scale(amax):
 class Fp8Plan:
     """Activation amax table [n_layer, 5]: slot 0 = input of the q/k/v linear, 1 = attention
     output, 2 = input of the first FFN linear, 3 = input of the second FFN linear, 4 = input of the
-    shared attention-bias generator (BT4-class)."""
+    shared attention-bias generator (BT4-class). The head linears are addressed as layer == n_layer:
+    slot 0 = input of lm_head (GPT, model_fp8.py:140) or of the policy-token and value linears
+    (BT4-class), slot 1 = input of the query|key linear of the policy head (BT4-class)."""
 
     def __init__(self, n_layer):
         self.n_layer = n_layer
         self.amax = torch.zeros(n_layer, 5)
-        self.head_amax = torch.zeros(1)     # input of lm_head (model_fp8.py:140); addressed as layer == n_layer, slot 0
+        self.head_amax = torch.zeros(5)     # the head row; addressed as layer == n_layer
         self.recording = False
+        self.heads = False                  # BT4-class: quantise the head linears too (their row of the table must be recorded)
         self.capture = None                 # a dict collects the e4m3 codes (uint8) of every quantised input by (layer, slot)
 
     def lin(self, x, layer, slot, weight, bias, weight_amax=None):
         """weight_amax: amax of the whole weight tensor when `weight` is a slice of it (padded vocabulary rows)."""
-        cell = self.head_amax[0:1] if layer == self.n_layer else self.amax[layer, slot:slot + 1]
+        cell = self.head_amax[slot:slot + 1] if layer == self.n_layer else self.amax[layer, slot:slot + 1]
         if self.recording:
             cell[0] = max(cell.item(), x.abs().max().item())
             return F.linear(x, weight, bias)
@@ -92,9 +95,7 @@ class Fp8Plan:
         """numpy [n_layer, 5], or [n_layer + 1, 5] with the lm_head row appended (the library's layout)."""
         if not head:
             return self.amax.numpy().copy()
-        last = torch.zeros(1, 5)
-        last[0, 0] = self.head_amax[0]
-        return torch.cat([self.amax, last]).numpy()
+        return torch.cat([self.amax, self.head_amax.view(1, 5)]).numpy()
 
 
 def _lin(plan, x, layer, slot, mod):
@@ -536,17 +537,30 @@ class BT4ClassOracle(nn.Module):
         x = _st(store, "stem", self.embed(planes))
         B, T, C = x.shape
         x = self.forward_layers(x, 0, self.num_layers, plan, store)
-        return self.heads(x, white, store)
+        return self.heads(x, white, store, plan if (plan is not None and plan.heads) else None)
 
     @torch.no_grad()
-    def heads(self, x, white, store=None):
-        """Trunk output x [B,64,C] and the side to move -> (policy logits [B,1858], wdl logits [B,3])."""
+    def heads(self, x, white, store=None, plan=None):
+        """Trunk output x [B,64,C] and the side to move -> (policy logits [B,1858], wdl logits [B,3]). With an e4m3
+        plan the three head linears that run on every token are quantised like the trunk's (the reference's recipe
+        turns every nn.Linear into a te.Linear, model_fp8.py:43,45,90,92,140): policy_tokens_lin and value dense1 share
+        the quantised trunk output, queries_pol and keys_pol are one linear over one concatenated weight."""
         B, T, C = x.shape
         vh = self.value_head
-        v1 = _st(store, "heads", F.mish(_slin(store, x, vh.dense1))).reshape(B, -1)
+        nl = self.num_layers
+        if plan is None:
+            v1 = F.mish(_slin(store, x, vh.dense1))
+            tok = F.mish(_slin(store, x, self.policy_tokens_lin))
+            qp, kp = _slin(store, tok, self.queries_pol), _slin(store, tok, self.keys_pol)
+        else:
+            v1 = F.mish(plan.lin(x, nl, 0, vh.dense1.weight, vh.dense1.bias))
+            tok = F.mish(plan.lin(x, nl, 0, self.policy_tokens_lin.weight, self.policy_tokens_lin.bias))
+            wqk = torch.cat([self.queries_pol.weight, self.keys_pol.weight])
+            bqk = torch.cat([self.queries_pol.bias, self.keys_pol.bias])
+            qp, kp = plan.lin(tok, nl, 1, wqk, bqk).split([C, C], dim=-1)
+        v1 = _st(store, "heads", v1).reshape(B, -1)
         wdl = _slin(store, _st(store, "heads", F.mish(_slin(store, v1, vh.dense2))), vh.dense3)
-        tok = _st(store, "heads", F.mish(_slin(store, x, self.policy_tokens_lin)))
-        qp, kp = _st(store, "heads", _slin(store, tok, self.queries_pol)), _st(store, "heads", _slin(store, tok, self.keys_pol))
+        tok, qp, kp = (_st(store, "heads", t) for t in (tok, qp, kp))
         a = torch.matmul(qp, kp.transpose(-2, -1)) / math.sqrt(C)       # [B, from, to]
         w_from, w_to, b_from, b_to, promo = self.tables
         wl = white.unsqueeze(1)

@@ -724,8 +724,8 @@ def test_shutdown_releases_and_later_calls_allocate_again(cuda):
     torch.manual_seed(5)
     A = torch.randn(64, 8192, device=cuda).bfloat16()
     W = (torch.randn(128, 8192, device=cuda) * 0.05).bfloat16()
-    A2 = (torch.randn(512, 1000, device=cuda) * 20).to(torch.float8_e4m3fn)      # K tail: 1000 is not whole 128-byte slabs
-    W2 = (torch.randn(512, 1000, device=cuda) * 20).to(torch.float8_e4m3fn)
+    A2 = (torch.randn(512, 1072, device=cuda) * 20).to(torch.float8_e4m3fn)      # K tail: 1072 bytes are not whole 128-byte slabs
+    W2 = (torch.randn(512, 1072, device=cuda) * 20).to(torch.float8_e4m3fn)
     before = run_gemm(A, W, _lib.F32, tile=4).clone(), run_gemm(A2, W2, _lib.BF16, descale=1e-3, tile=7).clone()
     torch.cuda.synchronize()
     lib().crl_shutdown()

@@ -386,7 +386,7 @@ def test_fp8_plan_linear_is_quantise_dequantise_matmul():
     plan.lin(x, 1, 2, w, b)
     plan.lin(x * 2, 2, 0, w, None)            # layer == n_layer: the lm_head cell
     plan.recording = False
-    assert plan.amax[1, 2].item() == x.abs().max().item() and plan.head_amax[0].item() == (2 * x).abs().max().item()
+    assert plan.amax[1, 2].item() == x.abs().max().item() and plan.head_amax[0].item() == (2 * x).abs().max().item() and plan.head_amax[1:].abs().max().item() == 0
     assert plan.table(head=True).shape == (3, 5) and plan.table(head=True)[2, 0] == plan.head_amax[0].item()
     q = lambda t, s: torch.tensor([_nearest_even(v, pos) for v in (t * s).flatten().tolist()]).view_as(t) / s
     sx, sw = 448.0 / x.abs().max().item(), 448.0 / w.abs().max().item()
