@@ -342,6 +342,14 @@ int crl_masked_nll_mean(const float* logp, const int64_t* target, int64_t ignore
  * TFLOP/s and the shader clock in GHz the kernel ran at. Synchronises the stream. */
 int crl_probe_mfma(int dtype, int random_bits, int iters, double* tflops, double* ghz, void* stream);
 
+/* Measurement probe with no counterpart in the reference: would the memory-bound kernels of a pass overlap with its
+ * products if the two ran on disjoint sets of CUs? Two streams with CU masks (gemm_cus of the 256 CUs for the e4m3
+ * product rows x 1024 x 1024, the rest for the trunk LayerNorm over `rows` rows of 1024) are timed alone on all CUs, alone on
+ * their share and side by side. out8: product us/launch on all CUs, on its share, beside the norm; norm us/launch on all
+ * CUs, on its share, beside the product; wall time of the side-by-side run in ms; the same launches back to back on all
+ * CUs in ms. Allocates its own operands; synchronises the device. */
+int crl_probe_cu_split(int gemm_cus, int rows, int iters, double* out8);
+
 #ifdef __cplusplus
 }
 #endif
