@@ -27,7 +27,7 @@ TRAFFIC_BYTES = {
     "bt4class_fp8_b4096": (1.46e9, "profiles/bench_bt4class_fp8_b4096_pmc_mfma_and_traffic.md"),
 }
 WORKLOADS = ["bt4class_fp8_b4096", "bt4class_bf16_b1024", "bt4class_fp8_b8192", "bt4class_fp8_b16384", "bt4class_bf16_b8192",
-             "bt4class_bf16_b16384", "grpo_scoring_gpt6x768_g8_b16_t256", "grpo_rollout_gpt6x768_g8_b16_t256"]
+             "bt4class_bf16_b16384", "bt4class_bf16_latency", "grpo_scoring_gpt6x768_g8_b16_t256", "grpo_rollout_gpt6x768_g8_b16_t256"]
 
 
 def parse():
@@ -95,6 +95,52 @@ def gemm_probe(a, torch, _lib, dev):
     print(json.dumps({"metric": "one GEMM product", "M": M, "N": N, "K": K, "operands": a.gemm_in, "tile": a.gemm_tile,
                       "vendor_yardstick": bool(a.gemm_vendor), "us_per_launch": round(us, 1), "tflops": round(2.0 * M * N * K / us / 1e6, 1),
                       "launches": a.steps + 3}))
+
+
+def latency_workload(a, torch, models, board, dev):
+    """Leaf-evaluation latency of the full-size bf16 model (BASELINE's MCTS mode): batches of 1, 8, 64 and 256 positions from
+    one seeded stream, each with its legal-move mask applied before the softmax; per batch size p50/p99 of a synchronous
+    evaluate call, and the kernel launches of one forward pass."""
+    model = models.BT4Class(15, 1024, 1536, 32, fp8=False, act_dtype=a.act_dtype, seed=0)
+    r = board.random_positions(3, 256, masks_leela=True)
+    planes, masks = torch.from_numpy(r["planes"]).to(dev), torch.from_numpy(r["masks_leela"]).to(dev)
+    per_batch = {}
+    for nb in (1, 8, 64, 256):
+        lp, lm = planes[:nb].contiguous(), masks[:nb].contiguous()
+        ts = []
+        for i in range(a.warmup + max(a.steps, 50)):
+            torch.cuda.synchronize()
+            t1 = time.perf_counter()
+            model.evaluate(lp, legal_mask=lm, T=1.0, want_probs=True)
+            torch.cuda.synchronize()
+            ts.append((time.perf_counter() - t1) * 1e3)
+        ts = sorted(ts[a.warmup:])
+        model._engine.set_profiling(True)
+        model._engine.forward(lp)
+        prof = model._engine.get_profile()
+        model._engine.set_profiling(False)
+        # (the per-family counters do not see the two launches outside them: the side-to-move extraction and the masked softmax)
+        per_batch["b%d" % nb] = {"p50_ms": round(ts[len(ts) // 2], 3), "p99_ms": round(ts[min(len(ts) - 1, int(len(ts) * 0.99))], 3),
+                                 "samples": len(ts), "launches_per_forward": sum(v["launches"] for v in prof.values()) + 2}
+    # the opt-in mode for tiny batches: K spread over more waves (a position's bits then depend on its batch)
+    kp = models.BT4Class(15, 1024, 1536, 32, fp8=False, act_dtype=a.act_dtype, seed=0, small_batch_k_parallel=True)
+    for nb in (1, 8):
+        lp, lm = planes[:nb].contiguous(), masks[:nb].contiguous()
+        ts = []
+        for i in range(a.warmup + max(a.steps, 50)):
+            torch.cuda.synchronize()
+            t1 = time.perf_counter()
+            kp.evaluate(lp, legal_mask=lm, T=1.0, want_probs=True)
+            torch.cuda.synchronize()
+            ts.append((time.perf_counter() - t1) * 1e3)
+        ts = sorted(ts[a.warmup:])
+        per_batch["b%d" % nb]["k_parallel_p50_ms"] = round(ts[len(ts) // 2], 3)
+    b64 = per_batch["b64"]
+    print(json.dumps({"metric": "p50 latency of one evaluate call, BT4-class bf16 b64 with legal-masked softmax", "value": b64["p50_ms"], "unit": "ms",
+                      "n_gpus": 1, "steps": max(a.steps, 50), "warmup": a.warmup, "ms_per_step": b64["p50_ms"], "higher_is_better": False,
+                      "scaling": "weak", "vs_baseline": None, "dtype": a.act_dtype, "data": "synthetic",
+                      "config": {"workload": a.workload, "layers": 15, "d_model": 1024, "heads": 32, "ffn": 1536, "batches": [1, 8, 64, 256]},
+                      "latency": per_batch, "roofline": None, "cpu_baseline": None}))
 
 
 def grpo_scoring(a, torch, models, board, dev):
@@ -216,6 +262,8 @@ def main():
         return
     if a.gemm:
         return gemm_probe(a, torch, _lib, dev)
+    if a.workload == "bt4class_bf16_latency":
+        return latency_workload(a, torch, models, board, dev)
     if a.workload.startswith("grpo_scoring"):
         return grpo_scoring(a, torch, models, board, dev)
     if a.workload.startswith("grpo_rollout"):
@@ -401,7 +449,7 @@ def main():
             plan = om.Fp8Plan(L)
             table = torch.from_numpy(eng.get_amax(head=True).copy())
             plan.amax, plan.head_amax = table[:L].clone(), table[L].clone()
-            plan.heads = bool(table[L, 0] > 0 and table[L, 1] > 0)      # the head linears run in e4m3 exactly when their row is calibrated
+            plan.heads = bool(a.fp8_heads)      # the emulation quantises the head linears exactly when the model does
             epol, ewdl = oracle.forward_pv(cp, plan)
             parity["vs_fp8_emulation"] = {"policy_rel_rms": round(rr(hp, epol), 5), "wdl_max_abs": round(float((hw - ewdl).abs().max().item()), 5),
                                           "emulation_vs_fp32_policy_rel_rms": round(rr(epol, rpol), 5)}

@@ -450,7 +450,10 @@ int Model::gemm(const Lin& L, const void* A, long lda, int in_dt, void* C, long 
   g.amax = o.amax; g.M = M; g.N = L.N; g.K = L.K; g.act = o.act;
   g.res_stats = o.res_stats; g.res_gamma = o.res_g; g.res_beta = cfg.norm_rms ? nullptr : o.res_b;
   g.descale = in_dt == DT_FP8 ? 1.f / (o.a_scale * L.wscale) : 1.f;
-  g.alpha = o.alpha; g.out_scale = o.out_scale; g.k_parallel = o.k_parallel ? 1 : 0;
+  g.alpha = o.alpha; g.out_scale = o.out_scale;
+  // Few rows: K spread over more waves (another summation order; the token steps of generation always, the forward pass
+  // only where the model was told that a position's bits may depend on the batch it travels in).
+  g.k_parallel = (o.k_parallel || (cfg.small_batch_k_parallel > 0 && M <= 512 && !o.res_stats)) ? 1 : 0;
   g.splitk_ws = ws.splitk; g.splitk_ws_bytes = Workspace::SPLITK_BYTES;
   if (o.ln_out) {
     g.nsplit = g.N;
