@@ -49,7 +49,7 @@ def parse():
                     help="also run three 1 GiB device copies, a kernel of known traffic to scale profiler byte counters with")
     ap.add_argument("--cu-split", default="", metavar="CUS[,CUS...]",
                     help="instead of a workload: for each CU count, time an e4m3 trunk product on that many CUs beside the trunk LayerNorm on the "
-                         "rest (two CU-masked streams; crl_probe_cu_split) and print one JSON line")
+                         "rest (two CU-masked streams; 256 = two plain streams; crl_probe_cu_split; --gemm-tile picks the product's kernel) and print one JSON line")
     ap.add_argument("--gemm", default="", metavar="M,N,K",
                     help="instead of a workload: time one crl_gemm product (3 warm-up + --steps launches, Gaussian operands) and print one JSON line")
     ap.add_argument("--gemm-tile", type=int, default=0, help="tile code of crl_gemm for --gemm (0 = the library's choice)")
@@ -253,8 +253,8 @@ def main():
         rows = []
         for cus in [int(v) for v in a.cu_split.split(",")]:
             out = (ct.c_double * 8)()
-            _lib.check(_lib.lib().crl_probe_cu_split(cus, 131072, max(a.steps, 10), out), "crl_probe_cu_split")
-            rows.append({"gemm_cus": cus, "norm_cus": 256 - cus,
+            _lib.check(_lib.lib().crl_probe_cu_split(cus, a.gemm_tile, 131072, max(a.steps, 10), out), "crl_probe_cu_split")
+            rows.append({"gemm_cus": cus, "norm_cus": 256 - cus if cus < 256 else 256, "gemm_tile": a.gemm_tile,
                          "gemm_us": {"all_cus": round(out[0], 1), "own_share": round(out[1], 1), "beside_norm": round(out[2], 1)},
                          "norm_us": {"all_cus": round(out[3], 1), "own_share": round(out[4], 1), "beside_gemm": round(out[5], 1)},
                          "side_by_side_ms": round(out[6], 3), "back_to_back_on_all_cus_ms": round(out[7], 3)})

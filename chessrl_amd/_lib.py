@@ -87,7 +87,7 @@ SIGNATURES = {
     "crl_model_generate": (_i, [_vp, _vp, _i, _i, _f, C.c_uint64, _i, _vp, _vp, _i, _vp]),
     "crl_sample": (_i, [_vp, _i64, _i, _i, _f, C.c_uint64, _i, _vp, _vp, _vp]),
     "crl_probe_mfma": (_i, [_i, _i, _i, _vp, _vp, _vp]),
-    "crl_probe_cu_split": (_i, [_i, _i, _i, _vp]),
+    "crl_probe_cu_split": (_i, [_i, _i, _i, _i, _vp]),
 }
 
 _lib = None

@@ -741,10 +741,11 @@ int crl_probe_mfma(int dtype, int random_bits, int iters, double* tflops, double
   return CRL_OK;
 }
 
-int crl_probe_cu_split(int gemm_cus, int rows, int iters, double* out8) {
+int crl_probe_cu_split(int gemm_cus, int tile, int rows, int iters, double* out8) {
   if (!out8) return arg_fail("crl_probe_cu_split: null output");
-  hipError_t e = run_cu_split_probe(gemm_cus, rows, iters, out8);
-  if (e == hipErrorInvalidValue) return arg_fail("crl_probe_cu_split: gemm_cus in 8..248, rows a positive multiple of 256, iters >= 1");
+  if (tile < 0 || tile > 14) return arg_fail("crl_probe_cu_split: tile is a crl_gemm tile code");
+  hipError_t e = run_cu_split_probe(gemm_cus, tile, rows, iters, out8);
+  if (e == hipErrorInvalidValue) return arg_fail("crl_probe_cu_split: gemm_cus in 8..248 or 256 (no masks), rows a positive multiple of 256, iters >= 1, a tile code crl_gemm accepts for e4m3 operands");
   return e == hipSuccess ? CRL_OK : hip_fail("crl_probe_cu_split", e);
 }
 

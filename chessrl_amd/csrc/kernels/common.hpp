@@ -333,7 +333,7 @@ hipError_t launch_add_int(int* p, int v, hipStream_t st);
 hipError_t launch_sample(const SampleArgs& a, hipStream_t st);
 // Back-to-back MFMAs from registers on every CU: sustained TFLOP/s and the clock it ran at.
 hipError_t run_mfma_probe(int dtype, int random_bits, int iters, double* tflops, double* ghz, hipStream_t st);
-hipError_t run_cu_split_probe(int gemm_cus, int rows, int iters, double* out8);
+hipError_t run_cu_split_probe(int gemm_cus, int tile, int rows, int iters, double* out8);
 // Slot of (query i, key j) inside a 4096-element attention bias tile.
 int attn_bias_slot_host(int i, int j);
 

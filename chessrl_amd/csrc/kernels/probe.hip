@@ -129,8 +129,9 @@ __global__ void probe_fill_kernel(uint32_t* p, long n, uint32_t keep, uint32_t s
 }
 }  // namespace
 
-hipError_t run_cu_split_probe(int gemm_cus, int rows, int iters, double* out) {
-  if (gemm_cus < 8 || gemm_cus > 248 || rows < 256 || rows % 256 || iters < 1) return hipErrorInvalidValue;
+hipError_t run_cu_split_probe(int gemm_cus, int tile, int rows, int iters, double* out) {
+  // gemm_cus == 256: no masks, two plain streams that share every CU
+  if (gemm_cus < 8 || (gemm_cus > 248 && gemm_cus != 256) || rows < 256 || rows % 256 || iters < 1) return hipErrorInvalidValue;
   const int N = 1024, K = 1024;
   hipError_t e = hipSuccess;
   uint8_t *A = nullptr, *W = nullptr, *X8 = nullptr;
@@ -143,8 +144,13 @@ hipError_t run_cu_split_probe(int gemm_cus, int rows, int iters, double* out) {
     uint32_t mg[8] = {}, mh[8] = {};
     for (int i = 0; i < 256; ++i) (i < gemm_cus ? mg : mh)[i / 32] |= 1u << (i % 32);
     PROBE_TRY(hipStreamCreateWithFlags(&sAll, hipStreamNonBlocking));
-    PROBE_TRY(hipExtStreamCreateWithCUMask(&sG, 8, mg));
-    PROBE_TRY(hipExtStreamCreateWithCUMask(&sH, 8, mh));
+    if (gemm_cus == 256) {
+      PROBE_TRY(hipStreamCreateWithFlags(&sG, hipStreamNonBlocking));
+      PROBE_TRY(hipStreamCreateWithFlags(&sH, hipStreamNonBlocking));
+    } else {
+      PROBE_TRY(hipExtStreamCreateWithCUMask(&sG, 8, mg));
+      PROBE_TRY(hipExtStreamCreateWithCUMask(&sH, 8, mh));
+    }
     for (auto& v : ev) PROBE_TRY(hipEventCreate(&v));
     PROBE_TRY(hipMalloc((void**)&A, (size_t)rows * K));
     PROBE_TRY(hipMalloc((void**)&W, (size_t)N * K));
@@ -168,7 +174,7 @@ hipError_t run_cu_split_probe(int gemm_cus, int rows, int iters, double* out) {
     std::memset(&la, 0, sizeof(la));
     la.x = X; la.ldx = N; la.in_dtype = DT_BF16; la.gamma = g; la.beta = b; la.out_fp8 = X8; la.fp8_scale = 16.f; la.ldo = N;
     la.rows = rows; la.C = N; la.eps = 1e-5f; la.out_dtype = DT_BF16;
-    auto gemm = [&](hipStream_t s) { return launch_gemm(ga, DT_FP8, DT_BF16, 0, s); };
+    auto gemm = [&](hipStream_t s) { return launch_gemm(ga, DT_FP8, DT_BF16, tile, s); };
     auto norm = [&](hipStream_t s) { return launch_layernorm(la, s); };
     auto time_alone = [&](hipStream_t s, int n, bool is_gemm, double* us) -> hipError_t {
       hipError_t te = hipSuccess;

@@ -766,6 +766,7 @@ int Model::forward_chunk(const float* planes, const uint8_t* ids, const uint8_t*
 
 int Model::run_layers(const float* x_in, int B, int first, int last, float* x_out, hipStream_t st) {
   if (!finalized) { set_error("run_layers: call crl_model_finalize first"); return CRL_ERR_STATE; }
+  if (cfg.arch != CRL_ARCH_BT4CLASS) { set_error("run_layers: only CRL_ARCH_BT4CLASS has a layer-window entry"); return CRL_ERR_ARG; }
   if (!x_in || !x_out || B <= 0 || first < 0 || last > cfg.n_layer || first >= last) { set_error("run_layers: bad arguments (0 <= first < last <= n_layer)"); return CRL_ERR_ARG; }
   if (B > cfg.micro_batch) { set_error("run_layers: at most one micro-batch of positions"); return CRL_ERR_ARG; }
   int rc = ensure_ws(B);

@@ -294,8 +294,8 @@ int crl_model_evaluate_fens(crl_model* m, const char* const* fens, int n, int ch
 int crl_model_search_1ply(crl_model* m, const char* const* fens, int n, int chunk, float temperature, uint64_t seed,
                           char* best_uci6, int32_t* n_moves, char* moves_uci6, float* values, int64_t capacity, int threads);
 /* Verification hooks with no counterpart in the reference (its layers are nn.Modules one can call one at a time:
- * new_paradigm/value.py:58-75 EncoderLayer.forward, model_bis.py:110-113 Block.forward). crl_model_run_layers runs encoder
- * layers [first, last) on a caller-supplied layer input x_in (device f32 [B*64, d_model], at most one micro-batch) and
+ * new_paradigm/value.py:58-75 EncoderLayer.forward, model_bis.py:110-113 Block.forward). crl_model_run_layers (CRL_ARCH_BT4CLASS
+ * only) runs encoder layers [first, last) on a caller-supplied layer input x_in (device f32 [B*64, d_model], at most one micro-batch) and
  * writes the output of layer last-1 to x_out (device f32, same shape). The window's first layer treats x_in as layer 0
  * treats the embedding (stored in the model's activation type; for an fp8 model its e4m3 copy is quantised from x_in
  * directly with that layer's scale), its last layer writes its output in the 16-bit type as the trunk's last layer does,
@@ -351,8 +351,9 @@ int crl_probe_mfma(int dtype, int random_bits, int iters, double* tflops, double
  * product rows x 1024 x 1024, the rest for the trunk LayerNorm over `rows` rows of 1024) are timed alone on all CUs, alone on
  * their share and side by side. out8: product us/launch on all CUs, on its share, beside the norm; norm us/launch on all
  * CUs, on its share, beside the product; wall time of the side-by-side run in ms; the same launches back to back on all
- * CUs in ms. Allocates its own operands; synchronises the device. */
-int crl_probe_cu_split(int gemm_cus, int rows, int iters, double* out8);
+ * CUs in ms. gemm_cus = 256 uses two plain streams instead (both kernels may use every CU); tile is the crl_gemm tile code of
+ * the product (0 = the library's choice). Allocates its own operands; synchronises the device. */
+int crl_probe_cu_split(int gemm_cus, int tile, int rows, int iters, double* out8);
 
 #ifdef __cplusplus
 }

@@ -205,6 +205,30 @@ def test_fp8_every_layer_teacher_forced(cuda):
     assert min(e_bias, e_rows, e_scale) > 1.5 * d_ab
 
 
+def test_layer_window_arguments(cuda):
+    """The layer-window hook checks its arguments: empty or reversed windows, layers past the end, more than one
+    micro-batch and the other architectures are CRL_ERR_ARG with a message; a bf16 model's window equals the oracle's layers
+    within the 16-bit anchor's error."""
+    from chessrl_amd import _lib
+    oracle = om.test_init_(om.BT4ClassOracle(policy_leela, 3, 256, 384, 8), seed=5)
+    m = models.BT4Class(3, 256, 384, 8, micro_batch=64)
+    m.load_state_dict(oracle.state_dict())
+    x = oracle.embed(torch.from_numpy(board.random_positions(9, 32)["planes"])).detach()
+    for first, last in ((0, 0), (2, 1), (0, 4), (-1, 2)):
+        with pytest.raises(_lib.CrlError, match="first < last"):
+            m._engine.run_layers(x.to(cuda), first, last)
+    with pytest.raises(_lib.CrlError, match="micro-batch"):
+        m._engine.run_layers(torch.zeros(65, 64, 256, device=cuda), 0, 1)
+    g = models.GPT(models.GPTConfig(block_size=256, vocab_size=1929, n_layer=1, n_head=8, n_embd=256))
+    with pytest.raises(_lib.CrlError, match="BT4CLASS"):
+        g._engine.run_layers(x.to(cuda), 0, 1)
+    with torch.no_grad():
+        want = oracle.forward_layers(x, 1, 3)
+        anchor = oracle.forward_layers(x, 1, 3, store=om.Storage(torch.bfloat16))
+    got = m._engine.run_layers(x.to(cuda), 1, 3).cpu()
+    assert rel_rms(got, want) <= 1.5 * rel_rms(anchor, want) + 1e-3
+
+
 def test_fp8_operand_codes_match_emulation(cuda):
     """The e4m3 operand copies the library writes inside a layer, byte for byte against the codes the emulation
     quantises on the same layer input (emulation B of the test above: bf16 storage where this path stores bf16,
