@@ -290,7 +290,7 @@ int Model::finalize() {
     // The reference's fp8 recipe turns every nn.Linear of the model into a te.Linear, the output head included
     // (model_fp8.py:43,45,90,92,140): in the e4m3 BT4-class model the three head linears that run on every token
     // (policy_tokens_lin, queries_pol|keys_pol, value_head.dense1) get e4m3 copies too. dense2 and dense3 (one row per
-    // position) stay 16-bit. Off unless asked for (cfg.fp8_lm_head = 1): on the benchmark model it takes 0.6 ms off a
+    // position) stay 16-bit. Off unless asked for (cfg.fp8_lm_head = 1): on the benchmark model it takes 0.8 ms off a
     // 49 ms pass and adds half again to the policy error against fp32.
     const bool f8heads = f8 && cfg.arch == CRL_ARCH_BT4CLASS && cfg.fp8_lm_head > 0;
     LIN(pol_tok, w("policy_tokens_lin.weight"), &w("policy_tokens_lin.bias"), C, C, hd, f8heads);

@@ -205,7 +205,7 @@ typedef struct crl_model_config {
                              nn.Linear (model_fp8.py:43,45,90,92,140): lm_head for GPT64; policy_tokens_lin, queries_pol|keys_pol
                              and value_head.dense1 for BT4-class. 1 = e4m3 heads, -1 = 16-bit heads, 0 = default: on for GPT64
                              (the reference's fp8 model), off for BT4-class (whose policy is a product of two quantised
-                             projections: its error against fp32 grows by half for about one percent of the pass). */
+                             projections: its error against fp32 grows by half for under two percent of the pass). */
   int32_t small_batch_k_parallel; /* 1: every product of a call of at most 8 positions spreads K over more waves or
                              workgroups, as the token steps of crl_model_generate do. Faster for single-position calls, but the
                              sums are then added in another order than in the tiled kernels, so a position's result is no
