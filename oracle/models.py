@@ -22,6 +22,10 @@ What each class follows (reference file:line):
                  Restated as quantise->dequantise->F.linear. PARITY UNPINNED against
                  transformer_engine itself; the arithmetic is pinned as listed below.
   rms_norm       the RMSNorm alternative of the trunk norms (no reference model uses it).
+  Storage        16-bit storage emulation: rounds named tensors of BT4ClassOracle's forward (weights, q|k|v, softmax
+                 output, residual sums, norm outputs, ...) to bf16/f16 and computes everything else in fp32. What a
+                 faithful 16-bit implementation can reach against the fp32 forward, site by site. Not a reference
+                 component; pinned below.
 
 Pins: GPTOracle (64-token forward, token forward, loss), BT4Oracle (policy and value) and
 relative_attention are checked in tests/test_golden.py against outputs of the reference's own
@@ -37,6 +41,9 @@ when the generated bias is zero and by a head-by-head loop with a hand-built bia
 (a transposed bias tile is shown to fail); the residual scale (2L)^-1/4, norm placement and
 mish position by a two-layer composition from plain tensor operations; the value head's
 token-major flatten likewise.
+Storage is pinned in tests/test_oracle.py: a named site is rounded exactly (x.to(dtype).float()), an unnamed one is left
+alone, embed -> forward_layers -> heads composes to forward_pv bit for bit, and with every site rounded the forward lands
+within 0.5-1.5x of torch's own `module.to(torch.bfloat16)` forward of the same oracle.
 fp8_quant_dequant / Fp8Plan are pinned against a table of all 256 e4m3fn codes built from the
 format's definition with an explicit nearest-even search (ties, subnormals, saturation), and the
 plan's linear against quantise-dequantise-matmul written out with that table; rms_norm against
