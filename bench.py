@@ -135,6 +135,20 @@ def latency_workload(a, torch, models, board, dev):
             ts.append((time.perf_counter() - t1) * 1e3)
         ts = sorted(ts[a.warmup:])
         per_batch["b%d" % nb]["k_parallel_p50_ms"] = round(ts[len(ts) // 2], 3)
+    # for comparison: the e4m3 model of the headline workload in the same leaf-evaluation mode
+    f8 = models.BT4Class(15, 1024, 1536, 32, fp8=True, act_dtype=a.act_dtype, seed=0)
+    f8.calibrate(torch.from_numpy(board.random_positions(2, 512)["planes"]).to(dev))
+    for nb in (1, 8, 64, 256):
+        lp, lm = planes[:nb].contiguous(), masks[:nb].contiguous()
+        ts = []
+        for i in range(a.warmup + max(a.steps, 50)):
+            torch.cuda.synchronize()
+            t1 = time.perf_counter()
+            f8.evaluate(lp, legal_mask=lm, T=1.0, want_probs=True)
+            torch.cuda.synchronize()
+            ts.append((time.perf_counter() - t1) * 1e3)
+        ts = sorted(ts[a.warmup:])
+        per_batch["b%d" % nb]["fp8_model_p50_ms"] = round(ts[len(ts) // 2], 3)
     b64 = per_batch["b64"]
     print(json.dumps({"metric": "p50 latency of one evaluate call, BT4-class bf16 b64 with legal-masked softmax", "value": b64["p50_ms"], "unit": "ms",
                       "n_gpus": 1, "steps": max(a.steps, 50), "warmup": a.warmup, "ms_per_step": b64["p50_ms"], "higher_is_better": False,
