@@ -10,7 +10,6 @@ Three questions, each answered against something independent of the HIP code:
 import copy
 import math
 
-import numpy as np
 import pytest
 import torch
 
