@@ -57,6 +57,11 @@ def build(verbose=True):
     r = subprocess.run(cmd, capture_output=True, text=True)
     if r.returncode != 0:
         raise RuntimeError("link failed:\n" + r.stderr)
+    # -shared lets unresolved names through to load time: a kernel whose host stub the compiler dropped shows up here.
+    nm = subprocess.run(["nm", "-u", LIB], capture_output=True, text=True)
+    missing = [l.split()[-1] for l in nm.stdout.splitlines() if "_ZN3crl" in l]
+    if missing:
+        raise RuntimeError("unresolved symbols of this library's own namespace:\n" + "\n".join(missing))
     if verbose:
         print("built", LIB)
     return LIB
