@@ -122,19 +122,6 @@ def latency_workload(a, torch, models, board, dev):
         # (the per-family counters do not see the two launches outside them: the side-to-move extraction and the masked softmax)
         per_batch["b%d" % nb] = {"p50_ms": round(ts[len(ts) // 2], 3), "p99_ms": round(ts[min(len(ts) - 1, int(len(ts) * 0.99))], 3),
                                  "samples": len(ts), "launches_per_forward": sum(v["launches"] for v in prof.values()) + 2}
-    # the opt-in mode for tiny batches: K spread over more waves (a position's bits then depend on its batch)
-    kp = models.BT4Class(15, 1024, 1536, 32, fp8=False, act_dtype=a.act_dtype, seed=0, small_batch_k_parallel=True)
-    for nb in (1, 8):
-        lp, lm = planes[:nb].contiguous(), masks[:nb].contiguous()
-        ts = []
-        for i in range(a.warmup + max(a.steps, 50)):
-            torch.cuda.synchronize()
-            t1 = time.perf_counter()
-            kp.evaluate(lp, legal_mask=lm, T=1.0, want_probs=True)
-            torch.cuda.synchronize()
-            ts.append((time.perf_counter() - t1) * 1e3)
-        ts = sorted(ts[a.warmup:])
-        per_batch["b%d" % nb]["k_parallel_p50_ms"] = round(ts[len(ts) // 2], 3)
     # for comparison: the e4m3 model of the headline workload in the same leaf-evaluation mode
     f8 = models.BT4Class(15, 1024, 1536, 32, fp8=True, act_dtype=a.act_dtype, seed=0)
     f8.calibrate(torch.from_numpy(board.random_positions(2, 512)["planes"]).to(dev))

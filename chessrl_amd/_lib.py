@@ -20,7 +20,7 @@ class ModelConfig(C.Structure):
         ("arch", C.c_int32), ("n_layer", C.c_int32), ("d_model", C.c_int32), ("n_head", C.c_int32),
         ("d_ff", C.c_int32), ("fp8", C.c_int32), ("micro_batch", C.c_int32), ("stream_f32", C.c_int32),
         ("head_dtype", C.c_int32), ("smolgen_compress", C.c_int32), ("smolgen_hidden", C.c_int32),
-        ("smolgen_gen", C.c_int32), ("eps", C.c_float), ("act_dtype", C.c_int32), ("ln_fold", C.c_int32), ("norm_rms", C.c_int32), ("fp8_lm_head", C.c_int32), ("small_batch_k_parallel", C.c_int32),
+        ("smolgen_gen", C.c_int32), ("eps", C.c_float), ("act_dtype", C.c_int32), ("ln_fold", C.c_int32), ("norm_rms", C.c_int32), ("fp8_lm_head", C.c_int32),
     ]
 
 

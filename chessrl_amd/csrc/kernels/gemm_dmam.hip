@@ -1,4 +1,4 @@
-// Instances of the 128x128 GEMM fed by direct-to-LDS loads through a four-stage ring (gemm_dmam_kernel.hpp), in a
+// Instances of the 128x128 and 64x64 GEMMs fed by direct-to-LDS loads through a ring of stages (gemm_dmam_kernel.hpp), in a
 // translation unit of their own.
 #include "gemm_dmam_kernel.hpp"
 
@@ -10,7 +10,21 @@ bool gemm_dmam_has(int in_dt, int out_dt) {
   return in_dt == out_dt && (in_dt == DT_BF16 || in_dt == DT_F16);
 }
 
-hipError_t launch_gemm_dmam(const GemmArgs& a, int in_dt, int out_dt, hipStream_t st) {
+// small_tile: the 64x64 tile with eight stages instead of the 128x128 tile with four.
+hipError_t launch_gemm_dmam(const GemmArgs& a, int in_dt, int out_dt, hipStream_t st, bool small_tile) {
+  if (small_tile) {
+    typedef DmamCfgT<64> S;
+    if (in_dt == DT_FP8) {
+      switch (out_dt) {
+        case DT_BF16: return launch_dmam<DT_FP8, DT_BF16, 0, S>(a, st);
+        case DT_F16: return launch_dmam<DT_FP8, DT_F16, 0, S>(a, st);
+        case DT_FP8: return launch_dmam<DT_FP8, DT_FP8, 0, S>(a, st);
+      }
+    }
+    if (in_dt == DT_BF16 && out_dt == DT_BF16) return launch_dmam<DT_BF16, DT_BF16, 0, S>(a, st);
+    if (in_dt == DT_F16 && out_dt == DT_F16) return launch_dmam<DT_F16, DT_F16, 0, S>(a, st);
+    return hipErrorInvalidValue;
+  }
   // (whole tiles in M, aligned rows, a bf16 residual or none, no maximum: the instances without the epilogue's guards)
   const bool lean = a.M % DmamCfg::BM == 0 && a.vec_ok && a.N % 8 == 0 && a.nsplit % 8 == 0 && !a.amax && a.res_rows == 0 && !a.ln_out &&
                     (!a.res || a.res_dtype == DT_BF16);

@@ -13,24 +13,31 @@
 
 namespace crl {
 
-// Eight waves of 64x32 on the tile (8 MFMAs per 12 fragment reads and slab). Four waves of 64x64 (16 MFMAs per 16 reads)
-// issue fewer instructions but have half as many loads and MFMA streams in flight: measured 4 to 5 % slower on bf16
-// and 6 to 10 % on e4m3 (M=4096, N=1024, K=1024: 17.0 -> 16.3 us bf16, 10.4 -> 9.3 us e4m3).
-struct DmamCfg {
-  static constexpr int BM = 128, BN = 128, WGM = 2, WGN = 4, NW = WGM * WGN, NT = 64 * NW;
+// BT = 128: eight waves of 64x32 on a 128x128 tile (8 MFMAs per 12 fragment reads and slab), four stages of 32 KB. Four
+// waves of 64x64 (16 MFMAs per 16 reads) issue fewer instructions but have half as many loads and MFMA streams in
+// flight: measured 4 to 5 % slower on bf16 and 6 to 10 % on e4m3 (M=4096, N=1024, K=1024: 17.0 -> 16.3 us bf16, 10.4 -> 9.3 us e4m3).
+// BT = 64: four waves of 32x32 on a 64x64 tile, eight stages of 16 KB, for products of at most a few hundred such tiles
+// (a forward pass over one to eight positions), where the time is the latency of walking K and the seven slabs in flight hide it.
+// Either way a wave fills 32 of a stage's rows with four load instructions.
+template <int BT>
+struct DmamCfgT {
+  static_assert(BT == 128 || BT == 64, "two tile sizes");
+  static constexpr int BM = BT, BN = BT, WGM = 2, WGN = BT / 32, NW = WGM * WGN, NT = 64 * NW;
   static constexpr int WM = BM / WGM, WN = BN / WGN, TM = WM / 32, TN = WN / 32;
-  static constexpr int ROWB = 128, NSTAGE = 4;
-  static constexpr int ROWS_PER_WAVE = 2 * BM / NW;             // a wave fills 32 of the 256 rows of a stage
-  static constexpr int LOADS = ROWS_PER_WAVE / 8;
+  static constexpr int ROWB = 128, NSTAGE = 512 / BT;
+  static constexpr int ROWS_PER_WAVE = 2 * BM / NW;             // 32
+  static constexpr int LOADS = ROWS_PER_WAVE / 8;               // 4
   static constexpr int PART_BYTES = NSTAGE * BN * ROWB;         // 64 KB: the weight rows of all stages, then the activation rows
   static constexpr int RING_BYTES = 2 * PART_BYTES;             // 128 KB
-  static constexpr int EPI_BYTES = NW * 32 * WN * 4;            // 32 KB
+  static constexpr int EPI_BYTES = NW * 32 * WN * 4;            // 32 KB (16 KB)
   static constexpr int STATS_OFF = RING_BYTES + 256;
   static constexpr int COLS_OFF = STATS_OFF + NW * 2 * WM * 4;  // per-column epilogue constants: [wave][bias, gain, offset][64]
   static constexpr int COLS_STRIDE = 3 * 64;                    // floats per wave (a wave's bias load lands 64 of them)
   static constexpr int LDS_BYTES = COLS_OFF + NW * COLS_STRIDE * 4;
+  static_assert(WN == 32 && LOADS == 4 && (NSTAGE - 2) * LOADS + 1 < 64, "wave shape; the counted waits fit the counter");
   static_assert(EPI_BYTES <= RING_BYTES && LDS_BYTES <= 160 * 1024, "LDS of a CU");
 };
+typedef DmamCfgT<128> DmamCfg;
 
 // A bare barrier: the waits it needs are written out in front of it (a __syncthreads waits for every outstanding memory
 // operation, i.e. for the slabs that are meant to stay in flight).
@@ -44,13 +51,12 @@ __device__ __forceinline__ void dmam_load16(__amdgpu_buffer_rsrc_t r, uint8_t* d
 }
 
 // LEAN: the epilogue without its edge and type guards (gemm_epilogue's LEAN = 1; the launcher says when).
-template <int IN_DT, int OUT_DT, int LEAN = 0>
-__global__ void __launch_bounds__(DmamCfg::NT) gemm_dmam_kernel(const GemmArgs a, const DmafWalk wk) {
-  typedef DmamCfg Cfg;
+template <typename Cfg, int IN_DT, int OUT_DT, int LEAN>
+__global__ void __launch_bounds__(Cfg::NT) gemm_dmam_kernel(const GemmArgs a, const DmafWalk wk) {
   constexpr int ESZ = IN_DT == DT_FP8 ? 1 : 2;                      // bytes per operand element
   constexpr int KSTEPS = Cfg::ROWB / (IN_DT == DT_FP8 ? 64 : 32);   // MFMA K steps per slab
   constexpr int BM = Cfg::BM, BN = Cfg::BN, TM = Cfg::TM, TN = Cfg::TN, LOADS = Cfg::LOADS, NSTAGE = Cfg::NSTAGE;
-  constexpr int STAGE = BN * Cfg::ROWB;   // bytes of one operand's rows in one stage (16 KB)
+  constexpr int STAGE = BN * Cfg::ROWB;   // bytes of one operand's rows in one stage
   extern __shared__ __align__(16) uint8_t smem[];
 
   // (the wave index as a scalar: everything derived from it, LDS destinations and descriptors, stays in scalar registers)
@@ -96,7 +102,7 @@ __global__ void __launch_bounds__(DmamCfg::NT) gemm_dmam_kernel(const GemmArgs a
       dmam_load16(r, dst + i * 1024, (int)voff[i], slab * Cfg::ROWB);
     });
   };
-  // Three slabs go out as early as their addresses exist.
+  // All slabs but one of the ring go out as early as their addresses exist.
 #pragma unroll
   for (int s0 = 0; s0 < NSTAGE - 1; ++s0) issue_slab(s0);
   __builtin_amdgcn_sched_barrier(0);
@@ -108,7 +114,7 @@ __global__ void __launch_bounds__(DmamCfg::NT) gemm_dmam_kernel(const GemmArgs a
     __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(a.bias + n),
                                      (__attribute__((address_space(3))) void*)(smem + Cfg::COLS_OFF + wave * (Cfg::COLS_STRIDE * 4)), 4, 0, 0);
   }
-  const int extra_loads = a.bias ? 1 : 0;   // (issued behind the three slabs: the first waits allow for it)
+  const int extra_loads = a.bias ? 1 : 0;   // (issued behind the first slabs: the first wait allows for it)
 
   f32x16_t acc[TN][TM];
 #pragma unroll
@@ -135,12 +141,12 @@ __global__ void __launch_bounds__(DmamCfg::NT) gemm_dmam_kernel(const GemmArgs a
   const bool wave_active = (m0 + wm * Cfg::WM < a.M) && (n0 + wn * Cfg::WN < a.N);
 
   for (int slab = 0; slab < nslab; ++slab) {
-    // This wave's loads of the slab have landed; the two slabs requested after it (and, the first time round, the
+    // This wave's loads of the slab have landed; the NSTAGE - 2 slabs requested after it (and, the first time round, the
     // column constants) may stay in flight.
-    if (slab == 0 && extra_loads) wait_vmcnt<2 * LOADS + 1>();
-    else wait_vmcnt<2 * LOADS>();
+    if (slab == 0 && extra_loads) wait_vmcnt<(NSTAGE - 2) * LOADS + 1>();
+    else wait_vmcnt<(NSTAGE - 2) * LOADS>();
     dmam_barrier();
-    // Stage (slab + 3) % 4 held slab - 1: every wave has finished with it before it reached this barrier.
+    // Stage (slab - 1) % NSTAGE held slab - 1: every wave has finished with it before it reached this barrier.
     issue_slab(slab + NSTAGE - 1);
     if (!wave_active) continue;
     const uint32_t soff = (slab & (NSTAGE - 1)) * STAGE;
@@ -177,24 +183,23 @@ __global__ void __launch_bounds__(DmamCfg::NT) gemm_dmam_kernel(const GemmArgs a
                                               reinterpret_cast<const float*>(smem + Cfg::COLS_OFF) + wave * Cfg::COLS_STRIDE);
 }
 
-template <int IN_DT, int OUT_DT, int LEAN = 0>
+template <int IN_DT, int OUT_DT, int LEAN = 0, typename Cfg = DmamCfg>
 static hipError_t launch_dmam(const GemmArgs& a, hipStream_t st) {
   static std::atomic<bool> attr_set[16] = {};
-  typedef DmamCfg Cfg;
   hipError_t e = hipSuccess;
   constexpr int ESZ = IN_DT == DT_FP8 ? 1 : 2;
   if ((a.K * ESZ) % DmamCfg::ROWB != 0 || a.K <= 0 || a.res_stats || (long)a.lda * ESZ * 128 >= (1L << 31) || (long)a.ldw * ESZ * 128 >= (1L << 31))
     return hipErrorInvalidValue;
   int dev = 0;
   (void)hipGetDevice(&dev);
-  auto kern = gemm_dmam_kernel<IN_DT, OUT_DT, LEAN>;
+  auto kern = gemm_dmam_kernel<Cfg, IN_DT, OUT_DT, LEAN>;
   if (!attr_set[dev]) {
     e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, Cfg::LDS_BYTES);
     if (e != hipSuccess) return e;
     attr_set[dev] = true;
   }
-  const int tiles_n = (a.N + DmamCfg::BN - 1) / DmamCfg::BN;
-  const int tiles = ((a.M + DmamCfg::BM - 1) / DmamCfg::BM) * tiles_n;
+  const int tiles_n = (a.N + Cfg::BN - 1) / Cfg::BN;
+  const int tiles = ((a.M + Cfg::BM - 1) / Cfg::BM) * tiles_n;
   if (tiles >= 65536) return hipErrorInvalidValue;
   DmafWalk wk{};
   wk.tiles_n = tiles_n;

@@ -453,7 +453,7 @@ int Model::gemm(const Lin& L, const void* A, long lda, int in_dt, void* C, long 
   g.alpha = o.alpha; g.out_scale = o.out_scale;
   // Few rows: K spread over more waves (another summation order; the token steps of generation always, the forward pass
   // only where the model was told that a position's bits may depend on the batch it travels in).
-  g.k_parallel = (o.k_parallel || (cfg.small_batch_k_parallel > 0 && chunk_positions <= 8 && !o.res_stats)) ? 1 : 0;
+  g.k_parallel = o.k_parallel ? 1 : 0;
   g.splitk_ws = ws.splitk; g.splitk_ws_bytes = Workspace::SPLITK_BYTES;
   if (o.ln_out) {
     g.nsplit = g.N;
@@ -534,7 +534,6 @@ int Model::forward_chunk(const float* planes, const uint8_t* ids, const uint8_t*
   // Layers [l0, l1) of this call: the whole trunk, or the window of run_layers (its input comes from the caller instead of
   // the embedding, its first layer reads that input as a plain residual and its last one writes the 16-bit output).
   const int l0 = win ? win->first : 0, l1 = win ? win->last : L;
-  chunk_positions = mb;
   const int T = 64 + t;          // tokens per position: the board, then t move tokens (CRL_ARCH_GPT64 only)
   const int M = mb * T;
   const bool f8 = cfg.fp8 && !calibrate && !force_16bit;

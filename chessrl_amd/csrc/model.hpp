@@ -90,7 +90,6 @@ struct Model {
   int* gen_k = nullptr;             // device counter: index of the token a replayed step samples
   hipStream_t cap_stream = nullptr; // records the step graph (nothing executes on it)
   bool decode_graph = false;
-  int chunk_positions = 0;     // positions of the forward_chunk call in flight (selects the small-batch product kernels)
   bool kv_capture = false;     // forward_chunk copies every layer's keys|values into the cache
   bool force_16bit = false;    // forward_chunk ignores cfg.fp8
 

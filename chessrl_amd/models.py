@@ -160,7 +160,7 @@ class _Engine:
 
     def __init__(self, arch, n_layer, d_model, n_head, d_ff, fp8=False, micro_batch=0, stream_f32=None,
                  head_dtype=None, act_dtype="bf16", compress=32, hidden=256, gen=256, ln_fold=None, norm_rms=False,
-                 fp8_lm_head=None, small_batch_k_parallel=False):
+                 fp8_lm_head=None):
         cfg = _lib.ModelConfig()
         cfg.arch, cfg.n_layer, cfg.d_model, cfg.n_head, cfg.d_ff = arch, n_layer, d_model, n_head, d_ff
         cfg.fp8 = 1 if fp8 else 0
@@ -169,7 +169,6 @@ class _Engine:
         cfg.stream_f32 = tri(stream_f32)
         cfg.ln_fold = tri(ln_fold)
         cfg.fp8_lm_head = tri(fp8_lm_head)
-        cfg.small_batch_k_parallel = 1 if small_batch_k_parallel else 0
         cfg.norm_rms = 1 if norm_rms else 0
         cfg.act_dtype = _lib.F16 if act_dtype in ("f16", "fp16") else _lib.BF16
         cfg.head_dtype = cfg.act_dtype if head_dtype is None else _lib.F16 if head_dtype in ("f16", "fp16") else _lib.BF16
@@ -702,17 +701,14 @@ class BT4Class(_ModelBase):
 
     def __init__(self, num_layers=15, d_model=1024, d_ff=1536, num_heads=32, fp8=False, micro_batch=0,
                  head_dtype=None, act_dtype="bf16", compress=32, hidden=256, gen=256, seed=0, stream_f32=None, ln_fold=None,
-                 norm_rms=False, fp8_heads=None, small_batch_k_parallel=False):
-        """fp8_heads: with fp8, run policy_tokens_lin, queries_pol|keys_pol and value dense1 in e4m3 too (off by default).
-        small_batch_k_parallel: batches of at most 8 positions spread K over more waves (faster single-position calls; the
-        result of a position then differs in its last bits from its row in a larger batch)."""
+                 norm_rms=False, fp8_heads=None):
+        """fp8_heads: with fp8, run policy_tokens_lin, queries_pol|keys_pol and value dense1 in e4m3 too (off by default)."""
         self.num_layers, self.d_model = num_layers, d_model
         self._shapes = bt4_shapes(num_layers, d_model, d_ff, num_heads, True, compress, hidden, gen)
         self._sd = _default_init(self._shapes, seed)
         self._engine = _Engine(_lib.ARCH_BT4CLASS, num_layers, d_model, num_heads, d_ff, fp8=fp8, micro_batch=micro_batch,
                                head_dtype=head_dtype, act_dtype=act_dtype, compress=compress, hidden=hidden, gen=gen,
-                               stream_f32=stream_f32, ln_fold=ln_fold, norm_rms=norm_rms, fp8_lm_head=fp8_heads,
-                               small_batch_k_parallel=small_batch_k_parallel)
+                               stream_f32=stream_f32, ln_fold=ln_fold, norm_rms=norm_rms, fp8_lm_head=fp8_heads)
         self._engine.load(self._sd)
 
     @torch.no_grad()

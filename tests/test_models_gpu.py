@@ -245,32 +245,6 @@ def test_bt4class_full_size_latency_batches_with_legal_masks(cuda, B):
     assert torch.equal(onehot.sum(-1).cpu(), torch.ones(B))
 
 
-@pytest.mark.parametrize("B", [1, 8])
-def test_bt4class_small_batch_k_parallel_option(cuda, B):
-    """small_batch_k_parallel: calls of at most 8 positions spread K over more waves (the kernels of the generation token
-    steps). Another summation order, the same accuracy: against the fp32 oracle at the bars of the latency test above,
-    and within 16-bit rounding noise of the default (tiled, batch-invariant) path."""
-    ref = full_size_reference()
-    m = models.BT4Class(15, 1024, 1536, 32, small_batch_k_parallel=True)
-    m.load_state_dict(ref["oracle"].state_dict())
-    planes, mask = ref["planes"][:B], ref["mask"][:B]
-    probs, wdl = m.evaluate(planes.to(cuda), legal_mask=mask.to(cuda), T=1.0, want_probs=True)
-    probs, wdl = probs.cpu(), wdl.cpu()
-    want = om.masked_policy(ref["rpol"][:B], mask, 1.0)
-    assert torch.equal(probs > 0, mask.bool())
-    assert (probs - want).abs().max() < 5e-3 and (wdl - ref["rwdl"][:B]).abs().max() <= 1e-2
-    base = ref["m_bf16"] if "m_bf16" in ref else None
-    if base is not None:
-        p0, w0 = base.evaluate(planes.to(cuda), legal_mask=mask.to(cuda), T=1.0, want_probs=True)
-        assert (p0.cpu() - probs).abs().max() < 2e-3 and (w0.cpu() - wdl).abs().max() < 1e-2
-    # larger batches are untouched by the option: bit-equal to the default path
-    if B == 8 and base is not None:
-        big = ref["planes"][:64].to(cuda)
-        pa, wa = m(big)
-        pb, wb = base(big)
-        assert torch.equal(pa, pb) and torch.equal(wa, wb)
-
-
 def test_bt4class_fp8_headline_config(cuda):
     """The headline configuration at full size: 15 x 1024 x 32 heads, FFN 1536, e4m3 trunk linears with static scales
     from a 512-position calibration batch (seed 2), benchmark initialisation (seed 0), positions seed 1. The HIP path
