@@ -211,7 +211,7 @@ int crl_gemm(const void* A, int64_t lda, const void* W, int64_t ldw, void* C, in
              float out_scale, float* amax, int tile, void* stream) {
   if (!A || !W || !C || M < 0 || N < 0 || K <= 0) return arg_fail("crl_gemm: bad arguments");
   if (in_dtype != DT_BF16 && in_dtype != DT_F16 && in_dtype != DT_FP8) return arg_fail("crl_gemm: in_dtype must be bf16, f16 or fp8");
-  if (out_dtype < 0 || out_dtype > 3 || tile < 0 || tile > 15 || tile == 6 || tile == 8) return arg_fail("crl_gemm: bad out_dtype or tile");
+  if (out_dtype < 0 || out_dtype > 3 || tile < 0 || tile > 16 || tile == 6 || tile == 8) return arg_fail("crl_gemm: bad out_dtype or tile");
   GemmArgs g;
   std::memset(&g, 0, sizeof(g));
   g.A = A; g.lda = lda; g.W = W; g.ldw = ldw; g.C = C; g.ldc = ldc; g.M = M; g.N = N; g.K = K; g.nsplit = N;

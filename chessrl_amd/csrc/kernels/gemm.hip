@@ -601,12 +601,13 @@ static hipError_t launch_in_out(const GemmArgs& a, int tile, hipStream_t st) {
       const int ks = splitk_plan_fixed(a, IN_DT == DT_FP8 ? 1 : 2, &per);
       if (ks > 1) return launch_splitk<CfgSmallK4, IN_DT, OUT_DT>(a, ks, per, st);
     }
-    // Fewer than 256 tiles of 128x128 and K in whole slabs: the ring kernels of gemm_dmam_kernel.hpp (bit-equal). On 64x64
-    // tiles while every tile has a CU of its own (tile 15; M=64, N=1024, K=1024 bf16 with weights from HBM: 13.6 -> 8.4 us),
-    // on 128x128 tiles beyond (tile 11; M=1024, N=3104: 20.7 -> 14.9 us; M=2048, N=1536: 18.0 -> 14.1 us; M=512, N=3104:
-    // 13.9 -> 12.5 us; level at M=1024, N=1536 and M=2048, N=1024).
+    // Fewer than 256 tiles of 128x128 and K in whole slabs: the ring kernels of gemm_dmam_kernel.hpp (bit-equal). On 32x32
+    // tiles while every such tile has a CU of its own (tile 16; one position), else on 64x64 tiles while every one of
+    // those has (tile 15; M=64, N=1024, K=1024 bf16 with weights from HBM: 13.6 us register-staged, 8.4 us on 15; from
+    // warm caches 9.1, 7.6 and, on 16, 6.9 us), on 128x128 tiles beyond (tile 11; M=1024, N=3104: 20.7 -> 14.9 us;
+    // M=2048, N=1536: 18.0 -> 14.1 us; M=512, N=3104: 13.9 -> 12.5 us; level at M=1024, N=1536 and M=2048, N=1024).
     if (tile == 1 && !a.k_parallel && !a.res_stats && ((long)a.K * (IN_DT == DT_FP8 ? 1 : 2)) % 128 == 0 && gemm_dmam_has(IN_DT, OUT_DT))
-      tile = small <= device_cus() ? 15 : 11;
+      tile = (long)((a.M + 31) / 32) * ((a.N + 31) / 32) <= device_cus() ? 16 : small <= device_cus() ? 15 : 11;
   }
   if (tile == 6 || tile == 8) return hipErrorInvalidValue;   // codes of two retired kernels
   // The 256x256 tile has three kernels. Eight waves in step (gemm_dma_kernel.hpp, tile 7): every operand type, any K. The
@@ -633,12 +634,12 @@ static hipError_t launch_in_out(const GemmArgs& a, int tile, hipStream_t st) {
   // (gemm_dmam_kernel.hpp, tile 11; bit-equal; one workgroup per CU). The second is 15 to 20 % faster while every tile has a
   // CU of its own (M=4096, N=1024, bf16: 20.1 -> 16.3 us at K=1024, 27.9 -> 23.0 at K=1536) and slower beyond (384 tiles: 25.9
   // -> 29.8 us), so tile 2 picks it for at most as many tiles as there are CUs.
-  if (tile == 15) return slabs && !a.res_stats && gemm_dmam_has(IN_DT, OUT_DT) ? launch_gemm_dmam(a, IN_DT, OUT_DT, st, true) : hipErrorInvalidValue;
+  if (tile == 15 || tile == 16) return slabs && !a.res_stats && gemm_dmam_has(IN_DT, OUT_DT) ? launch_gemm_dmam(a, IN_DT, OUT_DT, st, tile == 16 ? 32 : 64) : hipErrorInvalidValue;
   if (tile == 11 && !slabs) tile = 12;
   if (tile == 2 || tile == 11) {
     const long mid_tiles = (long)((a.M + 127) / 128) * ((a.N + 127) / 128);
     const bool can = slabs && !a.res_stats && gemm_dmam_has(IN_DT, OUT_DT) && mid_tiles < 65536;
-    if (can && (tile == 11 || mid_tiles <= device_cus())) return launch_gemm_dmam(a, IN_DT, OUT_DT, st, false);
+    if (can && (tile == 11 || mid_tiles <= device_cus())) return launch_gemm_dmam(a, IN_DT, OUT_DT, st, 128);
     if (tile == 11) return hipErrorInvalidValue;
   }
   if (tile == 2 || tile == 12) return launch_cfg<CfgMid, IN_DT, OUT_DT>(a, st);

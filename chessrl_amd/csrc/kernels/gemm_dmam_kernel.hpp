@@ -1,13 +1,12 @@
-// C[M,N] = epilogue(A[M,K] · W[N,K]^T) on a 128x128 workgroup tile fed by direct-to-LDS loads, K a whole number of
-// 128-byte slabs: the tile for problems of 256 to a few hundred such tiles (the out-projection, FFN and bias-generator
-// products of a 64-position batch), where every CU holds one workgroup of eight waves and nothing but the kernel's own
-// pipeline hides memory latency. The register-staged kernel of gemm.hip on the same tile keeps one slab in flight and
-// takes 1.3 us per slab for 0.27 us of MFMA work; here three slabs are in flight in a four-stage ring (32 KB per stage),
-// waited for with counted waits, and the addressing is that of gemm_dmaf_kernel.hpp: fragment addresses are lane
-// registers plus instruction immediates (moved from stage to stage by one add each per slab), loads go through buffer
-// descriptors with the slab offset in a scalar register, and past the end of K through a descriptor of zero length so
-// that every slab issues the same instructions and the counts hold. Same K order and epilogue as the other tiled
-// kernels: bit-equal results.
+// C[M,N] = epilogue(A[M,K] · W[N,K]^T) on a 128x128, 64x64 or 32x32 workgroup tile fed by direct-to-LDS loads through a
+// ring of stages, K a whole number of 128-byte slabs: the kernel for products of at most 256 tiles (the products of a
+// batch of 1 to 64 positions), where every CU holds one workgroup and nothing but the kernel's own pipeline hides memory
+// latency. The register-staged kernels of gemm.hip keep one slab in flight (128x128: 1.3 us per slab for 0.27 us of MFMA
+// work); here all stages but one are in flight (three of four on the 128x128 tile, fifteen of sixteen on the 32x32
+// tile), waited for with counted waits, and the addressing is that of gemm_dmaf_kernel.hpp: fragment addresses are lane
+// registers plus instruction immediates, loads go through buffer descriptors with the slab offset in a scalar register,
+// and past the end of K through a descriptor of zero length so that every slab issues the same instructions and the
+// counts hold. Same K order and epilogue as the other tiled kernels: bit-equal results.
 #pragma once
 #include "gemm_dmaf_kernel.hpp"
 
@@ -17,19 +16,24 @@ namespace crl {
 // waves of 64x64 (16 MFMAs per 16 reads) issue fewer instructions but have half as many loads and MFMA streams in
 // flight: measured 4 to 5 % slower on bf16 and 6 to 10 % on e4m3 (M=4096, N=1024, K=1024: 17.0 -> 16.3 us bf16, 10.4 -> 9.3 us e4m3).
 // BT = 64: four waves of 32x32 on a 64x64 tile, eight stages of 16 KB, for products of at most a few hundred such tiles
-// (a forward pass over one to eight positions), where the time is the latency of walking K and the seven slabs in flight hide it.
+// (a forward pass over a few positions), where the time is the latency of walking K and the seven slabs in flight hide it.
+// BT = 32: one wave computes a 32x32 tile and fills the weight rows, a second wave only fills the activation rows; sixteen
+// stages of 8 KB, so the whole of K = 1024 16-bit elements is in flight at once: one position's products, spread over
+// four times as many CUs as on 64x64 tiles.
 // Either way a wave fills 32 of a stage's rows with four load instructions.
 template <int BT>
 struct DmamCfgT {
-  static_assert(BT == 128 || BT == 64, "two tile sizes");
-  static constexpr int BM = BT, BN = BT, WGM = 2, WGN = BT / 32, NW = WGM * WGN, NT = 64 * NW;
+  static_assert(BT == 128 || BT == 64 || BT == 32, "three tile sizes");
+  static constexpr int BM = BT, BN = BT, WGM = BT >= 64 ? 2 : 1, WGN = BT >= 64 ? BT / 32 : 1;
+  static constexpr int NCOMP = WGM * WGN;                       // waves that compute
+  static constexpr int NW = BT >= 64 ? NCOMP : 2, NT = 64 * NW; // waves that load: all of them
   static constexpr int WM = BM / WGM, WN = BN / WGN, TM = WM / 32, TN = WN / 32;
   static constexpr int ROWB = 128, NSTAGE = 512 / BT;
   static constexpr int ROWS_PER_WAVE = 2 * BM / NW;             // 32
   static constexpr int LOADS = ROWS_PER_WAVE / 8;               // 4
   static constexpr int PART_BYTES = NSTAGE * BN * ROWB;         // 64 KB: the weight rows of all stages, then the activation rows
   static constexpr int RING_BYTES = 2 * PART_BYTES;             // 128 KB
-  static constexpr int EPI_BYTES = NW * 32 * WN * 4;            // 32 KB (16 KB)
+  static constexpr int EPI_BYTES = NCOMP * 32 * WN * 4;         // 32 KB (16 KB, 4 KB)
   static constexpr int STATS_OFF = RING_BYTES + 256;
   static constexpr int COLS_OFF = STATS_OFF + NW * 2 * WM * 4;  // per-column epilogue constants: [wave][bias, gain, offset][64]
   static constexpr int COLS_STRIDE = 3 * 64;                    // floats per wave (a wave's bias load lands 64 of them)
@@ -138,7 +142,7 @@ __global__ void __launch_bounds__(Cfg::NT) gemm_dmam_kernel(const GemmArgs a, co
     xb0[k] = lds0 + Cfg::PART_BYTES + (wm * Cfg::WM + lr) * Cfg::ROWB + ((kc ^ LX) << 4);
   }
 
-  const bool wave_active = (m0 + wm * Cfg::WM < a.M) && (n0 + wn * Cfg::WN < a.N);
+  const bool wave_active = wave < Cfg::NCOMP && (m0 + wm * Cfg::WM < a.M) && (n0 + wn * Cfg::WN < a.N);
 
   for (int slab = 0; slab < nslab; ++slab) {
     // This wave's loads of the slab have landed; the NSTAGE - 2 slabs requested after it (and, the first time round, the
@@ -177,6 +181,7 @@ __global__ void __launch_bounds__(Cfg::NT) gemm_dmam_kernel(const GemmArgs a, co
 
   wait_vmcnt<0>();
   dmam_barrier();  // every wave is done with the ring, and the empty loads past the end of K have retired
+  if (wave >= Cfg::NCOMP) return;   // (a wave that only loads)
 
   gemm_epilogue<Cfg::WM, Cfg::WN, OUT_DT, 0, LEAN>(a, acc, reinterpret_cast<float*>(smem) + wave * (32 * Cfg::WN),
                                               m0 + wm * Cfg::WM, n0 + wn * Cfg::WN, lane, nullptr,

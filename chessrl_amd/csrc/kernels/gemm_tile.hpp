@@ -524,7 +524,7 @@ bool gemm_dmaf_has(int in_dt, int out_dt, bool res_norm);
 hipError_t launch_gemm_dmaf(const GemmArgs& a, int in_dt, int out_dt, hipStream_t st);
 // gemm_dmam.hip: the 128x128 tile fed by direct-to-LDS loads through a four-stage ring (K in whole 128-byte slabs, no normalised residual).
 bool gemm_dmam_has(int in_dt, int out_dt);
-hipError_t launch_gemm_dmam(const GemmArgs& a, int in_dt, int out_dt, hipStream_t st, bool small_tile);
+hipError_t launch_gemm_dmam(const GemmArgs& a, int in_dt, int out_dt, hipStream_t st, int tile_size);
 // gemm_shortk.hip: K = 256 e4m3 operands, bare scaled product: a workgroup keeps 256 rows of A in registers and walks N.
 bool gemm_shortk_can(const GemmArgs& a, int in_dt, int out_dt);
 hipError_t launch_gemm_shortk(const GemmArgs& a, int in_dt, int out_dt, hipStream_t st);

@@ -303,10 +303,10 @@ def test_gemm_split_output_last_tile_column_carries_the_columns_behind_it(cuda, 
 @pytest.mark.parametrize("dt", ["bf16", "fp8"])
 def test_gemm_mid_tile_direct_to_lds_equals_register_staged(cuda, M, N, K, dt):
     """The 128x128 tile fed by direct-to-LDS loads through a four-stage ring (tile 11, what the library picks for up to 256
-    such tiles when K is whole 128-byte slabs) and the 64x64 tile on an eight-stage ring (tile 15, for up to 256 of those)
-    against the register-staged kernel (tile 12): same sums, bit-equal outputs; with bias, activation, residual and a
+    such tiles when K is whole 128-byte slabs), the 64x64 tile on an eight-stage ring (tile 15, for up to 256 of those) and
+    the 32x32 tile on a sixteen-stage ring (tile 16, likewise) against the register-staged kernel (tile 12): same sums, bit-equal outputs; with bias, activation, residual and a
     scaled e4m3 output. 1 to 32 slabs (fewer slabs than ring stages included), ragged M and N, K that is not whole slabs
-    (where 11 hands over to 12 and 15 is refused)."""
+    (where 11 hands over to 12 and 15 and 16 are refused)."""
     torch.manual_seed(M + N + K)
     if dt == "fp8":
         A = (torch.randn(M, K, device=cuda) * 30).to(torch.float8_e4m3fn)
@@ -329,13 +329,14 @@ def test_gemm_mid_tile_direct_to_lds_equals_register_staged(cuda, M, N, K, dt):
         assert torch.equal(o11, o12), (M, N, K, dt, kw["out_dt"], (o11.float() - o12.float()).abs().max().item())
         assert torch.equal(a11, a12)
         if (K * A.element_size()) % 128 == 0:
-            a15 = torch.zeros(1, device=cuda)
-            o15 = run_gemm(A, W, kw["out_dt"], tile=15, ldc=ldc, amax=a15, **{k: v for k, v in kw.items() if k != "out_dt"})
-            assert torch.equal(o15, o12) and torch.equal(a15, a12), (M, N, K, dt, kw["out_dt"])
+            for small in (15, 16):
+                a15 = torch.zeros(1, device=cuda)
+                o15 = run_gemm(A, W, kw["out_dt"], tile=small, ldc=ldc, amax=a15, **{k: v for k, v in kw.items() if k != "out_dt"})
+                assert torch.equal(o15, o12) and torch.equal(a15, a12), (M, N, K, dt, kw["out_dt"], small)
     if (K * A.element_size()) % 128 != 0:
         Cout = torch.zeros(M, ldc, dtype=torch.bfloat16, device=cuda)
         rc = lib().crl_gemm(p(A), K, p(W), K, p(Cout), ldc, M, N, K, _lib.FP8 if dt == "fp8" else _lib.BF16, _lib.BF16, None, 0, 1.0, 1.0,
-                            None, 0, _lib.F32, 1.0, None, 15, stream())
+                            None, 0, _lib.F32, 1.0, None, 16, stream())
         assert rc != 0
     ref = (A.float() @ W.float().t()) * descale
     out = run_gemm(A, W, _lib.BF16, descale=descale, tile=11, ldc=ldc)
