@@ -632,8 +632,9 @@ static hipError_t launch_in_out(const GemmArgs& a, int tile, hipStream_t st) {
   // The 128x128 tile has the register-staged kernel (any K, fp32 outputs, normalised residuals; two workgroups per CU;
   // tile 12 names it) and, for K in whole slabs, the direct-to-LDS kernel with three slabs in flight
   // (gemm_dmam_kernel.hpp, tile 11; bit-equal; one workgroup per CU). The second is 15 to 20 % faster while every tile has a
-  // CU of its own (M=4096, N=1024, bf16: 20.1 -> 16.3 us at K=1024, 27.9 -> 23.0 at K=1536) and slower beyond (384 tiles: 25.9
-  // -> 29.8 us), so tile 2 picks it for at most as many tiles as there are CUs.
+  // CU of its own (M=4096, N=1024, bf16: 20.1 -> 16.3 us at K=1024, 27.9 -> 23.0 at K=1536) and level beyond (384 tiles: 26.6 -> 24.9 us
+  // from warm caches, 768 tiles: 48.1 -> 49.2 us; no difference inside a 64-position forward pass), so tile 2 picks it for
+  // at most as many tiles as there are CUs.
   if (tile == 15 || tile == 16) return slabs && !a.res_stats && gemm_dmam_has(IN_DT, OUT_DT) ? launch_gemm_dmam(a, IN_DT, OUT_DT, st, tile == 16 ? 32 : 64) : hipErrorInvalidValue;
   if (tile == 11 && !slabs) tile = 12;
   if (tile == 2 || tile == 11) {
