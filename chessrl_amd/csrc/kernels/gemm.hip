@@ -513,13 +513,14 @@ static int splitk_plan(const GemmArgs& a, int esz, bool forced, int* slabs_per_s
 }
 
 // The same idea for the forward pass, where a row's result must not depend on how many rows the call has: narrow
-// outputs with a long K (the value head's 8192 -> 128 layer, the bias generator's 2048 -> 256 layer, both on one row
-// per position) are always cut into the same slices, a function of N and K alone, whenever the 64x64 tile is the
-// choice (fewer than 256 tiles of 128x128, i.e. under 16384 rows at these widths; the workspace holds that case).
-// At 64 rows the 8192 -> 128 layer otherwise runs on two workgroups for 98 us.
+// outputs with a very long K (the value head's 8192 -> 128 layer on one row per position: 128 slabs) are always cut
+// into the same slices, a function of N and K alone, whenever the 64x64 tile is the choice (fewer than 256 tiles of
+// 128x128, i.e. under 16384 rows at these widths; the workspace holds that case). At 64 rows that layer otherwise runs
+// on two workgroups for 98 us. From 64 slabs on: at 32 (the bias generator's 2048 -> 256 layer) the ring kernels walk
+// K in 10.3 us where the two passes of the sliced form take 11.3 (13.1 against 22.6 us at 4096 rows).
 static int splitk_plan_fixed(const GemmArgs& a, int esz, int* slabs_per_slice) {
   const int nslab = (int)(((long)a.K * esz + 127) >> 7);
-  if (a.N > 256 || nslab < 32) return 1;
+  if (a.N > 256 || nslab < 64) return 1;
   int ks = std::min(nslab / 16, 4);
   const int per = (nslab + ks - 1) / ks;
   ks = (nslab + per - 1) / per;

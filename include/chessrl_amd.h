@@ -108,7 +108,7 @@ int crl_random_positions(uint64_t seed, int n, int max_plies, double late_fracti
  * fp32 sums in a workspace of 64 MB that the library keeps per stream, and a second kernel that adds them in slice
  * order and applies the epilogue; 5 = 64x64 tiles whose K slabs four groups of four waves take in turn and add up in
  * LDS. Both are deterministic from launch to launch but differ from 1-3 in summation order. With tile 0, outputs of at
- * most 256 columns whose K is 4 KB or more per row are always K-sliced the same way (a function of N and K alone), so
+ * most 256 columns whose K is 8 KB or more per row are always K-sliced the same way (a function of N and K alone), so
  * the row-count independence holds for them too. The first K-sliced launch on a stream allocates that stream's
  * workspace: issue it once outside any graph capture. 7, 9 and 10 name the 256x256 kernels explicitly: 7 = eight waves in
  * step (any K, any operand type), 10 = the same with its address arithmetic kept out of the main loop (K in whole
