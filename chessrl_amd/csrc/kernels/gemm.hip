@@ -592,10 +592,12 @@ static hipError_t launch_in_out(const GemmArgs& a, int tile, hipStream_t st) {
     tile = big >= 160 ? 3 : mid >= 256 ? 2 : 1;
     // Few 64x64 tiles: nothing else on the CU hides the latency of walking K slab by slab, so four groups of waves
     // share the walk (measured with weights coming from HBM, M=128, K=768: 9.8 -> 8.2 us at N=2304, 12.3 -> 9.0 us at
-    // N=3072).
+    // N=3072) where the ring kernels below, which hide it with slabs in flight, do not apply (M=128, K=768 from warm
+    // caches: 7.1 us on four groups, 6.4 us on the ring; a 128-sequence rollout +4 %).
     const long small = (long)((a.M + 63) / 64) * ((a.N + 63) / 64);
     const long nslab = ((long)a.K * (IN_DT == DT_FP8 ? 1 : 2) + 127) >> 7;
-    if (tile == 1 && a.k_parallel && small <= 512 && nslab >= 8) tile = 5;
+    const bool ring_ok = !a.res_stats && ((long)a.K * (IN_DT == DT_FP8 ? 1 : 2)) % 128 == 0 && gemm_dmam_has(IN_DT, OUT_DT);
+    if (tile == 1 && a.k_parallel && small <= 512 && nslab >= 8 && !(ring_ok && small <= device_cus())) tile = 5;
     // (a residual that is normalised on the fly needs the tiled kernels' epilogue: no K slices for it)
     if (tile == 1 && !a.k_parallel && !a.res_stats) {
       int per = 0;
@@ -607,7 +609,7 @@ static hipError_t launch_in_out(const GemmArgs& a, int tile, hipStream_t st) {
     // those has (tile 15; M=64, N=1024, K=1024 bf16 with weights from HBM: 13.6 us register-staged, 8.4 us on 15; from
     // warm caches 9.1, 7.6 and, on 16, 6.9 us), on 128x128 tiles beyond (tile 11; M=1024, N=3104: 20.7 -> 14.9 us;
     // M=2048, N=1536: 18.0 -> 14.1 us; M=512, N=3104: 13.9 -> 12.5 us; level at M=1024, N=1536 and M=2048, N=1024).
-    if (tile == 1 && !a.k_parallel && !a.res_stats && ((long)a.K * (IN_DT == DT_FP8 ? 1 : 2)) % 128 == 0 && gemm_dmam_has(IN_DT, OUT_DT))
+    if (tile == 1 && ring_ok)
       tile = (long)((a.M + 31) / 32) * ((a.N + 31) / 32) <= device_cus() ? 16 : small <= device_cus() ? 15 : 11;
   }
   if (tile == 6 || tile == 8) return hipErrorInvalidValue;   // codes of two retired kernels
