@@ -173,11 +173,13 @@ def test_bt4class_batch_invariance(cuda, fp8):
     if fp8:
         m.calibrate(x[:128])
     pol, wdl = m(x)
-    # 1, 3, 64, 129, 161, 257 and 320 positions: the 64x64, 128x128 and 256x256 tiles of the trunk products, each with
-    # and without a ragged last tile (the e4m3 path re-normalises its residual in all three); 640: whole blocks of 256
-    # (position, head) rows and a bias tensor beyond 64 MB, where the e4m3 bias generator writes, and the attention
-    # kernel reads, the blocked layout (the 700 of the full call do not divide into blocks and stay row-major)
-    for sl in (slice(5, 6), slice(0, 3), slice(0, 64), slice(7, 136), slice(0, 161), slice(100, 357), slice(10, 330), slice(20, 660)):
+    # 1, 3, 8, 16, 32, 64, 129, 161, 257 and 320 positions: the 32x32, 64x64 and 128x128 tiles of the ring kernels, the
+    # register-staged 128x128 and the 256x256 tiles of the trunk products, each with and without a ragged last tile (the
+    # e4m3 path re-normalises its residual in the last three); 640: whole blocks of 256 (position, head) rows and a bias
+    # tensor beyond 64 MB, where the e4m3 bias generator writes, and the attention kernel reads, the blocked layout (the
+    # 700 of the full call do not divide into blocks and stay row-major)
+    for sl in (slice(5, 6), slice(0, 3), slice(40, 48), slice(0, 16), slice(3, 35), slice(0, 64), slice(7, 136), slice(0, 161), slice(100, 357),
+               slice(10, 330), slice(20, 660)):
         p2, w2 = m(x[sl].contiguous())
         assert torch.equal(p2, pol[sl]) and torch.equal(w2, wdl[sl])
     perm = torch.randperm(700, generator=torch.Generator().manual_seed(1))
