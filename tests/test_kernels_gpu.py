@@ -300,7 +300,7 @@ def test_gemm_split_output_last_tile_column_carries_the_columns_behind_it(cuda, 
 @pytest.mark.parametrize("M,N,K", [(128, 128, 64), (128, 128, 256), (4096, 1024, 1024), (4096, 1536, 1024), (4096, 1024, 1536), (2048, 4096, 256),
                                    (300, 700, 512), (1000, 3104, 1024), (4096, 200, 192), (130, 129, 128), (640, 3104, 1088),
                                    (64, 1024, 1024), (64, 3104, 1536), (37, 3, 128), (1, 1929, 4096), (512, 1536, 640)])
-@pytest.mark.parametrize("dt", ["bf16", "fp8"])
+@pytest.mark.parametrize("dt", ["bf16", "fp8", "f16"])
 def test_gemm_mid_tile_direct_to_lds_equals_register_staged(cuda, M, N, K, dt):
     """The 128x128 tile fed by direct-to-LDS loads through a four-stage ring (tile 11, what the library picks for up to 256
     such tiles when K is whole 128-byte slabs), the 64x64 tile on an eight-stage ring (tile 15, for up to 256 of those) and
@@ -313,13 +313,15 @@ def test_gemm_mid_tile_direct_to_lds_equals_register_staged(cuda, M, N, K, dt):
         W = (torch.randn(N, K, device=cuda) * 30).to(torch.float8_e4m3fn)
         descale = 1e-3
     else:
-        A = torch.randn(M, K, device=cuda).bfloat16()
-        W = (torch.randn(N, K, device=cuda) / K ** 0.5).bfloat16()
+        t16 = torch.float16 if dt == "f16" else torch.bfloat16
+        A = torch.randn(M, K, device=cuda).to(t16)
+        W = (torch.randn(N, K, device=cuda) / K ** 0.5).to(t16)
         descale = 1.0
+    o16 = _lib.F16 if dt == "f16" else _lib.BF16   # (16-bit operands keep their type on the way out)
     bias = torch.randn(N, device=cuda)
     ldc = (N + 7) // 8 * 8
     res = torch.randn(M, ldc, device=cuda).bfloat16()
-    cases = [dict(out_dt=_lib.BF16, bias=bias, act=2, descale=descale, alpha=0.43, res=res), dict(out_dt=_lib.BF16, descale=descale)]
+    cases = [dict(out_dt=o16, bias=bias, act=2, descale=descale, alpha=0.43, res=res), dict(out_dt=o16, descale=descale)]
     if dt == "fp8":
         cases.append(dict(out_dt=_lib.FP8, bias=bias, act=2, descale=descale, out_scale=7.0))
     for kw in cases:
@@ -334,12 +336,12 @@ def test_gemm_mid_tile_direct_to_lds_equals_register_staged(cuda, M, N, K, dt):
                 o15 = run_gemm(A, W, kw["out_dt"], tile=small, ldc=ldc, amax=a15, **{k: v for k, v in kw.items() if k != "out_dt"})
                 assert torch.equal(o15, o12) and torch.equal(a15, a12), (M, N, K, dt, kw["out_dt"], small)
     if (K * A.element_size()) % 128 != 0:
-        Cout = torch.zeros(M, ldc, dtype=torch.bfloat16, device=cuda)
-        rc = lib().crl_gemm(p(A), K, p(W), K, p(Cout), ldc, M, N, K, _lib.FP8 if dt == "fp8" else _lib.BF16, _lib.BF16, None, 0, 1.0, 1.0,
+        Cout = torch.zeros(M, ldc, dtype=TORCH_DT[o16], device=cuda)
+        rc = lib().crl_gemm(p(A), K, p(W), K, p(Cout), ldc, M, N, K, {"fp8": _lib.FP8, "f16": _lib.F16, "bf16": _lib.BF16}[dt], o16, None, 0, 1.0, 1.0,
                             None, 0, _lib.F32, 1.0, None, 16, stream())
         assert rc != 0
     ref = (A.float() @ W.float().t()) * descale
-    out = run_gemm(A, W, _lib.BF16, descale=descale, tile=11, ldc=ldc)
+    out = run_gemm(A, W, o16, descale=descale, tile=11, ldc=ldc)
     assert torch.allclose(out.float(), ref, rtol=2 ** -7, atol=2 ** -7 * ref.abs().max().item()), (out.float() - ref).abs().max()
 
 
