@@ -8,6 +8,7 @@ namespace crl {
 bool gemm_dmaf_has(int in_dt, int out_dt, bool res_norm) {
   if (res_norm) return in_dt == DT_FP8 && out_dt == DT_BF16;
   if (in_dt == DT_FP8) return out_dt == DT_BF16 || out_dt == DT_F16 || out_dt == DT_FP8;
+  if (in_dt == DT_BF16 && out_dt == DT_F32) return true;   // (an fp32 residual stream, fp32 logits)
   return in_dt == out_dt && (in_dt == DT_BF16 || in_dt == DT_F16);
 }
 
@@ -34,6 +35,7 @@ hipError_t launch_gemm_dmaf(const GemmArgs& a, int in_dt, int out_dt, hipStream_
   }
   if (in_dt == DT_BF16 && out_dt == DT_BF16) return lean == 2 ? launch_dmaf<DT_BF16, DT_BF16, 0, 2>(a, st) : lean == 1 ? launch_dmaf<DT_BF16, DT_BF16, 0, 1>(a, st) : launch_dmaf<DT_BF16, DT_BF16, 0>(a, st);
   if (in_dt == DT_F16 && out_dt == DT_F16) return launch_dmaf<DT_F16, DT_F16, 0>(a, st);
+  if (in_dt == DT_BF16 && out_dt == DT_F32) return launch_dmaf<DT_BF16, DT_F32, 0>(a, st);
   return hipErrorInvalidValue;
 }
 
