@@ -7,6 +7,7 @@ namespace crl {
 // false: no instance for this combination (the caller keeps the register-staged kernel).
 bool gemm_dmam_has(int in_dt, int out_dt) {
   if (in_dt == DT_FP8) return out_dt == DT_BF16 || out_dt == DT_F16 || out_dt == DT_FP8;
+  if (in_dt == DT_BF16 && out_dt == DT_F32) return true;   // (an fp32 residual stream, fp32 logits)
   return in_dt == out_dt && (in_dt == DT_BF16 || in_dt == DT_F16);
 }
 
@@ -21,6 +22,7 @@ static hipError_t launch_small(const GemmArgs& a, int in_dt, int out_dt, hipStre
   }
   if (in_dt == DT_BF16 && out_dt == DT_BF16) return launch_dmam<DT_BF16, DT_BF16, 0, S>(a, st);
   if (in_dt == DT_F16 && out_dt == DT_F16) return launch_dmam<DT_F16, DT_F16, 0, S>(a, st);
+  if (in_dt == DT_BF16 && out_dt == DT_F32) return launch_dmam<DT_BF16, DT_F32, 0, S>(a, st);
   return hipErrorInvalidValue;
 }
 
@@ -43,6 +45,7 @@ hipError_t launch_gemm_dmam(const GemmArgs& a, int in_dt, int out_dt, hipStream_
   }
   if (in_dt == DT_BF16 && out_dt == DT_BF16) return launch_dmam<DT_BF16, DT_BF16>(a, st);
   if (in_dt == DT_F16 && out_dt == DT_F16) return launch_dmam<DT_F16, DT_F16>(a, st);
+  if (in_dt == DT_BF16 && out_dt == DT_F32) return launch_dmam<DT_BF16, DT_F32>(a, st);
   return hipErrorInvalidValue;
 }
 

@@ -119,7 +119,8 @@ int crl_random_positions(uint64_t seed, int n, int max_plies, double late_fracti
  * 128x128 kernels (same sums and bits as 2): 11 = fed by direct-to-LDS loads through a four-stage ring (whole slabs; what 2
  * runs for at most one tile per CU), 12 = register-staged (any K; 11 hands over to it where K is not whole slabs).
  * 15 and 16 = the 64x64 tile on an eight-stage and the 32x32 tile on a sixteen-stage ring of direct-to-LDS loads (same sums
- * and bits as 1; whole slabs, bf16/f16/e4m3 operands with a 16-bit or e4m3 output, else CRL_ERR_ARG). Below 256 tiles of
+ * and bits as 1; whole slabs; e4m3 operands with a 16-bit or e4m3 output, bf16/f16 operands with an output of their own
+ * type, bf16 operands with an fp32 output; else CRL_ERR_ARG). Below 256 tiles of
  * 128x128, tile 0 runs 16 while every 32x32 tile has a CU of its own, 15 while every 64x64 tile has, 11 beyond, and 1 where
  * they do not apply.
  * 13 and 14 name the kernel for K = 256 e4m3 elements whose workgroups keep 256 rows of A in registers and walk N (the
